@@ -1,0 +1,148 @@
+/*
+ * libblr - structured-linear forward kernels for AMD MI355X (gfx950).
+ *
+ * C ABI of the shared library.  Every entry point
+ *   - takes plain device pointers and sizes (no framework types),
+ *   - only enqueues work on the HIP stream it is given (NULL = the null stream); it never
+ *     synchronises, never allocates and never frees device memory,
+ *   - borrows every buffer for the duration of the enqueued work,
+ *   - returns 0 on success or a negative blr_status; the text of the last failure on the
+ *     calling thread is available from blr_last_error().
+ *
+ * Row-major everywhere.  "M" is the number of token rows (batch * sequence).  x may be a
+ * strided view: row m starts at x + m * ldx elements.  Weights must be contiguous.
+ * dtype selects the element type of x, of the floating-point weights and of out.
+ *
+ * Each entry point names the function of the reference implementation
+ * (pabillam/mem-efficient-blr) whose arithmetic and operand layout it reproduces.
+ */
+#ifndef BLR_H
+#define BLR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  BLR_OK = 0,
+  BLR_ERR_BAD_ARG = -1,       /* null pointer, non-positive size, unknown enum value        */
+  BLR_ERR_BAD_SHAPE = -2,     /* in_f % b, out_f % b, rank % b ... violated                  */
+  BLR_ERR_WORKSPACE = -3,     /* workspace missing or smaller than blr_*_workspace_bytes()  */
+  BLR_ERR_UNSUPPORTED = -4,   /* combination not implemented (e.g. decode algo with fp32)   */
+  BLR_ERR_LAUNCH = -5,        /* the HIP runtime refused a launch                            */
+  BLR_ERR_NO_DEVICE = -6
+} blr_status;
+
+typedef enum { BLR_F16 = 0, BLR_BF16 = 1, BLR_F32 = 2 } blr_dtype;
+
+/* BLAST U factor: (b, r, q) for the partial/full function names, (b, q, r) for the bmm names
+ * (reference models/wrappers.py:151-159).                                                    */
+typedef enum { BLR_U_RQ = 0, BLR_U_QR = 1 } blr_u_layout;
+
+/* BLAST S factor: (b1=j, b2=i, r) for partial/full names, (r, b2=i, b1=j) for bmm names,
+ * (b2=i, b1=j, r) for the torch baseline layout (reference layer.py:193-200).               */
+typedef enum { BLR_S_JIR = 0, BLR_S_RIJ = 1, BLR_S_IJR = 2 } blr_s_layout;
+
+/* Which kernel family serves a call.  AUTO picks STREAM for M <= 16 (HBM-bound) and TILED above. */
+typedef enum {
+  BLR_ALGO_AUTO = 0,
+  BLR_ALGO_STREAM = 1,        /* persistent streaming kernel, one launch, M <= 16, f16/bf16 */
+  BLR_ALGO_TILED = 2,         /* MFMA tiled GEMMs with the rank-space intermediate in HBM   */
+  BLR_ALGO_FUSED = 3,         /* MFMA two-stage kernel, rank-space intermediate kept in LDS */
+  BLR_ALGO_STREAM_SPLIT = 4   /* the STREAM phases as separate launches (no grid barrier)   */
+} blr_algo;
+
+/* Monarch second factor: (l, s, r) for the right / right_ideal names, (l, r, s) for right_left
+ * (reference models/wrappers.py:26-31).                                                      */
+typedef enum { BLR_W2_SR = 0, BLR_W2_RS = 1 } blr_w2_layout;
+
+/* Monarch output order: out[n, s*l + ll] (reference monarch_funcs.py:44) or the blocked
+ * out[n, ll*S + s] of the right_ideal names (reference triton_funcs/monarch_kernels.py:1004). */
+typedef enum { BLR_OUT_INTERLEAVED = 0, BLR_OUT_BLOCKED = 1 } blr_monarch_out;
+
+const char* blr_last_error(void);
+int blr_version(void);
+/* Number of compute units of the current device (0 if no device). */
+int blr_device_cus(void);
+
+/* ---- BLAST --------------------------------------------------------------------------------
+ * out[m, i*q + qq] = sum_r U_i[qq, r] * (sum_j S[i, j, r] * (sum_p x[m, j*p + pp] * V_j[pp, r]))
+ * Replaces triton_blast_{partial,partial_grouped,partial_grouped_persistent,full}_{fp16,fp32}
+ * (reference triton_funcs/blast_kernels.py:2614-2995; U (b,r,q), S (j,i,r)) and
+ * triton_blast_bmm_{fp16,fp32} (:2998-3065; U (b,q,r), S (r,i,j)).  V is always (b, p, r).
+ * y_out / z_out: optional (may be NULL) (b, M, r) buffers of dtype receiving the two
+ * intermediates the *_fp32 names return.  They force the TILED algorithm.                    */
+size_t blr_blast_workspace_bytes(int M, int in_f, int out_f, int b, int r, int dtype, int algo);
+int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                  void* out, int64_t ldo, void* z_out, void* y_out,
+                  int M, int in_f, int out_f, int b, int r,
+                  int dtype, int u_layout, int s_layout, int algo,
+                  void* ws, size_t ws_bytes, void* stream);
+
+/* ---- weight-quantized BLAST ---------------------------------------------------------------
+ * Same product with U and V stored as symmetric int8 (bits = 8) or packed int4 (bits = 4) codes
+ * and fp16 per-output-channel scales: U codes (b, q, r[/2]) + u_scales (b, q); V codes
+ * (b, p, r[/2]) + v_scales (b, r); S (r, i, j) of dtype.  Served behind the name
+ * triton_blast_bmm_int8_fp16 (reference triton_funcs/blast_sym_quant_kernels.py:558-580).
+ * M <= 16, r % 32 == 0.                                                                      */
+size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits);
+int blr_blast_q_fwd(const void* x, int64_t ldx,
+                    const void* u_codes, const void* u_scales,
+                    const void* v_codes, const void* v_scales, const void* S,
+                    void* out, int64_t ldo,
+                    int M, int in_f, int out_f, int b, int r,
+                    int dtype, int bits, int algo,
+                    void* ws, size_t ws_bytes, void* stream);
+
+/* Symmetric per-channel quantizer producing the codes/scales consumed above.  w is viewed as
+ * (outer, reduce, inner) contiguous; the max-abs runs over `reduce`.  scales: fp16 (outer, inner).
+ * codes: int8 (outer, reduce, inner), or for bits = 4 two codes per byte along the flattened
+ * last axis (low nibble = even index).  No reference counterpart (the reference has no weight
+ * quantizer).                                                                                */
+int blr_quantize_sym(const void* w, int dtype, int64_t outer, int64_t reduce, int64_t inner,
+                     int bits, void* codes, void* scales, void* stream);
+
+/* ---- Monarch ------------------------------------------------------------------------------
+ * w1 (b, in_f/b, rank) with pre-permuted columns (reference layer.py:221-224), w2 per
+ * w2_layout.  Replaces triton_monarch_{right,right_ideal,right_left}_{fp16,fp32}
+ * (reference triton_funcs/monarch_kernels.py:823-1099).  out1 (optional, may be NULL) receives
+ * the permuted intermediate (b, M, rank) that the *_fp32 names return.                        */
+size_t blr_monarch_workspace_bytes(int M, int in_f, int out_f, int b, int rank, int dtype, int algo);
+int blr_monarch_fwd(const void* x, int64_t ldx, const void* w1, const void* w2,
+                    void* out, int64_t ldo, void* out1,
+                    int M, int in_f, int out_f, int b, int rank,
+                    int dtype, int w2_layout, int out_order, int algo,
+                    void* ws, size_t ws_bytes, void* stream);
+
+/* ---- low rank -----------------------------------------------------------------------------
+ * out = (x A) B with A (in_f, r), B (r, out_f).  Replaces triton_low_rank_{fp16,fp32}
+ * (reference triton_funcs/low_rank_kernels.py:394-417).  z_out optional (M, r).              */
+size_t blr_low_rank_workspace_bytes(int M, int in_f, int out_f, int r, int dtype, int algo);
+int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
+                     void* out, int64_t ldo, void* z_out,
+                     int M, int in_f, int out_f, int r, int dtype, int algo,
+                     void* ws, size_t ws_bytes, void* stream);
+
+/* ---- dense --------------------------------------------------------------------------------
+ * out = x W with W (in_f, out_f).  Replaces triton_dense_{fp16,fp32}
+ * (reference triton_funcs/dense_kernels.py:360-381).                                         */
+size_t blr_dense_workspace_bytes(int M, int in_f, int out_f, int dtype, int algo);
+int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
+                  int M, int in_f, int out_f, int dtype, int algo,
+                  void* ws, size_t ws_bytes, void* stream);
+
+/* ---- bandwidth probe ----------------------------------------------------------------------
+ * Streams `bytes` bytes from src with the load pattern of the streaming kernels and writes one
+ * checksum word per workgroup to dst (dst needs 4 * blr_probe_dst_words() bytes).  Role of the
+ * reference's *_load_store_* kernels (reference triton_funcs/dense_kernels.py:383-412,
+ * low_rank_kernels.py:419-450): an empirical bandwidth ceiling for the decode kernels.        */
+int blr_probe_dst_words(void);
+int blr_stream_probe(const void* src, size_t bytes, void* dst, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BLR_H */

@@ -1,0 +1,392 @@
+// extern "C" entry points of libblr: argument validation, algorithm choice, workspace carving.
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+#include "blr_common.h"
+
+namespace blr {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int device_cus() {
+  static std::once_flag once;
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return 0; }
+  std::call_once(once, [] {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return; }
+    for (int d = 0; d < n && d < 64; ++d) {
+      int v = 0;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, d) == hipSuccess) cus[d] = v;
+    }
+  });
+  return cus[dev];
+}
+
+static int elt_size(int dtype) { return dtype == BLR_F32 ? 4 : 2; }
+static bool dtype_ok(int dtype) { return dtype == BLR_F16 || dtype == BLR_BF16 || dtype == BLR_F32; }
+
+// ---- quantizer --------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float ld_f32(const T* p, int64_t i) { return TypeTraits<T>::to_f32(p[i]); }
+
+__device__ __forceinline__ int quant_code(float w, float s, float qmax) {
+  float q = rintf(__fdiv_rn(w, s));
+  q = fminf(fmaxf(q, -qmax), qmax);
+  return (int)q;
+}
+__device__ __forceinline__ float make_scale(float amax, float qmax, f16* store) {
+  f16 s16 = (f16)__fdiv_rn(amax, qmax);
+  if ((float)s16 == 0.0f) s16 = (f16)1.0f;
+  *store = s16;
+  return (float)s16;
+}
+
+// inner == 1: one workgroup per channel row, max over the contiguous axis.
+template <typename T>
+__global__ __launch_bounds__(256) void quant_rows_kernel(const T* __restrict__ w, int64_t reduce, int bits,
+                                                         uint8_t* __restrict__ codes, f16* __restrict__ scales) {
+  __shared__ float s_max[4];
+  __shared__ float s_scale;
+  const int64_t row = blockIdx.x;
+  const T* wr = w + row * reduce;
+  float amax = 0.0f;
+  for (int64_t k = threadIdx.x; k < reduce; k += 256) amax = fmaxf(amax, fabsf(ld_f32(wr, k)));
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+  if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  const float qmax = bits == 8 ? 127.0f : 7.0f;
+  if (threadIdx.x == 0) {
+    float m = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    s_scale = make_scale(m, qmax, &scales[row]);
+  }
+  __syncthreads();
+  const float s = s_scale;
+  if (bits == 8) {
+    int8_t* c = reinterpret_cast<int8_t*>(codes) + row * reduce;
+    for (int64_t k = threadIdx.x; k < reduce; k += 256) c[k] = (int8_t)quant_code(ld_f32(wr, k), s, qmax);
+  } else {
+    uint8_t* c = codes + row * (reduce / 2);
+    for (int64_t k = threadIdx.x; k < reduce / 2; k += 256) {
+      int lo = quant_code(ld_f32(wr, 2 * k), s, qmax), hi = quant_code(ld_f32(wr, 2 * k + 1), s, qmax);
+      c[k] = (uint8_t)((lo & 0xF) | ((hi & 0xF) << 4));
+    }
+  }
+}
+
+// inner > 1: thread per inner column (or column pair for int4), max over the strided axis.
+template <typename T>
+__global__ __launch_bounds__(256) void quant_cols_kernel(const T* __restrict__ w, int64_t reduce, int64_t inner, int bits,
+                                                         uint8_t* __restrict__ codes, f16* __restrict__ scales) {
+  const int64_t o = blockIdx.y;
+  const int per = bits == 8 ? 1 : 2;
+  const int64_t c0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * per;
+  if (c0 >= inner) return;
+  const T* wo = w + o * reduce * inner;
+  const float qmax = bits == 8 ? 127.0f : 7.0f;
+  float amax[2] = {0.0f, 0.0f};
+  for (int64_t k = 0; k < reduce; ++k)
+    for (int u = 0; u < per; ++u) amax[u] = fmaxf(amax[u], fabsf(ld_f32(wo, k * inner + c0 + u)));
+  float s[2];
+  for (int u = 0; u < per; ++u) s[u] = make_scale(amax[u], qmax, &scales[o * inner + c0 + u]);
+  if (bits == 8) {
+    int8_t* c = reinterpret_cast<int8_t*>(codes) + o * reduce * inner;
+    for (int64_t k = 0; k < reduce; ++k) c[k * inner + c0] = (int8_t)quant_code(ld_f32(wo, k * inner + c0), s[0], qmax);
+  } else {
+    uint8_t* c = codes + o * reduce * (inner / 2);
+    for (int64_t k = 0; k < reduce; ++k) {
+      int lo = quant_code(ld_f32(wo, k * inner + c0), s[0], qmax), hi = quant_code(ld_f32(wo, k * inner + c0 + 1), s[1], qmax);
+      c[k * (inner / 2) + c0 / 2] = (uint8_t)((lo & 0xF) | ((hi & 0xF) << 4));
+    }
+  }
+}
+
+template <typename T>
+static int quantize_t(const void* w, int64_t outer, int64_t reduce, int64_t inner, int bits, void* codes, void* scales, hipStream_t st) {
+  if (inner == 1) {
+    hipLaunchKernelGGL(quant_rows_kernel<T>, dim3((unsigned)outer), dim3(256), 0, st, (const T*)w, reduce, bits, (uint8_t*)codes, (f16*)scales);
+  } else {
+    int per = bits == 8 ? 1 : 2;
+    dim3 grid((unsigned)cdiv(cdiv(inner, per), 256), (unsigned)outer);
+    hipLaunchKernelGGL(quant_cols_kernel<T>, grid, dim3(256), 0, st, (const T*)w, reduce, inner, bits, (uint8_t*)codes, (f16*)scales);
+  }
+  BLR_CHECK_LAUNCH("quantize");
+  return BLR_OK;
+}
+
+}  // namespace blr
+
+using namespace blr;
+
+extern "C" {
+
+const char* blr_last_error(void) { return g_err; }
+int blr_version(void) { return 100; }
+int blr_device_cus(void) { return device_cus(); }
+
+static int resolve_algo(int algo, int M, int dtype, bool want_intermediates) {
+  if (algo == BLR_ALGO_AUTO) {
+    if (dtype != BLR_F32 && M <= 16 && !want_intermediates) return BLR_ALGO_STREAM;
+    return BLR_ALGO_TILED;
+  }
+  return algo;
+}
+
+// ---- BLAST ------------------------------------------------------------------------------------
+size_t blr_blast_workspace_bytes(int M, int in_f, int out_f, int b, int r, int dtype, int algo) {
+  if (M <= 0 || b <= 0 || r <= 0) return 0;
+  int a = resolve_algo(algo, M, dtype, false);
+  size_t tiled = 2 * align_up((size_t)b * M * r * elt_size(dtype), 256);
+  if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
+    size_t s = stream_blast_workspace(M, in_f, out_f, b, r, 16);
+    return s > tiled ? s : tiled;
+  }
+  return tiled;
+}
+
+static int check_blast_shape(const char* who, int M, int in_f, int out_f, int b, int r) {
+  if (M <= 0 || in_f <= 0 || out_f <= 0 || b <= 0 || r <= 0) { set_error("%s: non-positive size", who); return BLR_ERR_BAD_ARG; }
+  if (b == 1) { set_error("%s: b must not be 1", who); return BLR_ERR_BAD_SHAPE; }   // reference blast_funcs.py:34
+  if (in_f % b || out_f % b) { set_error("%s: in_f=%d / out_f=%d not divisible by b=%d", who, in_f, out_f, b); return BLR_ERR_BAD_SHAPE; }
+  return BLR_OK;
+}
+
+int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                  void* out, int64_t ldo, void* z_out, void* y_out,
+                  int M, int in_f, int out_f, int b, int r,
+                  int dtype, int u_layout, int s_layout, int algo,
+                  void* ws, size_t ws_bytes, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!x || !U || !V || !S || !out) { set_error("blast: null pointer"); return BLR_ERR_BAD_ARG; }
+  if (!dtype_ok(dtype) || u_layout < 0 || u_layout > 1 || s_layout < 0 || s_layout > 2) { set_error("blast: bad enum"); return BLR_ERR_BAD_ARG; }
+  int rc = check_blast_shape("blast", M, in_f, out_f, b, r);
+  if (rc) return rc;
+  if (ldx < in_f || ldo < out_f) { set_error("blast: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  const int P = in_f / b, Q = out_f / b;
+  int a = resolve_algo(algo, M, dtype, z_out || y_out);
+  if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
+    if (dtype == BLR_F32 || M > 16 || z_out || y_out) { set_error("blast: streaming algorithm needs f16/bf16, M <= 16, no intermediates"); return BLR_ERR_UNSUPPORTED; }
+    StreamBlastArgs s = {};
+    s.x = x; s.ldx = ldx; s.U = U; s.V = V; s.S = S; s.out = out; s.ldo = ldo;
+    s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
+    s.dtype = dtype; s.u_layout = u_layout; s.s_layout = s_layout; s.wbits = 16;
+    s.ws = ws; s.ws_bytes = ws_bytes; s.split = (a == BLR_ALGO_STREAM_SPLIT);
+    return stream_blast_launch(s, st);
+  }
+  if (a != BLR_ALGO_TILED) { set_error("blast: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
+  const size_t es = elt_size(dtype);
+  const size_t ybytes = align_up((size_t)b * M * r * es, 256);
+  size_t need = (y_out ? 0 : ybytes) + (z_out ? 0 : ybytes);
+  if (need && (!ws || ws_bytes < need)) { set_error("blast: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
+  char* wp = reinterpret_cast<char*>(ws);
+  void* Y = y_out ? y_out : (void*)wp; if (!y_out) wp += ybytes;
+  void* Z = z_out ? z_out : (void*)wp;
+
+  GemmArgs g1 = {};
+  g1.A = x; g1.lda = ldx; g1.sA = P;
+  g1.B = V; g1.ldb = r; g1.sB = (int64_t)P * r; g1.b_kn = 1;
+  g1.C = Y; g1.ldc = r; g1.sC = (int64_t)M * r; g1.cn = 1;
+  g1.M = M; g1.N = r; g1.K = P; g1.batch = b;
+  rc = gemm_launch(g1, dtype, st);
+  if (rc) return rc;
+
+  int64_t si, sj, sr;
+  if (s_layout == BLR_S_JIR) { sj = (int64_t)b * r; si = r; sr = 1; }
+  else if (s_layout == BLR_S_RIJ) { sr = (int64_t)b * b; si = b; sj = 1; }
+  else { si = (int64_t)b * r; sj = r; sr = 1; }
+  rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st);
+  if (rc) return rc;
+
+  GemmArgs g2 = {};
+  g2.A = Z; g2.lda = r; g2.sA = (int64_t)M * r;
+  g2.B = U;
+  if (u_layout == BLR_U_RQ) { g2.b_kn = 1; g2.ldb = Q; g2.sB = (int64_t)r * Q; }
+  else { g2.b_kn = 0; g2.ldb = r; g2.sB = (int64_t)Q * r; }
+  g2.C = out; g2.ldc = ldo; g2.sC = Q; g2.cn = 1;
+  g2.M = M; g2.N = Q; g2.K = r; g2.batch = b;
+  return gemm_launch(g2, dtype, st);
+}
+
+// ---- quantized BLAST -----------------------------------------------------------------------------
+size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits) {
+  if (M <= 0 || b <= 0 || r <= 0) return 0;
+  return stream_blast_workspace(M, in_f, out_f, b, r, bits);
+}
+
+int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void* u_scales,
+                    const void* v_codes, const void* v_scales, const void* S,
+                    void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
+                    int dtype, int bits, int algo, void* ws, size_t ws_bytes, void* stream) {
+  if (!x || !u_codes || !u_scales || !v_codes || !v_scales || !S || !out) { set_error("blast_q: null pointer"); return BLR_ERR_BAD_ARG; }
+  if (bits != 8 && bits != 4) { set_error("blast_q: bits must be 8 or 4"); return BLR_ERR_BAD_ARG; }
+  if (dtype != BLR_F16 && dtype != BLR_BF16) { set_error("blast_q: dtype must be f16 or bf16"); return BLR_ERR_UNSUPPORTED; }
+  int rc = check_blast_shape("blast_q", M, in_f, out_f, b, r);
+  if (rc) return rc;
+  if (M > 16) { set_error("blast_q: M=%d > 16 not served by the streaming kernel", M); return BLR_ERR_UNSUPPORTED; }
+  if (r % 32) { set_error("blast_q: r=%d must be a multiple of 32", r); return BLR_ERR_BAD_SHAPE; }
+  if (ldx < in_f || ldo < out_f) { set_error("blast_q: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  if (!aligned(u_codes, 16) || !aligned(v_codes, 16)) { set_error("blast_q: code buffers must be 16-byte aligned"); return BLR_ERR_BAD_ARG; }
+  StreamBlastArgs s = {};
+  s.x = x; s.ldx = ldx; s.U = u_codes; s.V = v_codes; s.S = S; s.u_scales = u_scales; s.v_scales = v_scales;
+  s.out = out; s.ldo = ldo; s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
+  s.dtype = dtype; s.u_layout = BLR_U_QR; s.s_layout = BLR_S_RIJ; s.wbits = bits;
+  s.ws = ws; s.ws_bytes = ws_bytes; s.split = (algo == BLR_ALGO_STREAM_SPLIT);
+  return stream_blast_launch(s, (hipStream_t)stream);
+}
+
+int blr_quantize_sym(const void* w, int dtype, int64_t outer, int64_t reduce, int64_t inner,
+                     int bits, void* codes, void* scales, void* stream) {
+  if (!w || !codes || !scales) { set_error("quantize: null pointer"); return BLR_ERR_BAD_ARG; }
+  if (outer <= 0 || reduce <= 0 || inner <= 0 || (bits != 8 && bits != 4) || !dtype_ok(dtype)) { set_error("quantize: bad argument"); return BLR_ERR_BAD_ARG; }
+  if (bits == 4 && ((inner == 1 ? reduce : inner) % 2)) { set_error("quantize: int4 needs an even contiguous axis"); return BLR_ERR_BAD_SHAPE; }
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == BLR_F32) return quantize_t<float>(w, outer, reduce, inner, bits, codes, scales, st);
+  if (dtype == BLR_F16) return quantize_t<f16>(w, outer, reduce, inner, bits, codes, scales, st);
+  return quantize_t<bf16>(w, outer, reduce, inner, bits, codes, scales, st);
+}
+
+// ---- Monarch --------------------------------------------------------------------------------------
+size_t blr_monarch_workspace_bytes(int M, int in_f, int out_f, int b, int rank, int dtype, int algo) {
+  if (M <= 0 || b <= 0 || rank <= 0) return 0;
+  int a = resolve_algo(algo, M, dtype, false);
+  size_t tiled = align_up((size_t)b * M * rank * elt_size(dtype), 256);
+  if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
+    size_t s = stream_generic_workspace(2, M, in_f, out_f, b, rank);
+    return s > tiled ? s : tiled;
+  }
+  return tiled;
+}
+
+int blr_monarch_fwd(const void* x, int64_t ldx, const void* w1, const void* w2,
+                    void* out, int64_t ldo, void* out1,
+                    int M, int in_f, int out_f, int b, int rank,
+                    int dtype, int w2_layout, int out_order, int algo,
+                    void* ws, size_t ws_bytes, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!x || !w1 || !w2 || !out) { set_error("monarch: null pointer"); return BLR_ERR_BAD_ARG; }
+  if (!dtype_ok(dtype) || w2_layout < 0 || w2_layout > 1 || out_order < 0 || out_order > 1) { set_error("monarch: bad enum"); return BLR_ERR_BAD_ARG; }
+  if (M <= 0 || in_f <= 0 || out_f <= 0 || b <= 0 || rank <= 0) { set_error("monarch: non-positive size"); return BLR_ERR_BAD_ARG; }
+  if (in_f % b || out_f % b || rank % b) { set_error("monarch: in_f, out_f and rank must be divisible by b=%d", b); return BLR_ERR_BAD_SHAPE; }   // reference wrappers.py:13-14
+  if (ldx < in_f || ldo < out_f) { set_error("monarch: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  const int P = in_f / b, S = out_f / b, per = rank / b;
+  int a = resolve_algo(algo, M, dtype, out1 != nullptr);
+  if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
+    if (dtype == BLR_F32 || M > 16 || out1) { set_error("monarch: streaming algorithm needs f16/bf16, M <= 16, no intermediates"); return BLR_ERR_UNSUPPORTED; }
+    StreamGenericArgs s = {};
+    s.x = x; s.ldx = ldx; s.W1 = w1; s.W2 = w2; s.out = out; s.ldo = ldo;
+    s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = rank; s.dtype = dtype; s.op = 2;
+    s.w2_layout = w2_layout; s.out_order = out_order; s.ws = ws; s.ws_bytes = ws_bytes; s.split = (a == BLR_ALGO_STREAM_SPLIT);
+    return stream_generic_launch(s, st);
+  }
+  if (a != BLR_ALGO_TILED) { set_error("monarch: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
+  const size_t need = out1 ? 0 : align_up((size_t)b * M * rank * elt_size(dtype), 256);
+  if (need && (!ws || ws_bytes < need)) { set_error("monarch: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
+  void* O1 = out1 ? out1 : ws;
+
+  GemmArgs g1 = {};
+  g1.A = x; g1.lda = ldx; g1.sA = P;
+  g1.B = w1; g1.ldb = rank; g1.sB = (int64_t)P * rank; g1.b_kn = 1;
+  g1.C = O1; g1.ldc = rank; g1.sC = 0; g1.cn = 1;
+  g1.epi = EPI_MONARCH_SCATTER; g1.per = per; g1.sL = (int64_t)M * rank;
+  g1.M = M; g1.N = rank; g1.K = P; g1.batch = b;
+  int rc = gemm_launch(g1, dtype, st);
+  if (rc) return rc;
+
+  GemmArgs g2 = {};
+  g2.A = O1; g2.lda = rank; g2.sA = (int64_t)M * rank;
+  g2.B = w2;
+  if (w2_layout == BLR_W2_SR) { g2.b_kn = 0; g2.ldb = rank; g2.sB = (int64_t)S * rank; }
+  else { g2.b_kn = 1; g2.ldb = S; g2.sB = (int64_t)rank * S; }
+  g2.C = out; g2.ldc = ldo;
+  if (out_order == BLR_OUT_INTERLEAVED) { g2.sC = 1; g2.cn = b; }
+  else { g2.sC = S; g2.cn = 1; }
+  g2.M = M; g2.N = S; g2.K = rank; g2.batch = b;
+  return gemm_launch(g2, dtype, st);
+}
+
+// ---- low rank -------------------------------------------------------------------------------------
+size_t blr_low_rank_workspace_bytes(int M, int in_f, int out_f, int r, int dtype, int algo) {
+  if (M <= 0 || r <= 0) return 0;
+  int a = resolve_algo(algo, M, dtype, false);
+  size_t tiled = align_up((size_t)M * r * elt_size(dtype), 256);
+  if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
+    size_t s = stream_generic_workspace(1, M, in_f, out_f, 1, r);
+    return s > tiled ? s : tiled;
+  }
+  return tiled;
+}
+
+int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
+                     void* out, int64_t ldo, void* z_out,
+                     int M, int in_f, int out_f, int r, int dtype, int algo,
+                     void* ws, size_t ws_bytes, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!x || !A || !B || !out) { set_error("low_rank: null pointer"); return BLR_ERR_BAD_ARG; }
+  if (!dtype_ok(dtype)) { set_error("low_rank: bad dtype"); return BLR_ERR_BAD_ARG; }
+  if (M <= 0 || in_f <= 0 || out_f <= 0 || r <= 0) { set_error("low_rank: non-positive size"); return BLR_ERR_BAD_ARG; }
+  if (ldx < in_f || ldo < out_f) { set_error("low_rank: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  int a = resolve_algo(algo, M, dtype, z_out != nullptr);
+  if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
+    if (dtype == BLR_F32 || M > 16 || z_out) { set_error("low_rank: streaming algorithm needs f16/bf16, M <= 16, no intermediates"); return BLR_ERR_UNSUPPORTED; }
+    StreamGenericArgs s = {};
+    s.x = x; s.ldx = ldx; s.W1 = A; s.W2 = B; s.out = out; s.ldo = ldo;
+    s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = 1; s.r = r; s.dtype = dtype; s.op = 1;
+    s.ws = ws; s.ws_bytes = ws_bytes; s.split = (a == BLR_ALGO_STREAM_SPLIT);
+    return stream_generic_launch(s, st);
+  }
+  if (a != BLR_ALGO_TILED) { set_error("low_rank: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
+  const size_t need = z_out ? 0 : align_up((size_t)M * r * elt_size(dtype), 256);
+  if (need && (!ws || ws_bytes < need)) { set_error("low_rank: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
+  void* Z = z_out ? z_out : ws;
+  GemmArgs g1 = {};
+  g1.A = x; g1.lda = ldx; g1.B = A; g1.ldb = r; g1.b_kn = 1;
+  g1.C = Z; g1.ldc = r; g1.cn = 1; g1.M = M; g1.N = r; g1.K = in_f; g1.batch = 1;
+  int rc = gemm_launch(g1, dtype, st);
+  if (rc) return rc;
+  GemmArgs g2 = {};
+  g2.A = Z; g2.lda = r; g2.B = B; g2.ldb = out_f; g2.b_kn = 1;
+  g2.C = out; g2.ldc = ldo; g2.cn = 1; g2.M = M; g2.N = out_f; g2.K = r; g2.batch = 1;
+  return gemm_launch(g2, dtype, st);
+}
+
+// ---- dense ----------------------------------------------------------------------------------------
+size_t blr_dense_workspace_bytes(int M, int in_f, int out_f, int dtype, int algo) {
+  if (M <= 0) return 0;
+  int a = resolve_algo(algo, M, dtype, false);
+  if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) return stream_generic_workspace(0, M, in_f, out_f, 1, 0);
+  return 0;
+}
+
+int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
+                  int M, int in_f, int out_f, int dtype, int algo,
+                  void* ws, size_t ws_bytes, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!x || !W || !out) { set_error("dense: null pointer"); return BLR_ERR_BAD_ARG; }
+  if (!dtype_ok(dtype)) { set_error("dense: bad dtype"); return BLR_ERR_BAD_ARG; }
+  if (M <= 0 || in_f <= 0 || out_f <= 0) { set_error("dense: non-positive size"); return BLR_ERR_BAD_ARG; }
+  if (ldx < in_f || ldo < out_f) { set_error("dense: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  int a = resolve_algo(algo, M, dtype, false);
+  if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
+    if (dtype == BLR_F32 || M > 16) { set_error("dense: streaming algorithm needs f16/bf16 and M <= 16"); return BLR_ERR_UNSUPPORTED; }
+    StreamGenericArgs s = {};
+    s.x = x; s.ldx = ldx; s.W1 = W; s.out = out; s.ldo = ldo;
+    s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = 1; s.r = 0; s.dtype = dtype; s.op = 0;
+    s.ws = ws; s.ws_bytes = ws_bytes; s.split = (a == BLR_ALGO_STREAM_SPLIT);
+    return stream_generic_launch(s, st);
+  }
+  if (a != BLR_ALGO_TILED) { set_error("dense: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
+  GemmArgs g = {};
+  g.A = x; g.lda = ldx; g.B = W; g.ldb = out_f; g.b_kn = 1;
+  g.C = out; g.ldc = ldo; g.cn = 1; g.M = M; g.N = out_f; g.K = in_f; g.batch = 1;
+  return gemm_launch(g, dtype, st);
+}
+
+}  // extern "C"

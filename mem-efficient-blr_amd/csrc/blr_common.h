@@ -1,0 +1,132 @@
+// Shared device/host helpers for libblr (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/blr.h"
+
+namespace blr {
+
+typedef _Float16 f16;
+typedef __bf16 bf16;
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+template <typename T> struct TypeTraits;
+template <> struct TypeTraits<f16> {
+  using vec8 = f16x8;
+  using vec4 = f16x4;
+  static __device__ __forceinline__ float to_f32(f16 v) { return (float)v; }
+  static __device__ __forceinline__ f16 from_f32(float v) { return (f16)v; }
+  static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct TypeTraits<bf16> {
+  using vec8 = bf16x8;
+  using vec4 = bf16x4;
+  static __device__ __forceinline__ float to_f32(bf16 v) { return (float)v; }
+  static __device__ __forceinline__ bf16 from_f32(float v) { return (bf16)v; }
+  static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct TypeTraits<float> {
+  static __device__ __forceinline__ float to_f32(float v) { return v; }
+  static __device__ __forceinline__ float from_f32(float v) { return v; }
+};
+
+// 16-byte global load / store of 8 two-byte elements (pointer must be 16-byte aligned).
+template <typename V> __device__ __forceinline__ V ldg16(const void* p) {
+  return *reinterpret_cast<const V*>(p);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// ---- host side ------------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int device_cus();
+// true when p is aligned to `bytes`.
+static inline bool aligned(const void* p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) % bytes) == 0; }
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+#define BLR_CHECK_LAUNCH(what)                                              \
+  do {                                                                      \
+    hipError_t e__ = hipGetLastError();                                     \
+    if (e__ != hipSuccess) {                                                \
+      blr::set_error("%s: launch failed: %s", what, hipGetErrorString(e__)); \
+      return BLR_ERR_LAUNCH;                                                \
+    }                                                                       \
+  } while (0)
+
+// ---- tiled GEMM (blr_gemm.hip) ----------------------------------------------------------
+enum { EPI_PLAIN = 0, EPI_MONARCH_SCATTER = 1 };
+struct GemmArgs {
+  const void* A; int64_t lda; int64_t sA;   // A[bt*sA + m*lda + k]
+  const void* B; int64_t ldb; int64_t sB;   // b_kn: B[bt*sB + k*ldb + n]   else: B[bt*sB + n*ldb + k]
+  void* C; int64_t ldc; int64_t sC; int64_t cn;   // C[bt*sC + m*ldc + n*cn]
+  int M, N, K, batch;
+  int b_kn;
+  int epi;          // EPI_*
+  int per;          // EPI_MONARCH_SCATTER: column c of batch kk -> C[(c/per)*sL + m*ldc + kk*per + c%per]
+  int64_t sL;
+};
+// dtype: blr_dtype.  Returns blr_status.
+int gemm_launch(const GemmArgs& a, int dtype, hipStream_t st);
+
+// ---- BLAST rank-space mix, tiled path (blr_gemm.hip) ------------------------------------
+// Z[i, m, r] = sum_j S(i, j, r) * Y[j, m, r];  Y, Z (b, M, R) contiguous of dtype.
+int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
+                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st);
+
+// ---- streaming (decode) engine (blr_stream.hip) -------------------------------------------
+struct StreamBlastArgs {
+  const void* x; int64_t ldx;
+  const void* U; const void* V; const void* S;
+  const void* u_scales; const void* v_scales;   // quantized only (fp16)
+  void* out; int64_t ldo;
+  int M, in_f, out_f, b, r;
+  int dtype, u_layout, s_layout;
+  int wbits;                                    // 16 = floating weights, 8 / 4 = codes
+  void* ws; size_t ws_bytes;
+  int split;                                    // 1: separate launches per phase
+};
+size_t stream_blast_workspace(int M, int in_f, int out_f, int b, int r, int wbits);
+int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st);
+
+struct StreamGenericArgs {                      // dense / low-rank / monarch at M <= 16
+  const void* x; int64_t ldx;
+  const void* W1; const void* W2;               // dense: W1 only
+  void* out; int64_t ldo;
+  int M, in_f, out_f, b, r;                     // dense: r = 0; low rank: b = 1
+  int dtype;
+  int op;                                       // 0 dense, 1 low rank, 2 monarch
+  int w2_layout, out_order;                     // monarch
+  void* ws; size_t ws_bytes;
+  int split;
+};
+size_t stream_generic_workspace(int op, int M, int in_f, int out_f, int b, int r);
+int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st);
+
+}  // namespace blr

@@ -1,0 +1,366 @@
+// Tiled batched GEMM for the prefill-sized (M > 16) shapes and for the fp32 verification
+// variants, plus the BLAST rank-space mix used by the unfused (TILED) algorithm.
+//
+// f16 / bf16: 256-thread workgroups (4 waves as 2x2), v_mfma_f32_32x32x16 tiles, operands
+// staged through LDS as [row][64 + 8] two-byte elements (the 16-byte pad makes the 128-bit
+// fragment reads bank-conflict free).  Activations and (b,q,r)-style weights are K-contiguous
+// and copied straight in; (k, n)-ordered weights (n contiguous - the layout most of the
+// reference's kernel names use) are transposed in registers on their way into LDS.
+// fp32: plain FMA tiles, used only by the *_fp32 verification names.
+#include "blr_common.h"
+
+namespace blr {
+
+constexpr int BK = 64;          // k extent of an LDS tile
+constexpr int LDS_LD = BK + 8;  // row stride in elements
+
+template <typename T, int BM, int BN>
+struct GemmSmem {
+  T a[BM][LDS_LD];
+  T b[BN][LDS_LD];
+};
+
+// ---- global -> register staging ------------------------------------------------------------
+// K-contiguous operand: tile of ROWS rows x 64 k.  Thread t owns vectors v = t + i*256,
+// row = v / 8, k-vector = v % 8 (8 lanes cover one 128-byte row segment).
+template <typename T, int ROWS>
+struct KcStage {
+  static constexpr int NV = ROWS * 8 / 256;
+  typename TypeTraits<T>::vec8 v[NV];
+
+  __device__ __forceinline__ void load(const T* base, int64_t ld, int row0, int nrows, int k0, int K,
+                                       bool vec_ok, int tid) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      int vi = tid + i * 256;
+      int row = vi >> 3, kv = (vi & 7) * 8;
+      int gr = row0 + row, gk = k0 + kv;
+      typename TypeTraits<T>::vec8 val;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) val[e] = (T)0.0f;
+      if (gr < nrows && gk < K) {
+        const T* p = base + (int64_t)gr * ld + gk;
+        if (vec_ok && gk + 8 <= K) {
+          val = ldg16<typename TypeTraits<T>::vec8>(p);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (gk + e < K) val[e] = p[e];
+        }
+      }
+      v[i] = val;
+    }
+  }
+  __device__ __forceinline__ void store(T (*s)[LDS_LD], int tid) const {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      int vi = tid + i * 256;
+      int row = vi >> 3, kv = (vi & 7) * 8;
+      *reinterpret_cast<typename TypeTraits<T>::vec8*>(&s[row][kv]) = v[i];
+    }
+  }
+};
+
+// (k, n)-ordered operand: tile of 64 k x COLS n, n contiguous in memory.  Thread owns 4(k) x 8(n)
+// micro-blocks: kq = lane % 16 (k0 = 4*kq), nv = wave*4 + lane/16 (+16 per pass).  Written to LDS
+// transposed as [n][k] with 8-byte stores; with kq fastest across lanes those stores run at full
+// LDS rate.
+template <typename T, int COLS>
+struct KnStage {
+  static constexpr int NP = COLS / 128;
+  typename TypeTraits<T>::vec8 v[NP][4];
+
+  __device__ __forceinline__ void load(const T* base, int64_t ld, int col0, int ncols, int k0, int K,
+                                       bool vec_ok, int tid) {
+    int lane = tid & 63, wave = tid >> 6;
+    int kq = lane & 15;
+#pragma unroll
+    for (int ps = 0; ps < NP; ++ps) {
+      int nv = wave * 4 + (lane >> 4) + ps * 16;
+      int gn = col0 + nv * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int gk = k0 + kq * 4 + i;
+        typename TypeTraits<T>::vec8 val;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) val[e] = (T)0.0f;
+        if (gk < K && gn < ncols) {
+          const T* p = base + (int64_t)gk * ld + gn;
+          if (vec_ok && gn + 8 <= ncols) {
+            val = ldg16<typename TypeTraits<T>::vec8>(p);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (gn + e < ncols) val[e] = p[e];
+          }
+        }
+        v[ps][i] = val;
+      }
+    }
+  }
+  __device__ __forceinline__ void store(T (*s)[LDS_LD], int tid) const {
+    int lane = tid & 63, wave = tid >> 6;
+    int kq = lane & 15;
+#pragma unroll
+    for (int ps = 0; ps < NP; ++ps) {
+      int nv = wave * 4 + (lane >> 4) + ps * 16;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        typename TypeTraits<T>::vec4 w;
+        w[0] = v[ps][0][e]; w[1] = v[ps][1][e]; w[2] = v[ps][2][e]; w[3] = v[ps][3][e];
+        *reinterpret_cast<typename TypeTraits<T>::vec4*>(&s[nv * 8 + e][kq * 4]) = w;
+      }
+    }
+  }
+};
+
+__device__ __forceinline__ int64_t epi_offset(const GemmArgs& g, int bt, int m, int n) {
+  if (g.epi == EPI_MONARCH_SCATTER) {
+    int dst_blk = n / g.per, j = n - dst_blk * g.per;
+    return (int64_t)dst_blk * g.sL + (int64_t)m * g.ldc + (int64_t)bt * g.per + j;
+  }
+  return (int64_t)bt * g.sC + (int64_t)m * g.ldc + (int64_t)n * g.cn;
+}
+
+template <typename T, int BM, int BN, bool B_KN>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int a_vec, int b_vec) {
+  constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;    // 32x32 MFMA tiles per wave
+  using V8 = typename TypeTraits<T>::vec8;
+  __shared__ GemmSmem<T, BM, BN> sm;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // Tile order: consecutive workgroups walk down M for one N tile, so the weight tile they share
+  // stays hot in L2 / Infinity Cache while the activations stream past.
+  int tile = blockIdx.x;
+  int tm_i = tile % tiles_m, tn_i = tile / tiles_m;
+  const int bt = blockIdx.y;
+  const int m0 = tm_i * BM, n0 = tn_i * BN;
+
+  const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)bt * g.sA;
+  const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)bt * g.sB;
+  T* C = reinterpret_cast<T*>(g.C);
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  KcStage<T, BM> sa;
+  KcStage<T, BN> sb_kc;
+  KnStage<T, BN> sb_kn;
+
+  const int KT = (g.K + BK - 1) / BK;
+  sa.load(A, g.lda, m0, g.M, 0, g.K, a_vec, tid);
+  if (B_KN) sb_kn.load(B, g.ldb, n0, g.N, 0, g.K, b_vec, tid);
+  else sb_kc.load(B, g.ldb, n0, g.N, 0, g.K, b_vec, tid);
+
+  for (int kt = 0; kt < KT; ++kt) {
+    __syncthreads();                       // previous tile fully consumed
+    sa.store(sm.a, tid);
+    if (B_KN) sb_kn.store(sm.b, tid);
+    else sb_kc.store(sm.b, tid);
+    __syncthreads();
+    if (kt + 1 < KT) {                     // next tile's loads fly while this one is multiplied
+      int k0 = (kt + 1) * BK;
+      sa.load(A, g.lda, m0, g.M, k0, g.K, a_vec, tid);
+      if (B_KN) sb_kn.load(B, g.ldb, n0, g.N, k0, g.K, b_vec, tid);
+      else sb_kc.load(B, g.ldb, n0, g.N, k0, g.K, b_vec, tid);
+    }
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      const int kof = kk * 16 + (lane >> 5) * 8;
+      V8 af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = *reinterpret_cast<const V8*>(&sm.a[wm * WM + i * 32 + (lane & 31)][kof]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bf[j] = *reinterpret_cast<const V8*>(&sm.b[wn * WN + j * 32 + (lane & 31)][kof]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = TypeTraits<T>::mfma32(af[i], bf[j], acc[i][j]);
+    }
+  }
+
+  // D fragment: element e of lane l is row (e/4)*8 + (l/32)*4 + e%4, column l%32.
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int col = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        int row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row < g.M && col < g.N) C[epi_offset(g, bt, row, col)] = TypeTraits<T>::from_f32(acc[i][j][e]);
+      }
+    }
+}
+
+// ---- fp32 verification GEMM: 64x64 tile, 16x16 threads, 4x4 outputs per thread ---------------
+template <bool B_KN>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) {
+  __shared__ float as[16][64 + 1];
+  __shared__ float bs[16][64 + 1];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int bt = blockIdx.y;
+  const int m0 = (blockIdx.x % tiles_m) * 64, n0 = (blockIdx.x / tiles_m) * 64;
+  const float* A = reinterpret_cast<const float*>(g.A) + (int64_t)bt * g.sA;
+  const float* B = reinterpret_cast<const float*>(g.B) + (int64_t)bt * g.sB;
+  float* C = reinterpret_cast<float*>(g.C);
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < g.K; k0 += 16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int idx = tid + i * 256;               // 0..1023
+      {                                      // A tile: row = idx / 16, k = idx % 16
+        int r = idx >> 4, k = idx & 15;
+        int gr = m0 + r, gk = k0 + k;
+        as[k][r] = (gr < g.M && gk < g.K) ? A[(int64_t)gr * g.lda + gk] : 0.0f;
+      }
+      if (B_KN) {                            // k = idx / 64, n = idx % 64
+        int k = idx >> 6, n = idx & 63;
+        int gk = k0 + k, gn = n0 + n;
+        bs[k][n] = (gk < g.K && gn < g.N) ? B[(int64_t)gk * g.ldb + gn] : 0.0f;
+      } else {                               // n = idx / 16, k = idx % 16
+        int n = idx >> 4, k = idx & 15;
+        int gk = k0 + k, gn = n0 + n;
+        bs[k][n] = (gk < g.K && gn < g.N) ? B[(int64_t)gn * g.ldb + gk] : 0.0f;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { av[i] = as[k][ty * 4 + i]; bv[i] = bs[k][tx * 4 + i]; }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int row = m0 + ty * 4 + i, col = n0 + tx * 4 + j;
+      if (row < g.M && col < g.N) C[epi_offset(g, bt, row, col)] = acc[i][j];
+    }
+}
+
+template <typename T, int BM, int BN>
+static int launch_mfma(const GemmArgs& g, hipStream_t st) {
+  int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
+  // 16-byte vector loads need every row start and every k (or n) offset to be 16-byte aligned.
+  int a_vec = aligned(g.A, 16) && g.lda % 8 == 0 && g.sA % 8 == 0;
+  int b_vec = aligned(g.B, 16) && g.ldb % 8 == 0 && g.sB % 8 == 0;
+  dim3 grid(tiles_m * tiles_n, g.batch);
+  if (g.b_kn) hipLaunchKernelGGL((gemm_mfma_kernel<T, BM, BN, true>), grid, dim3(256), 0, st, g, tiles_m, tiles_n, a_vec, b_vec);
+  else hipLaunchKernelGGL((gemm_mfma_kernel<T, BM, BN, false>), grid, dim3(256), 0, st, g, tiles_m, tiles_n, a_vec, b_vec);
+  BLR_CHECK_LAUNCH("gemm_mfma");
+  return BLR_OK;
+}
+
+template <typename T>
+static int pick_mfma(const GemmArgs& g, hipStream_t st) {
+  // Large problems take the 256x128 tile (more MFMA work per LDS byte); when that would leave
+  // most of the 256 CUs idle, or N is narrow, fall back to 128x128.
+  int64_t big_tiles = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
+  if (g.M >= 256 && big_tiles >= 2 * device_cus()) return launch_mfma<T, 256, 128>(g, st);
+  return launch_mfma<T, 128, 128>(g, st);
+}
+
+int gemm_launch(const GemmArgs& g, int dtype, hipStream_t st) {
+  if (g.M <= 0 || g.N <= 0 || g.K <= 0 || g.batch <= 0) { set_error("gemm: empty problem"); return BLR_ERR_BAD_ARG; }
+  if (dtype == BLR_F16) return pick_mfma<f16>(g, st);
+  if (dtype == BLR_BF16) return pick_mfma<bf16>(g, st);
+  if (dtype == BLR_F32) {
+    int tiles_m = (int)cdiv(g.M, 64), tiles_n = (int)cdiv(g.N, 64);
+    dim3 grid(tiles_m * tiles_n, g.batch);
+    if (g.b_kn) hipLaunchKernelGGL((gemm_f32_kernel<true>), grid, dim3(256), 0, st, g, tiles_m);
+    else hipLaunchKernelGGL((gemm_f32_kernel<false>), grid, dim3(256), 0, st, g, tiles_m);
+    BLR_CHECK_LAUNCH("gemm_f32");
+    return BLR_OK;
+  }
+  set_error("gemm: unknown dtype %d", dtype);
+  return BLR_ERR_BAD_ARG;
+}
+
+// ---- BLAST rank-space mix ------------------------------------------------------------------
+// Workgroup = (64-wide r chunk) x (32 rows of m per pass); the S slab S(:, :, r chunk) is staged
+// in LDS as fp32 [j][i][64] once per workgroup and reused for every m pass.
+template <typename T, int MAXB>
+__global__ __launch_bounds__(256) void blast_mix_kernel(const T* __restrict__ Y, const T* __restrict__ S,
+                                                        T* __restrict__ Z, int M, int b, int R,
+                                                        int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg) {
+  extern __shared__ float s_lds[];           // [b][b][64]  (j, i, r)
+  const int tid = threadIdx.x;
+  const int r0 = blockIdx.x * 64;
+  const int rr = tid & 63, ms = tid >> 6;    // 64 r lanes x 4 m slots
+  for (int idx = tid; idx < b * b * 64; idx += 256) {
+    int r = idx & 63, ji = idx >> 6;
+    int j = ji / b, i = ji - j * b;
+    float v = 0.0f;
+    if (r0 + r < R) v = TypeTraits<T>::to_f32(S[(int64_t)i * s_si + (int64_t)j * s_sj + (int64_t)(r0 + r) * s_sr]);
+    s_lds[idx] = v;
+  }
+  __syncthreads();
+  const int r = r0 + rr;
+  if (r >= R) return;
+  const int m_begin = blockIdx.y * m_per_wg;
+  const int m_end = min(M, m_begin + m_per_wg);
+  for (int m = m_begin + ms; m < m_end; m += 4) {
+    if (MAXB > 0) {                          // b <= MAXB: every Y value is loaded once
+      float yv[MAXB > 0 ? MAXB : 1];
+#pragma unroll
+      for (int j = 0; j < MAXB; ++j) yv[j] = (j < b) ? TypeTraits<T>::to_f32(Y[((int64_t)j * M + m) * R + r]) : 0.0f;
+      for (int i = 0; i < b; ++i) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < MAXB; ++j)
+          if (j < b) acc = fmaf(s_lds[(j * b + i) * 64 + rr], yv[j], acc);
+        Z[((int64_t)i * M + m) * R + r] = TypeTraits<T>::from_f32(acc);
+      }
+    } else {
+      for (int i = 0; i < b; ++i) {
+        float acc = 0.0f;
+        for (int j = 0; j < b; ++j)
+          acc = fmaf(s_lds[(j * b + i) * 64 + rr], TypeTraits<T>::to_f32(Y[((int64_t)j * M + m) * R + r]), acc);
+        Z[((int64_t)i * M + m) * R + r] = TypeTraits<T>::from_f32(acc);
+      }
+    }
+  }
+}
+
+template <typename T>
+static void mix_dispatch(dim3 grid, size_t lds, hipStream_t st, const void* Y, const void* S, void* Z, int M, int b, int R,
+                         int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg) {
+  if (b <= 16)
+    hipLaunchKernelGGL((blast_mix_kernel<T, 16>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+  else
+    hipLaunchKernelGGL((blast_mix_kernel<T, 0>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+}
+
+int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
+                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st) {
+  size_t lds = (size_t)b * b * 64 * sizeof(float);
+  if (lds > 64 * 1024) { set_error("blast mix: b=%d too large for the LDS slab", b); return BLR_ERR_UNSUPPORTED; }
+  int r_chunks = (int)cdiv(R, 64);
+  int m_per_wg = 64;
+  while ((int64_t)r_chunks * cdiv(M, m_per_wg) < 1024 && m_per_wg > 4) m_per_wg /= 2;
+  dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
+  if (dtype == BLR_F16) mix_dispatch<f16>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+  else if (dtype == BLR_BF16) mix_dispatch<bf16>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+  else mix_dispatch<float>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+  BLR_CHECK_LAUNCH("blast_mix");
+  return BLR_OK;
+}
+
+}  // namespace blr

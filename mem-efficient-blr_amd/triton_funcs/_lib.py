@@ -1,0 +1,127 @@
+"""ctypes binding of libblr.so (the HIP kernels) for the triton_funcs call surface.
+
+The library is built in-tree (``build.py`` next to this package) into ``../lib/libblr.so``;
+``BLR_LIB`` overrides the path.  There is no fallback: if the library is missing, or a call
+fails, the caller gets an exception.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.environ.get("BLR_LIB", os.path.join(_HERE, "..", "lib", "libblr.so"))
+
+# enums of include/blr.h
+F16, BF16, F32 = 0, 1, 2
+U_RQ, U_QR = 0, 1
+S_JIR, S_RIJ, S_IJR = 0, 1, 2
+ALGO_AUTO, ALGO_STREAM, ALGO_TILED, ALGO_FUSED, ALGO_STREAM_SPLIT = 0, 1, 2, 3, 4
+W2_SR, W2_RS = 0, 1
+OUT_INTERLEAVED, OUT_BLOCKED = 0, 1
+
+_c = ctypes
+_vp, _i, _i64, _sz = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_size_t
+
+_SIGNATURES = {
+    "blr_last_error": (_c.c_char_p, []),
+    "blr_version": (_i, []),
+    "blr_device_cus": (_i, []),
+    "blr_blast_workspace_bytes": (_sz, [_i] * 7),
+    "blr_blast_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp] + [_i] * 9 + [_vp, _sz, _vp]),
+    "blr_blast_q_workspace_bytes": (_sz, [_i] * 6),
+    "blr_blast_q_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64] + [_i] * 8 + [_vp, _sz, _vp]),
+    "blr_quantize_sym": (_i, [_vp, _i, _i64, _i64, _i64, _i, _vp, _vp, _vp]),
+    "blr_monarch_workspace_bytes": (_sz, [_i] * 7),
+    "blr_monarch_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _i64, _vp] + [_i] * 9 + [_vp, _sz, _vp]),
+    "blr_low_rank_workspace_bytes": (_sz, [_i] * 6),
+    "blr_low_rank_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _i64, _vp] + [_i] * 6 + [_vp, _sz, _vp]),
+    "blr_dense_workspace_bytes": (_sz, [_i] * 5),
+    "blr_dense_fwd": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp]),
+    "blr_probe_dst_words": (_i, []),
+    "blr_stream_probe": (_i, [_vp, _sz, _vp, _vp]),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+class BlrError(RuntimeError):
+    pass
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES)
+
+
+def lib():
+    """Load libblr.so once; raise if it is not there."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                path = os.path.abspath(LIB_PATH)
+                if not os.path.exists(path):
+                    raise BlrError(f"libblr.so not found at {path}: build it with `python mem-efficient-blr_amd/build.py`")
+                handle = ctypes.CDLL(path)
+                for name, (res, args) in _SIGNATURES.items():
+                    fn = getattr(handle, name)
+                    fn.restype, fn.argtypes = res, args
+                _lib = handle
+    return _lib
+
+
+def check(rc, what):
+    if rc != 0:
+        raise BlrError(f"{what} failed ({rc}): {lib().blr_last_error().decode()}")
+
+
+def dtype_code(dt):
+    if dt == torch.float16:
+        return F16
+    if dt == torch.bfloat16:
+        return BF16
+    if dt == torch.float32:
+        return F32
+    raise BlrError(f"unsupported dtype {dt}")
+
+
+def stream_ptr(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def rows(x):
+    """(…, in) -> 2-D view (N, in) with unit inner stride (copy only if the strides force one)."""
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+        x2 = x2.contiguous()
+    return x2
+
+
+# Workspaces, one per (device, stream, kind).  kind "stream": the streaming kernels keep their
+# barrier and split counters in its head; it must start zeroed, they leave it zeroed, and nothing
+# else may scribble on it.  kind "scratch": plain scratch of the tiled kernels.  Work on one stream
+# is ordered, so sharing inside a stream is safe.
+_workspaces = {}
+
+
+def workspace(device, nbytes, algo=ALGO_AUTO, M=None, dtype=None):
+    streaming = algo in (ALGO_STREAM, ALGO_STREAM_SPLIT) or (
+        algo == ALGO_AUTO and M is not None and M <= 16 and dtype != F32)
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream, "stream" if streaming else "scratch")
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        size = max(int(nbytes), 1 << 20)
+        ws = torch.zeros(size, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def require_gpu(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise BlrError("libblr kernels need tensors on the GPU (there is no CPU path)")

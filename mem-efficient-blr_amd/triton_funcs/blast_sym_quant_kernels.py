@@ -1,0 +1,116 @@
+"""Symmetric-quantized BLAST behind the reference's triton_funcs.blast_sym_quant_kernels names.
+
+``triton_blast_bmm_int8_fp16(x, U, V, S, config)`` keeps the reference's signature and bmm
+operand layouts (U (b, q, r), V (b, p, r), S (r, b2, b1); reference
+triton_funcs/blast_sym_quant_kernels.py:558-580).  U and V are passed as ``QuantFactor``s -
+int8 or packed-int4 codes plus fp16 per-output-channel scales, made once by
+``quantize_blast_factors`` - and are dequantised in registers inside the streaming kernel:
+the scale of V is folded into S, the scale of U is applied to the output row.
+
+The reference has no weight quantizer; the scheme is this library's own: symmetric, per output
+channel, scale = fp16(max|w| / Qmax) (1 for an all-zero channel), code = clamp(rne(w / scale),
+-Qmax, Qmax) with Qmax = 127 (int8) or 7 (int4); int4 codes are packed two per byte along r,
+low nibble = even r.
+"""
+from __future__ import annotations
+
+from typing import NamedTuple
+
+import torch
+
+from . import _lib as L
+
+__all__ = ["QuantFactor", "quantize_sym", "quantize_blast_factors", "triton_blast_bmm_int8_fp16",
+           "triton_blast_bmm_int4_fp16", "get_triton_blast_bmm_xv_int8_fp16_config",
+           "get_triton_blast_bmm_sxv_int8_fp16_config", "get_triton_blast_bmm_usxv_int8_fp16_config"]
+
+_last_config = {}
+
+
+class QuantFactor(NamedTuple):
+    codes: torch.Tensor      # int8 (…, r) or uint8 (…, r/2) when bits == 4
+    scales: torch.Tensor     # float16
+    bits: int
+    shape: tuple             # logical (unpacked) shape of the factor
+
+
+def quantize_sym(w, reduce_dim, bits=8):
+    """Quantize ``w`` on the GPU with max-abs taken over ``reduce_dim``.
+
+    Returns (codes, scales): codes int8 of w's shape (bits=8) or uint8 with the last axis halved
+    (bits=4); scales float16 of w's shape without ``reduce_dim``."""
+    L.require_gpu(w)
+    assert bits in (8, 4)
+    w = w.contiguous()
+    reduce_dim = reduce_dim % w.dim()
+    outer = 1
+    for d in w.shape[:reduce_dim]:
+        outer *= d
+    inner = 1
+    for d in w.shape[reduce_dim + 1:]:
+        inner *= d
+    red = w.shape[reduce_dim]
+    if bits == 8:
+        codes = torch.empty(w.shape, dtype=torch.int8, device=w.device)
+    else:
+        assert w.shape[-1] % 2 == 0, "int4 packing needs an even last axis"
+        codes = torch.empty(w.shape[:-1] + (w.shape[-1] // 2,), dtype=torch.uint8, device=w.device)
+    scales = torch.empty(w.shape[:reduce_dim] + w.shape[reduce_dim + 1:], dtype=torch.float16, device=w.device)
+    rc = L.lib().blr_quantize_sym(w.data_ptr(), L.dtype_code(w.dtype), outer, red, inner, bits,
+                                  codes.data_ptr(), scales.data_ptr(), L.stream_ptr(w.device))
+    L.check(rc, "blr_quantize_sym")
+    return codes, scales
+
+
+def quantize_blast_factors(U, V, bits=8):
+    """U (b, q, r) -> per-(b, q) scales; V (b, p, r) -> per-(b, r) scales (V maps p -> r)."""
+    uc, us = quantize_sym(U, 2, bits)
+    vc, vs = quantize_sym(V, 1, bits)
+    return QuantFactor(uc, us, bits, tuple(U.shape)), QuantFactor(vc, vs, bits, tuple(V.shape))
+
+
+def triton_blast_bmm_int8_fp16(x, U, V, S, config=(None, None, None)):
+    if not (isinstance(U, QuantFactor) and isinstance(V, QuantFactor)):
+        raise L.BlrError("triton_blast_bmm_int8_fp16 takes QuantFactor U and V (see quantize_blast_factors)")
+    L.require_gpu(x, S, U.codes, V.codes)
+    assert U.bits == V.bits
+    b1, p, r = V.shape
+    b2, q, r_u = U.shape
+    assert b1 == b2                                   # reference blast_sym_quant_kernels.py:568-569
+    assert b1 != 1 and b2 != 1
+    assert r_u == r
+    assert tuple(S.shape) == (r, b2, b1) and S.is_contiguous()
+    assert x.dtype in (torch.float16, torch.bfloat16) and S.dtype == x.dtype
+    assert x.shape[-1] == b1 * p
+    algo = L.ALGO_AUTO
+    if isinstance(config, dict):
+        algo = int(config.get("algo", L.ALGO_AUTO))
+    dt = L.dtype_code(x.dtype)
+    x2 = L.rows(x)
+    M, in_f, out_f = x2.shape[0], b1 * p, b2 * q
+    out = torch.empty((M, out_f), device=x.device, dtype=x.dtype)
+    lib = L.lib()
+    ws = L.workspace(x.device, lib.blr_blast_q_workspace_bytes(M, in_f, out_f, b1, r, U.bits), L.ALGO_STREAM)
+    rc = lib.blr_blast_q_fwd(x2.data_ptr(), x2.stride(0), U.codes.data_ptr(), U.scales.data_ptr(),
+                             V.codes.data_ptr(), V.scales.data_ptr(), S.data_ptr(), out.data_ptr(), out.stride(0),
+                             M, in_f, out_f, b1, r, dt, U.bits, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
+    L.check(rc, "triton_blast_bmm_int8_fp16")
+    _last_config["q"] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": b1, "rank": r, "bits": U.bits}
+    return out.reshape(*x.shape[:-1], out_f)
+
+
+def triton_blast_bmm_int4_fp16(x, U, V, S, config=(None, None, None)):
+    assert isinstance(U, QuantFactor) and U.bits == 4
+    return triton_blast_bmm_int8_fp16(x, U, V, S, config)
+
+
+def get_triton_blast_bmm_xv_int8_fp16_config():
+    return _last_config.get("q")
+
+
+def get_triton_blast_bmm_sxv_int8_fp16_config():
+    return _last_config.get("q")
+
+
+def get_triton_blast_bmm_usxv_int8_fp16_config():
+    return _last_config.get("q")

@@ -1,0 +1,164 @@
+"""GPU parity: BLAST through the C ABI (via the triton_funcs call surface) vs the CPU oracle.
+
+Tolerance: max|y - y_ref| <= 1e-2 * max|y_ref| for fp16 (2e-2 for bf16, 1e-4 for fp32), y_ref
+computed in float64 from the same dtype-rounded inputs.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import blr_oracle as O
+from gpu_util import assert_close, back, blast_inputs, dev, rounded, say
+
+pytestmark = pytest.mark.gpu
+
+ALGO = {"auto": 0, "stream": 1, "tiled": 2, "split": 4}
+
+
+def _run_blast(fn_name, x, U, Vt, S, dtype, algo=None):
+    from triton_funcs import blast_kernels as K
+    fn = getattr(K, fn_name)
+    if "bmm" in fn_name:
+        Uk, Vk, Sk = O.blast_to_bmm_layout(U, Vt, S)
+    else:
+        Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+    args = [dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype)]
+    if fn_name.endswith("fp16") and algo is not None:
+        return fn(*args, {"algo": ALGO[algo]})
+    return fn(*args)
+
+
+def _ref(x, U, Vt, S, dtype):
+    return O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))
+
+
+SMALL = [(2, 3, 2, 2, (2,)), (3, 5, 7, 6, (2, 3)), (4, 8, 16, 8, (1, 5)), (2, 40, 24, 72, (1, 33))]
+
+
+@pytest.mark.parametrize("shape", SMALL)
+@pytest.mark.parametrize("name", ["triton_blast_partial_fp32", "triton_blast_partial_grouped_fp32",
+                                  "triton_blast_partial_grouped_persistent_fp32", "triton_blast_full_fp32",
+                                  "triton_blast_bmm_fp32"])
+def test_blast_fp32_names_with_intermediates(name, shape):
+    b, p, q, r, lead = shape
+    say(f"[case] {name} b={b} p={p} q={q} r={r} lead={lead}")
+    x, U, Vt, S = blast_inputs(b, p, q, r, lead, seed=1)
+    out, z, y = _run_blast(name, x, U, Vt, S, torch.float32)
+    ro, rz, ry = _ref(x, U, Vt, S, torch.float32)
+    assert tuple(out.shape) == tuple(lead) + (b * q,)
+    assert_close(out, ro, torch.float32, name + " out")
+    if "bmm" in name:      # y (r, b1, N), z (b2, r, N)
+        assert_close(y, np.transpose(ry, (2, 0, 1)), torch.float32, name + " y")
+        assert_close(z, np.transpose(rz, (0, 2, 1)), torch.float32, name + " z")
+    else:                  # y (b1, N, r), z (b2, N, r)
+        assert_close(y, ry, torch.float32, name + " y")
+        assert_close(z, rz, torch.float32, name + " z")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("algo", ["stream", "split", "tiled"])
+@pytest.mark.parametrize("name", ["triton_blast_full_fp16", "triton_blast_bmm_fp16"])
+@pytest.mark.parametrize("shape", SMALL + [(4, 64, 96, 128, (3,)), (16, 32, 40, 64, (16,))])
+def test_blast_small_all_algorithms(name, shape, algo, dtype):
+    b, p, q, r, lead = shape
+    say(f"[case] {name} algo={algo} {dtype} b={b} p={p} q={q} r={r} lead={lead}")
+    x, U, Vt, S = blast_inputs(b, p, q, r, lead, seed=2)
+    if algo in ("stream", "split") and int(np.prod(lead)) > 16:
+        from triton_funcs import _lib as L
+        with pytest.raises(L.BlrError):            # the streaming kernels serve M <= 16 only
+            _run_blast(name, x, U, Vt, S, dtype, algo)
+        return
+    out = _run_blast(name, x, U, Vt, S, dtype, algo)
+    assert out.dtype == dtype and tuple(out.shape) == tuple(lead) + (b * q,)
+    assert_close(out, _ref(x, U, Vt, S, dtype)[0], dtype, f"{name}/{algo}")
+
+
+def test_blast_gpt2_config_fp32_and_fp16():
+    """BASELINE config 1: x [1,128,768], b=4, U [4,768,128], V [4,192,128], S [4,4,128], seed 0."""
+    b, p, q, r = 4, 192, 768, 128
+    x, U, Vt, S = blast_inputs(b, p, q, r, (1, 128), seed=0)
+    say("[case] gpt2 c_fc fp32")
+    out, z, y = _run_blast("triton_blast_partial_grouped_fp32", x, U, Vt, S, torch.float32)
+    ro, rz, ry = _ref(x, U, Vt, S, torch.float32)
+    assert tuple(out.shape) == (1, 128, 3072)
+    assert_close(out, ro, torch.float32, "gpt2 fp32 out")
+    assert_close(z, rz, torch.float32, "gpt2 fp32 z")
+    for name in ("triton_blast_partial_grouped_fp16", "triton_blast_bmm_fp16"):
+        say(f"[case] gpt2 c_fc {name}")
+        out = _run_blast(name, x, U, Vt, S, torch.float16)
+        assert_close(out, _ref(x, U, Vt, S, torch.float16)[0], torch.float16, "gpt2 " + name)
+
+
+LLAMA = {"qkvo": (256, 256, 512), "gate_up": (256, 1376, 1024), "down": (688, 256, 1024)}
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("layer", list(LLAMA))
+@pytest.mark.parametrize("name", ["triton_blast_full_fp16", "triton_blast_partial_grouped_fp16", "triton_blast_bmm_fp16"])
+def test_blast_llama7b_decode(name, layer, M):
+    p, q, r = LLAMA[layer]
+    b = 16
+    say(f"[case] llama7b {layer} {name} M={M}")
+    x, U, Vt, S = blast_inputs(b, p, q, r, (1, M), seed=0)
+    for algo in ("stream", "split"):
+        out = _run_blast(name, x, U, Vt, S, torch.float16, algo)
+        assert_close(out, _ref(x, U, Vt, S, torch.float16)[0], torch.float16, f"{layer}/{name}/{algo}/M{M}")
+
+
+@pytest.mark.parametrize("layer", list(LLAMA))
+@pytest.mark.parametrize("name", ["triton_blast_full_fp16", "triton_blast_bmm_fp16"])
+def test_blast_llama7b_prefill_rows(name, layer):
+    """M = 2048 at full shape; rows are independent, so a sample of rows is checked against the oracle."""
+    p, q, r = LLAMA[layer]
+    b, M = 16, 2048
+    say(f"[case] llama7b {layer} {name} M={M}")
+    x, U, Vt, S = blast_inputs(b, p, q, r, (1, M), seed=0)
+    out = _run_blast(name, x, U, Vt, S, torch.float16)
+    assert tuple(out.shape) == (1, M, b * q)
+    rows = [0, 1, 31, 32, 127, 128, 255, 256, 1000, 1791, 2046, 2047]
+    ref = _ref(x[:, rows], U, Vt, S, torch.float16)[0]
+    assert_close(out[:, rows], ref, torch.float16, f"{layer}/{name}/M{M}")
+    assert torch.isfinite(out).all()
+
+
+def test_blast_linearity_full_size():
+    """Size-independent property at full gate_up shape: f(2a - 3b) == 2 f(a) - 3 f(b) within rounding."""
+    from triton_funcs import blast_kernels as K
+    p, q, r = LLAMA["gate_up"]
+    b = 16
+    x, U, Vt, S = blast_inputs(b, p, q, r, (2, 64), seed=3)
+    Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+    Uk, Vk, Sk = dev(Uk, torch.float16), dev(Vk, torch.float16), dev(Sk, torch.float16)
+    xa, xb = dev(x[0:1], torch.float16), dev(x[1:2], torch.float16)
+    say("[case] linearity gate_up M=64")
+    fa = K.triton_blast_full_fp16(xa, Uk, Vk, Sk).float()
+    fb = K.triton_blast_full_fp16(xb, Uk, Vk, Sk).float()
+    fc = K.triton_blast_full_fp16((2 * xa.float() - 3 * xb.float()).half(), Uk, Vk, Sk).float()
+    ref = 2 * fa - 3 * fb
+    assert (fc - ref).abs().max() <= 2e-2 * ref.abs().max()
+
+
+def test_blast_strided_x_and_bad_args():
+    from triton_funcs import blast_kernels as K
+    from triton_funcs import _lib as L
+    b, p, q, r = 4, 16, 8, 32
+    x, U, Vt, S = blast_inputs(b, p, q, r, (6,), seed=4)
+    Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+    big = torch.zeros((6, 2 * b * p), device="cuda", dtype=torch.float16)
+    big[:, : b * p] = dev(x, torch.float16)
+    xv = big[:, : b * p]                                   # row stride 2*in_f
+    say("[case] strided x")
+    out = K.triton_blast_full_fp16(xv, dev(Uk, torch.float16), dev(Vk, torch.float16), dev(Sk, torch.float16))
+    assert_close(out, _ref(x, U, Vt, S, torch.float16)[0], torch.float16, "strided x")
+    with pytest.raises(AssertionError):                      # b1 != b2
+        K.triton_blast_full_fp16(xv, dev(Uk[:2], torch.float16), dev(Vk, torch.float16), dev(Sk, torch.float16))
+    lib = L.lib()
+    rc = lib.blr_blast_fwd(None, 0, None, None, None, None, 0, None, None, 1, 8, 8, 2, 2, 0, 0, 0, 0, None, 0, None)
+    assert rc == -1 and b"null" in lib.blr_last_error()
+    t = torch.zeros(64, device="cuda", dtype=torch.float16)
+    rc = lib.blr_blast_fwd(t.data_ptr(), 9, t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), 9, None, None,
+                           1, 9, 9, 2, 2, 0, 0, 0, 0, None, 0, None)
+    assert rc == -2                                          # in_f not divisible by b
+    rc = lib.blr_blast_fwd(t.data_ptr(), 8, t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), 8, None, None,
+                           1, 8, 8, 2, 2, 0, 0, 0, 2, None, 0, None)
+    assert rc == -3                                          # tiled algorithm without a workspace
