@@ -50,6 +50,7 @@ struct PhaseDesc {
   int batch, K, N;
   int lpr_log2, kc, ksplit, nchunks;        // KN tiling
   int nk_split_k;                           // NK: the 4 waves of a workgroup split K instead of rows
+  int kn_mfma;                              // KN: matrix-core variant (lanes transpose 8x8 blocks in registers)
   int amode; const void* a; int64_t lda, a_bs;
   int emode; void* o; int64_t ldo, o_bs, o_ns;
   int perm_per;                             // > 0: Monarch scatter on E_F32
@@ -238,11 +239,71 @@ __device__ __forceinline__ float act_load(const PhaseDesc& d, int M, int bt, int
   return acc;
 }
 
-// ---- KN phase -----------------------------------------------------------------------------------
-__device__ __forceinline__ bool nk_use_dot(const PhaseDesc& d, int MT);
-__device__ __forceinline__ bool nkd_prefetch(const PhaseDesc& d, int item, u32x4 (&pf)[8]);
-__device__ __forceinline__ bool nk_prefetch(const PhaseDesc& d, int item, u32x4 (&pf)[8]);
+// Split-k epilogue of a KN item: once this workgroup's partial sums are device-visible it checks
+// in on the column chunk's counter; the last one to do so adds all slots in a fixed order and emits.
+template <typename T>
+__device__ __forceinline__ void kn_splitk_finish(const PhaseDesc& d, int M, int bt, int nc, int n0, int NC, float* red,
+                                                 float* zcur, int trb) {
+  __shared__ int s_last;
+  const int tid = threadIdx.x;
+  if (d.ksplit <= 1) return;
+  drain_stores();                                  // this workgroup's partial sums are device-visible
+  __syncthreads();
+  if (tid == 0) {
+    unsigned old = __hip_atomic_fetch_add(&d.counters[bt * d.nchunks + nc], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (old == (unsigned)(d.ksplit - 1));
+  }
+  __syncthreads();
+  TR(trb + 4);
+  if (!s_last) return;                             // (uniform over the workgroup)
+  const int64_t slot = (int64_t)d.batch * M * d.N;
+  if ((d.N & 3) == 0 && slot * d.ksplit * 4 < 0x7fffffffLL) {
+    // All 256 threads: thread (vc, sg) adds slots sg, sg+G, ... of four columns, then the G
+    // groups are added in order through LDS.  One or two rounds of 16-byte loads in total.
+    const int vcols = NC >> 2;
+    const int G = 256 / vcols;
+    const int vc = tid % vcols, sg = tid / vcols;
+    f32x4* red4 = reinterpret_cast<f32x4*>(red);
+    for (int m = 0; m < M; ++m) {
+      f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+      const int gn = n0 + vc * 4;
+      if (sg < G && gn < d.N) {
+        const uint32_t off0 = (uint32_t)((((int64_t)bt * M + m) * d.N + gn) * 4);
+        int sidx = sg;
+        for (; sidx + 7 * G < d.ksplit; sidx += 8 * G) {
+          f32x4 t[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) t[u] = ld_dev4(d.part, off0 + (uint32_t)((sidx + u * G) * slot * 4));
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v += t[u];
+        }
+        for (; sidx < d.ksplit; sidx += G) v += ld_dev4(d.part, off0 + (uint32_t)(sidx * slot * 4));
+      }
+      __syncthreads();
+      if (sg < G) red4[sg * vcols + vc] = v;
+      __syncthreads();
+      if (tid < vcols && gn < d.N) {
+        f32x4 t = red4[tid];
+        for (int g = 1; g < G; ++g) t += red4[g * vcols + tid];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) emit<T>(d, M, bt, m, gn + e, t[e], zcur);
+      }
+    }
+  } else {
+    for (int idx = tid; idx < NC * M; idx += 256) {
+      int m = idx / NC, col = idx - m * NC;
+      int gn = n0 + col;
+      if (gn >= d.N) continue;
+      const float* p0 = &d.part[((int64_t)bt * M + m) * d.N + gn];
+      float v = 0.0f;
+      for (int sidx = 0; sidx < d.ksplit; ++sidx) v += ld_dev(p0 + sidx * slot);
+      emit<T>(d, M, bt, m, gn, v, zcur);
+    }
+  }
+  if (tid == 0) __hip_atomic_store(&d.counters[bt * d.nchunks + nc], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
+// ---- KN phase -----------------------------------------------------------------------------------
 struct KnItem {
   int nc, ks, bt, k0, kc, n0, n;
   bool col_ok;
@@ -261,38 +322,16 @@ __device__ __forceinline__ KnItem kn_item(const PhaseDesc& d, int item, int cv) 
   return it;
 }
 
-template <int WB> __device__ __forceinline__ Raw8<WB> from_prefetch(const u32x4& v);
-template <> __device__ __forceinline__ Raw8<16> from_prefetch<16>(const u32x4& v) { return Raw8<16>{v}; }
-template <> __device__ __forceinline__ Raw8<8> from_prefetch<8>(const u32x4& v) { return Raw8<8>{u32x2{v[0], v[1]}}; }   // never taken
-template <> __device__ __forceinline__ Raw8<4> from_prefetch<4>(const u32x4& v) { return Raw8<4>{v[0]}; }                // never taken
-
-// Issue the first UNR row loads of `item` (f16/bf16, 16-byte friendly rows).  Returns whether it did.
-__device__ __forceinline__ bool kn_prefetch(const PhaseDesc& d, int item, u32x4 (&pf)[UNR]) {
-  const int tid = threadIdx.x;
-  const int rpp = 256 >> d.lpr_log2;
-  const int cv = tid & ((1 << d.lpr_log2) - 1), rs = tid >> d.lpr_log2;
-  if (item >= d.batch * d.ksplit * d.nchunks) return false;
-  KnItem it = kn_item(d, item, cv);
-  if (!it.col_ok || rs + (UNR - 1) * rpp >= it.kc) return false;
-#pragma unroll
-  for (int u = 0; u < UNR; ++u) pf[u] = load_raw8<16>(d.W, it.wbase + (int64_t)(rs + u * rpp) * d.ldw).v;
-  return true;
-}
-
 template <typename T, int MT, int WB, bool VEC>
 __device__ __forceinline__ void phase_kn(const PhaseDesc& d, int M, float* smem, int trb, float* zcur) {
-  u32x4 pf[UNR]; bool pf_ok = false; const PhaseDesc* later = nullptr; const int MT_rt = MT;   // cross-phase prefetch: disabled
-  (void)pf; (void)MT_rt;
   constexpr int KC_LD = AS_FLOATS / MT;            // row stride of the staged activations
   float* a_s = smem;                               // [MT][KC_LD]
   float* red = smem + AS_FLOATS;                   // [4 waves][RED_MG][NC_MAX]
-  __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lpr = 1 << d.lpr_log2, rpp = 256 >> d.lpr_log2;
   const int cv = tid & (lpr - 1), rs = tid >> d.lpr_log2;
   const int NC = lpr * 8;
   const int total = d.batch * d.ksplit * d.nchunks;
-  const bool pf_mine = pf_ok && later == nullptr;  // pf holds this phase's first slab (set by an earlier phase)
   for (int item = blockIdx.x; item < total; item += gridDim.x) {
     const KnItem it = kn_item(d, item, cv);
     const int bt = it.bt, kc = it.kc, n0 = it.n0;
@@ -302,19 +341,9 @@ __device__ __forceinline__ void phase_kn(const PhaseDesc& d, int M, float* smem,
     Raw8<WB> raw[UNR];
     bool have_raw = false;
     if (VEC && it.col_ok && kk + (UNR - 1) * rpp < kc) {
-      if (WB == 16 && pf_mine && item == (int)blockIdx.x) {
 #pragma unroll
-        for (int u = 0; u < UNR; ++u) raw[u] = from_prefetch<WB>(pf[u]);
-      } else {
-#pragma unroll
-        for (int u = 0; u < UNR; ++u) raw[u] = load_raw8<WB>(d.W, it.wbase + (int64_t)(kk + u * rpp) * d.ldw);
-      }
+      for (int u = 0; u < UNR; ++u) raw[u] = load_raw8<WB>(d.W, it.wbase + (int64_t)(kk + u * rpp) * d.ldw);
       have_raw = true;
-    }
-    if (later && item == (int)blockIdx.x) {        // this phase's rows are on their way: now start the last phase's first slab
-      if (later->kind == PH_KN) pf_ok = kn_prefetch(*later, blockIdx.x, pf);
-      else if (later->kind == PH_NK) pf_ok = nk_use_dot(*later, MT_rt) ? nkd_prefetch(*later, blockIdx.x, pf) : nk_prefetch(*later, blockIdx.x, pf);
-      later = nullptr;
     }
     __syncthreads();
     if ((d.amode == A_F32 || d.amode == A_Z) && ((d.K | it.k0 | kc) & 3) == 0) {       // 16-byte device-scope loads
@@ -421,67 +450,103 @@ __device__ __forceinline__ void phase_kn(const PhaseDesc& d, int M, float* smem,
       }
     }
     TR(trb + 3);
-    if (d.ksplit > 1) {
-      drain_stores();                              // this workgroup's partial sums are device-visible
-      __syncthreads();
-      if (tid == 0) {
-        unsigned old = __hip_atomic_fetch_add(&d.counters[bt * d.nchunks + it.nc], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (old == (unsigned)(d.ksplit - 1));
+    kn_splitk_finish<T>(d, M, bt, it.nc, n0, NC, red, zcur, trb);
+  }
+}
+
+// ---- KN phase on the matrix cores (M up to 16 at the cost of M = 1) ------------------------------------
+// Column chunk of 128 (16 lanes x 8), 16 row slots of 8 consecutive rows: one batch of eight
+// 16-byte loads per lane covers 128 rows x 128 columns.  Each lane transposes its 8x8 block in
+// registers (v_perm) into eight B fragments of v_mfma_f32_16x16x32 - fragment e holds column
+// 8*cv + e for the lane's 8 rows - and the activations, staged in LDS as [16][k], are the A
+// fragment.  A wave contracts its own 32 rows per batch; the four waves are added through LDS.
+constexpr int KNM_KC_MAX = 384;                  // 16 x (384 + 8) two-byte activations fit the staging area
+
+template <typename T>
+__device__ __forceinline__ void phase_kn_mfma(const PhaseDesc& d, int M, float* smem, int trb, float* zcur) {
+  using V8 = typename TypeTraits<T>::vec8;
+  T* a_s = reinterpret_cast<T*>(smem);              // [16][ka_ld]
+  float* red = smem + AS_FLOATS;                   // [4 waves][4 fragments][64 lanes][4]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int cv = lane & 15, kg = lane >> 4, rs = wave * 4 + kg;
+  const int NC = 128;
+  const int total = d.batch * d.ksplit * d.nchunks;
+  for (int item = blockIdx.x; item < total; item += gridDim.x) {
+    const KnItem it = kn_item(d, item, cv);
+    const int bt = it.bt, kc = it.kc, n0 = it.n0;
+    const int kcp = (kc + 127) / 128 * 128;
+    const int ka_ld = kcp + 8;
+    u32x4 raw[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) raw[u] = load_raw8<16>(d.W, it.wbase + (int64_t)min(rs * 8 + u, kc - 1) * d.ldw).v;
+    __syncthreads();
+    if ((d.amode == A_F32 || d.amode == A_Z) && ((d.K | it.k0 | kc) & 3) == 0) {
+      const int kq = kcp >> 2;
+      for (int idx = tid; idx < 16 * kq; idx += 256) {
+        int m = idx / kq, ka = (idx - m * kq) * 4;
+        f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (m < M && ka < kc) v = ld_dev4(d.amode == A_Z ? zcur : reinterpret_cast<const float*>(d.a), (uint32_t)((((int64_t)bt * M + m) * d.K + it.k0 + ka) * 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a_s[m * ka_ld + ka + e] = TypeTraits<T>::from_f32(v[e]);
       }
-      __syncthreads();
-      TR(trb + 4);
-      if (s_last) {                                // every other k-chunk of this column chunk is done
-        const int64_t slot = (int64_t)d.batch * M * d.N;
-        if ((d.N & 3) == 0 && slot * d.ksplit * 4 < 0x7fffffffLL) {
-          // All 256 threads: thread (vc, sg) adds slots sg, sg+G, ... of four columns, then the G
-          // groups are added in order through LDS.  One or two rounds of 16-byte loads in total.
-          const int vcols = NC >> 2;
-          const int G = 256 / vcols;
-          const int vc = tid % vcols, sg = tid / vcols;
-          f32x4* red4 = reinterpret_cast<f32x4*>(red);
-          for (int m = 0; m < M; ++m) {
-            f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-            const int gn = n0 + vc * 4;
-            if (sg < G && gn < d.N) {
-              const uint32_t off0 = (uint32_t)((((int64_t)bt * M + m) * d.N + gn) * 4);
-              int sidx = sg;
-              for (; sidx + 7 * G < d.ksplit; sidx += 8 * G) {
-                f32x4 t[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) t[u] = ld_dev4(d.part, off0 + (uint32_t)((sidx + u * G) * slot * 4));
-#pragma unroll
-                for (int u = 0; u < 8; ++u) v += t[u];
-              }
-              for (; sidx < d.ksplit; sidx += G) v += ld_dev4(d.part, off0 + (uint32_t)(sidx * slot * 4));
-            }
-            __syncthreads();
-            if (sg < G) red4[sg * vcols + vc] = v;
-            __syncthreads();
-            if (tid < vcols && gn < d.N) {
-              f32x4 t = red4[tid];
-              for (int g = 1; g < G; ++g) t += red4[g * vcols + tid];
-#pragma unroll
-              for (int e = 0; e < 4; ++e) emit<T>(d, M, bt, m, gn + e, t[e], zcur);
-            }
-          }
-        } else {
-          for (int idx = tid; idx < NC * M; idx += 256) {
-            int m = idx / NC, col = idx - m * NC;
-            int gn = n0 + col;
-            if (gn >= d.N) continue;
-            const float* p0 = &d.part[((int64_t)bt * M + m) * d.N + gn];
-            float v = 0.0f;
-            for (int sidx = 0; sidx < d.ksplit; ++sidx) v += ld_dev(p0 + sidx * slot);
-            emit<T>(d, M, bt, m, gn, v, zcur);
-          }
-        }
-        if (tid == 0) __hip_atomic_store(&d.counters[bt * d.nchunks + it.nc], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      for (int idx = tid; idx < 16 * kcp; idx += 256) {
+        int m = idx / kcp, ka = idx - m * kcp;
+        a_s[m * ka_ld + ka] = TypeTraits<T>::from_f32((m < M && ka < kc) ? act_load<T>(d, M, bt, m, it.k0 + ka, zcur) : 0.0f);
       }
     }
-  }
-  if (later) {                                     // this workgroup had no item in this phase: still start the last phase's slab
-    if (later->kind == PH_KN) pf_ok = kn_prefetch(*later, blockIdx.x, pf);
-    else if (later->kind == PH_NK) pf_ok = nk_use_dot(*later, MT_rt) ? nkd_prefetch(*later, blockIdx.x, pf) : nk_prefetch(*later, blockIdx.x, pf);
+    __syncthreads();
+    TR(trb + 1);
+    f32x4 acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int kcur = 0; kcur < kcp; kcur += 128) {
+      u32x4 cur[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) cur[u] = raw[u];
+      if (kcur + 128 < kcp) {
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) raw[u] = load_raw8<16>(d.W, it.wbase + (int64_t)min(kcur + 128 + rs * 8 + u, kc - 1) * d.ldw).v;
+      }
+      const V8 af = *reinterpret_cast<const V8*>(&a_s[cv * ka_ld + kcur + rs * 8]);   // row m = lane % 16
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        u32x4 b;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          b[q] = __builtin_amdgcn_perm(cur[2 * q + 1][e >> 1], cur[2 * q][e >> 1], (e & 1) ? 0x07060302u : 0x05040100u);
+        acc[e] = TypeTraits<T>::mfma16(af, __builtin_bit_cast(V8, b), acc[e]);
+      }
+    }
+    TR(trb + 2);
+    // add the four waves, four fragments at a time; lane l of fragment e holds rows m = 4 (l / 16) + i, column n0 + 8 (l % 16) + e
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < 4; ++e) *reinterpret_cast<f32x4*>(&red[((wave * 4 + e) * 64 + lane) * 4]) = acc[h * 4 + e];
+      __syncthreads();
+      {
+        const int e = tid >> 6, l = tid & 63;
+        f32x4 v = *reinterpret_cast<const f32x4*>(&red[((0 * 4 + e) * 64 + l) * 4]);
+        v += *reinterpret_cast<const f32x4*>(&red[((1 * 4 + e) * 64 + l) * 4]);
+        v += *reinterpret_cast<const f32x4*>(&red[((2 * 4 + e) * 64 + l) * 4]);
+        v += *reinterpret_cast<const f32x4*>(&red[((3 * 4 + e) * 64 + l) * 4]);
+        const int gn = n0 + (l & 15) * 8 + h * 4 + e;
+        if (gn < d.N) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int m = (l >> 4) * 4 + i;
+            if (m < M) {
+              if (d.ksplit == 1) emit<T>(d, M, bt, m, gn, v[i], zcur);
+              else st_dev(&d.part[(((int64_t)it.ks * d.batch + bt) * M + m) * d.N + gn], v[i]);
+            }
+          }
+        }
+      }
+    }
+    TR(trb + 3);
+    kn_splitk_finish<T>(d, M, bt, it.nc, n0, NC, red, zcur, trb);
   }
 }
 
@@ -538,22 +603,8 @@ __device__ __forceinline__ u32x4 nk_load16(const void* W, int64_t row_off, int k
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + byte));
 }
 
-__device__ __forceinline__ bool nk_prefetch(const PhaseDesc& d, int item, u32x4 (&pf)[UNR]) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int Kp = (d.K + 31) / 32 * 32;
-  const int rows_per_item = d.nk_split_k ? 16 : 64;
-  if (item >= d.batch * ((d.N + rows_per_item - 1) / rows_per_item)) return false;
-  NkItem it = nk_item<32>(d, item, wave, lane & 15, Kp);
-  const int Kfull = d.K / 32 * 32;
-  if (it.kbeg + UNR * 32 > min(it.kend, Kfull)) return false;
-#pragma unroll
-  for (int u = 0; u < UNR; ++u) pf[u] = nk_load16<16>(d.W, it.row_off, it.kbeg + u * 32 + (lane >> 4) * 8);
-  return true;
-}
-
 template <typename T, int WB, bool VEC>
 __device__ __forceinline__ void phase_nk(const PhaseDesc& d, int M, float* smem, float* zcur) {
-  u32x4 pf[UNR]; const bool pf_ok = false; (void)pf;
   using V8 = typename TypeTraits<T>::vec8;
   constexpr int KSTEP = (WB == 16) ? 32 : (WB == 8 ? 64 : 128);   // k per 16-byte lane load x 4 lane groups
   constexpr int LANE_K = KSTEP / 4;                                  // k covered by one lane's 16 bytes
@@ -574,13 +625,8 @@ __device__ __forceinline__ void phase_nk(const PhaseDesc& d, int M, float* smem,
     int kk = it.kbeg;
     bool have_raw = false;
     if (VEC && kk + UNR * KSTEP <= kend_full) {       // weights do not depend on the activations: start them first
-      if (WB == 16 && pf_ok && item == (int)blockIdx.x) {
 #pragma unroll
-        for (int u = 0; u < UNR; ++u) raw[u] = pf[u];
-      } else {
-#pragma unroll
-        for (int u = 0; u < UNR; ++u) raw[u] = nk_load16<WB>(d.W, it.row_off, kk + u * KSTEP + kg * LANE_K);
-      }
+      for (int u = 0; u < UNR; ++u) raw[u] = nk_load16<WB>(d.W, it.row_off, kk + u * KSTEP + kg * LANE_K);
       have_raw = true;
     }
     if (it.bt != staged_bt) {
@@ -667,26 +713,8 @@ __device__ __forceinline__ bool nk_use_dot(const PhaseDesc& d, int MT) {
   return MT <= 4 && d.wbits == 16 && d.vec_ok && (d.K % 8 == 0) && d.K <= 512 * dot_kch(MT) && !d.nk_split_k;
 }
 
-__device__ __forceinline__ bool nkd_prefetch(const PhaseDesc& d, int item, u32x4 (&pf)[UNR]) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rgroups = (d.N + 63) / 64;
-  if (item >= d.batch * rgroups) return false;
-  const int kch = (d.K + 511) / 512;
-  if (4 * kch > UNR) return false;
-  const int rg = item % rgroups, bt = item / rgroups;
-  const int row0 = rg * 64 + wave * 16;
-#pragma unroll
-  for (int u = 0; u < UNR; ++u) {
-    const int r4 = u / 2, c = u % 2;               // matches the kch <= 2 layout of phase_nk_dot's first group
-    const int n = min(row0 + r4, d.N - 1), k = min(c * 512 + lane * 8, d.K - 8);
-    pf[u] = nk_load16<16>(d.W, (int64_t)bt * d.w_bs + (int64_t)n * d.ldw, k);
-  }
-  return true;
-}
-
 template <typename T, int MT>
 __device__ __forceinline__ void phase_nk_dot(const PhaseDesc& d, int M, float* smem, float* zcur) {
-  u32x4 pf[UNR]; const bool pf_ok = false; (void)pf;
   float* a_s = smem;                               // [MT][K] fp32
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rgroups = (d.N + 63) / 64;
@@ -708,12 +736,7 @@ __device__ __forceinline__ void phase_nk_dot(const PhaseDesc& d, int M, float* s
       }
     };
     u32x4 raw[UNR];
-    if (pf_ok && item == (int)blockIdx.x) {
-#pragma unroll
-      for (int u = 0; u < UNR; ++u) raw[u] = pf[u];
-    } else {
-      load_group(0, raw);
-    }
+    load_group(0, raw);
     if (bt != staged_bt) {
       __syncthreads();
       for (int idx = tid; idx < MT * d.K; idx += 256) {
@@ -865,7 +888,10 @@ __device__ __forceinline__ void phase_mix(const PhaseDesc& d, int M) {
 
 template <typename T, int MT, int WB, bool VEC>
 __device__ __forceinline__ void run_phase(const PhaseDesc& d, int M, float* smem, int trb, float* zcur) {
-  if (d.kind == PH_KN) phase_kn<T, MT, WB, VEC>(d, M, smem, trb, zcur);
+  if (d.kind == PH_KN) {
+    if (WB == 16 && VEC && d.kn_mfma) phase_kn_mfma<T>(d, M, smem, trb, zcur);
+    else phase_kn<T, MT, WB, VEC>(d, M, smem, trb, zcur);
+  }
   else if (d.kind == PH_NK) {
     if (MT <= 4 && WB == 16 && VEC && nk_use_dot(d, MT)) phase_nk_dot<T, (MT <= 4 ? MT : 1)>(d, M, smem, zcur);
     else phase_nk<T, WB, VEC>(d, M, smem, zcur);
@@ -944,8 +970,25 @@ size_t lds_bytes_for(const StreamParams& p) {
 int mt_for(int M) { return M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16))); }
 
 // Choose the KN tiling: lanes per row, k-chunk and split count, aiming at `target` work items.
-bool plan_kn(PhaseDesc& d, int MT, int target) {
+// Smallest M served by the matrix-core KN variant (tuning aid: BLR_KN_MFMA_MIN_M).
+int kn_mfma_min_m() { static int v = env_int("BLR_KN_MFMA_MIN_M", 5); return v; }
+
+bool plan_kn(PhaseDesc& d, int MT, int target, int M = 0) {
   const int vecs = (d.N + 7) / 8;
+  if (M >= kn_mfma_min_m() && d.wbits == 16 && d.vec_ok && d.K >= 8) {
+    d.kn_mfma = 1; d.lpr_log2 = 4;
+    d.nchunks = (vecs + 15) / 16;
+    if ((int64_t)d.batch * d.nchunks > MAX_COUNTERS / 2) { set_error("stream: too many column chunks"); return false; }
+    int split = (int)(target / ((int64_t)d.batch * d.nchunks));
+    if (split < 1) split = 1;
+    if (split > KSPLIT_MAX) split = KSPLIT_MAX;
+    int kc = ((d.K + split - 1) / split + 127) / 128 * 128;
+    if (kc > KNM_KC_MAX) kc = KNM_KC_MAX;
+    if (kc > d.K) kc = d.K;
+    d.kc = kc; d.ksplit = (d.K + kc - 1) / kc;
+    if (d.ksplit > KSPLIT_MAX) { set_error("stream: K=%d too deep", d.K); return false; }
+    return true;
+  }
   const int kc_max = AS_FLOATS / MT;
   int lg_full = 2;
   while ((1 << lg_full) < vecs && lg_full < 6) ++lg_full;   // lanes per row: next pow2 >= N/8 within [4, 64]
@@ -1145,7 +1188,7 @@ int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st) {
   }
   y.part = w.part; y.counters = w.counters;
   y.vec_ok = (a.wbits != 16) ? 1 : (aligned(a.V, 16) && a.r % 8 == 0);
-  if (!plan_kn(y, MT, target)) return BLR_ERR_UNSUPPORTED;
+  if (!plan_kn(y, MT, target, a.M)) return BLR_ERR_UNSUPPORTED;
 
   if (p.nph == 3) p.ph[1] = mix;
 
@@ -1165,7 +1208,7 @@ int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st) {
   if (a.u_layout == BLR_U_RQ) {
     o.kind = PH_KN; o.w_bs = (int64_t)a.r * Q; o.ldw = Q;
     o.vec_ok = (a.wbits != 16) ? 1 : (aligned(a.U, 16) && Q % 8 == 0);
-    if (!plan_kn(o, MT, target)) return BLR_ERR_UNSUPPORTED;
+    if (!plan_kn(o, MT, target, a.M)) return BLR_ERR_UNSUPPORTED;
   } else {
     o.kind = PH_NK; o.w_bs = (int64_t)Q * a.r; o.ldw = a.r;
     o.vec_ok = (a.wbits != 16) ? 1 : (aligned(a.U, 16) && a.r % 8 == 0);
@@ -1199,7 +1242,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
     d.emode = E_OUT; d.o = a.out; d.ldo = a.ldo; d.o_bs = 0; d.o_ns = 1;
     d.part = w.part; d.counters = w.counters;
     d.vec_ok = aligned(a.W1, 16) && a.out_f % 8 == 0;
-    if (!plan_kn(d, MT, target)) return BLR_ERR_UNSUPPORTED;
+    if (!plan_kn(d, MT, target, a.M)) return BLR_ERR_UNSUPPORTED;
     return launch(p, a.dtype, a.split, st);
   }
   if (a.op == 1) {                             // low rank: z = x A (in, r); out = z B (r, out)
@@ -1211,14 +1254,14 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
     d.emode = E_F32; d.o = w.buf0; d.ldo = a.r;
     d.part = w.part; d.counters = w.counters;
     d.vec_ok = aligned(a.W1, 16) && a.r % 8 == 0;
-    if (!plan_kn(d, MT, target)) return BLR_ERR_UNSUPPORTED;
+    if (!plan_kn(d, MT, target, a.M)) return BLR_ERR_UNSUPPORTED;
     PhaseDesc& e = p.ph[1];
     e.kind = PH_KN; e.wbits = 16; e.W = a.W2; e.ldw = a.out_f; e.batch = 1; e.K = a.r; e.N = a.out_f;
     e.amode = A_F32; e.a = w.buf0;
     e.emode = E_OUT; e.o = a.out; e.ldo = a.ldo; e.o_ns = 1;
     e.part = w.part; e.counters = w.counters + MAX_COUNTERS / 2;
     e.vec_ok = aligned(a.W2, 16) && a.out_f % 8 == 0;
-    if (!plan_kn(e, MT, target)) return BLR_ERR_UNSUPPORTED;
+    if (!plan_kn(e, MT, target, a.M)) return BLR_ERR_UNSUPPORTED;
     return launch(p, a.dtype, a.split, st);
   }
   // Monarch: out1 = scatter(x_k w1_k); out = out1_l w2_l
@@ -1231,7 +1274,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
   d.emode = E_F32; d.o = w.buf0; d.ldo = a.r; d.perm_per = per;
   d.part = w.part; d.counters = w.counters;
   d.vec_ok = aligned(a.W1, 16) && a.r % 8 == 0;
-  if (!plan_kn(d, MT, target)) return BLR_ERR_UNSUPPORTED;
+  if (!plan_kn(d, MT, target, a.M)) return BLR_ERR_UNSUPPORTED;
   PhaseDesc& e = p.ph[1];
   e.wbits = 16; e.W = a.W2; e.batch = a.b; e.K = a.r; e.N = S;
   e.amode = A_F32; e.a = w.buf0;
@@ -1242,7 +1285,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
   if (a.w2_layout == BLR_W2_RS) {
     e.kind = PH_KN; e.w_bs = (int64_t)a.r * S; e.ldw = S;
     e.vec_ok = aligned(a.W2, 16) && S % 8 == 0;
-    if (!plan_kn(e, MT, target)) return BLR_ERR_UNSUPPORTED;
+    if (!plan_kn(e, MT, target, a.M)) return BLR_ERR_UNSUPPORTED;
   } else {
     e.kind = PH_NK; e.w_bs = (int64_t)S * a.r; e.ldw = a.r;
     e.vec_ok = aligned(a.W2, 16) && a.r % 8 == 0;
