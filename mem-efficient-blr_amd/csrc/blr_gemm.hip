@@ -7,6 +7,9 @@
 // and copied straight in; (k, n)-ordered weights (n contiguous - the layout most of the
 // reference's kernel names use) are transposed in registers on their way into LDS.
 // fp32: plain FMA tiles, used only by the *_fp32 verification names.
+#include <cstdlib>
+#include <mutex>
+#include <set>
 #include "blr_common.h"
 
 namespace blr {
@@ -21,33 +24,41 @@ struct GemmSmem {
 };
 
 // ---- global -> register staging ------------------------------------------------------------
+// Both stagers keep per-thread base pointers computed once (rows / columns outside the problem
+// are clamped to the last valid one - their results are never stored), so that a full k tile is
+// fetched with unconditional 16-byte loads at a uniform offset.  Only the last, partial k tile
+// and operands that are not 16-byte friendly take the guarded element-wise path.
+//
 // K-contiguous operand: tile of ROWS rows x 64 k.  Thread t owns vectors v = t + i*256,
 // row = v / 8, k-vector = v % 8 (8 lanes cover one 128-byte row segment).
 template <typename T, int ROWS>
 struct KcStage {
   static constexpr int NV = ROWS * 8 / 256;
-  typename TypeTraits<T>::vec8 v[NV];
+  using V8 = typename TypeTraits<T>::vec8;
+  V8 v[NV];
+  const T* p[NV];
 
-  __device__ __forceinline__ void load(const T* base, int64_t ld, int row0, int nrows, int k0, int K,
-                                       bool vec_ok, int tid) {
+  __device__ __forceinline__ void init(const T* base, int64_t ld, int row0, int nrows, int tid) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       int vi = tid + i * 256;
       int row = vi >> 3, kv = (vi & 7) * 8;
-      int gr = row0 + row, gk = k0 + kv;
-      typename TypeTraits<T>::vec8 val;
+      p[i] = base + (int64_t)min(row0 + row, nrows - 1) * ld + kv;
+    }
+  }
+  __device__ __forceinline__ void load(int k0, int K, bool vec_ok, int tid) {
+    if (vec_ok && k0 + BK <= K) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) val[e] = (T)0.0f;
-      if (gr < nrows && gk < K) {
-        const T* p = base + (int64_t)gr * ld + gk;
-        if (vec_ok && gk + 8 <= K) {
-          val = ldg16<typename TypeTraits<T>::vec8>(p);
-        } else {
+      for (int i = 0; i < NV; ++i) v[i] = ldg16<V8>(p[i] + k0);
+      return;
+    }
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (gk + e < K) val[e] = p[e];
-        }
-      }
+    for (int i = 0; i < NV; ++i) {
+      int kv = ((tid + i * 256) & 7) * 8;
+      int gk = k0 + kv;
+      V8 val;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) val[e] = (gk + e < K) ? p[i][k0 + e] : (T)0.0f;
       v[i] = val;
     }
   }
@@ -56,7 +67,7 @@ struct KcStage {
     for (int i = 0; i < NV; ++i) {
       int vi = tid + i * 256;
       int row = vi >> 3, kv = (vi & 7) * 8;
-      *reinterpret_cast<typename TypeTraits<T>::vec8*>(&s[row][kv]) = v[i];
+      *reinterpret_cast<V8*>(&s[row][kv]) = v[i];
     }
   }
 };
@@ -68,35 +79,54 @@ struct KcStage {
 template <typename T, int COLS>
 struct KnStage {
   static constexpr int NP = COLS / 128;
-  typename TypeTraits<T>::vec8 v[NP][4];
+  using V8 = typename TypeTraits<T>::vec8;
+  V8 v[NP][4];
+  const T* p[NP];
+  int64_t ld;
+  int nvalid[NP];                           // columns of this thread's vector that exist (0..8)
 
-  __device__ __forceinline__ void load(const T* base, int64_t ld, int col0, int ncols, int k0, int K,
-                                       bool vec_ok, int tid) {
+  __device__ __forceinline__ void init(const T* base, int64_t ld_, int col0, int ncols, int tid, bool vec_ok) {
     int lane = tid & 63, wave = tid >> 6;
     int kq = lane & 15;
+    ld = ld_;
 #pragma unroll
     for (int ps = 0; ps < NP; ++ps) {
       int nv = wave * 4 + (lane >> 4) + ps * 16;
       int gn = col0 + nv * 8;
+      nvalid[ps] = max(0, min(8, ncols - gn));
+      if (vec_ok) gn = min(gn, ncols - 8);   // clamp to the last whole vector (ncols % 8 == 0 here)
+      else gn = min(gn, ncols - 1);
+      p[ps] = base + (int64_t)(kq * 4) * ld + gn;
+    }
+  }
+  __device__ __forceinline__ void load(int k0, int K, bool vec_ok, int tid) {
+    if (vec_ok && k0 + BK <= K) {
+#pragma unroll
+      for (int ps = 0; ps < NP; ++ps)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[ps][i] = ldg16<V8>(p[ps] + (int64_t)(k0 + i) * ld);
+      return;
+    }
+    int kq = tid & 15;
+#pragma unroll
+    for (int ps = 0; ps < NP; ++ps)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         int gk = k0 + kq * 4 + i;
-        typename TypeTraits<T>::vec8 val;
+        V8 val;
 #pragma unroll
         for (int e = 0; e < 8; ++e) val[e] = (T)0.0f;
-        if (gk < K && gn < ncols) {
-          const T* p = base + (int64_t)gk * ld + gn;
-          if (vec_ok && gn + 8 <= ncols) {
-            val = ldg16<typename TypeTraits<T>::vec8>(p);
-          } else {
+        if (gk < K) {
+          const T* q = p[ps] + (int64_t)(k0 + i) * ld;
+          if (vec_ok) val = ldg16<V8>(q);
+          else {
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-              if (gn + e < ncols) val[e] = p[e];
+              if (e < nvalid[ps]) val[e] = q[e];
           }
         }
         v[ps][i] = val;
       }
-    }
   }
   __device__ __forceinline__ void store(T (*s)[LDS_LD], int tid) const {
     int lane = tid & 63, wave = tid >> 6;
@@ -123,11 +153,13 @@ __device__ __forceinline__ int64_t epi_offset(const GemmArgs& g, int bt, int m, 
 }
 
 template <typename T, int BM, int BN, bool B_KN>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int a_vec, int b_vec) {
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int a_vec, int b_vec, int c_vec) {
   constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;    // 32x32 MFMA tiles per wave
   using V8 = typename TypeTraits<T>::vec8;
-  __shared__ GemmSmem<T, BM, BN> sm;
+  using Smem = GemmSmem<T, BM, BN>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  Smem* sm = reinterpret_cast<Smem*>(smem_raw);  // two stages
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -155,21 +187,25 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
   KnStage<T, BN> sb_kn;
 
   const int KT = (g.K + BK - 1) / BK;
-  sa.load(A, g.lda, m0, g.M, 0, g.K, a_vec, tid);
-  if (B_KN) sb_kn.load(B, g.ldb, n0, g.N, 0, g.K, b_vec, tid);
-  else sb_kc.load(B, g.ldb, n0, g.N, 0, g.K, b_vec, tid);
+  sa.init(A, g.lda, m0, g.M, tid);
+  if (B_KN) sb_kn.init(B, g.ldb, n0, g.N, tid, b_vec);
+  else sb_kc.init(B, g.ldb, n0, g.N, tid);
+  sa.load(0, g.K, a_vec, tid);
+  if (B_KN) sb_kn.load(0, g.K, b_vec, tid);
+  else sb_kc.load(0, g.K, b_vec, tid);
+  sa.store(sm[0].a, tid);
+  if (B_KN) sb_kn.store(sm[0].b, tid);
+  else sb_kc.store(sm[0].b, tid);
+  __syncthreads();
 
   for (int kt = 0; kt < KT; ++kt) {
-    __syncthreads();                       // previous tile fully consumed
-    sa.store(sm.a, tid);
-    if (B_KN) sb_kn.store(sm.b, tid);
-    else sb_kc.store(sm.b, tid);
-    __syncthreads();
-    if (kt + 1 < KT) {                     // next tile's loads fly while this one is multiplied
+    Smem& cur = sm[kt & 1];
+    const bool more = kt + 1 < KT;
+    if (more) {                            // next tile's global loads fly while this one is multiplied
       int k0 = (kt + 1) * BK;
-      sa.load(A, g.lda, m0, g.M, k0, g.K, a_vec, tid);
-      if (B_KN) sb_kn.load(B, g.ldb, n0, g.N, k0, g.K, b_vec, tid);
-      else sb_kc.load(B, g.ldb, n0, g.N, k0, g.K, b_vec, tid);
+      sa.load(k0, g.K, a_vec, tid);
+      if (B_KN) sb_kn.load(k0, g.K, b_vec, tid);
+      else sb_kc.load(k0, g.K, b_vec, tid);
     }
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
@@ -177,18 +213,50 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
       V8 af[TM], bf[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        af[i] = *reinterpret_cast<const V8*>(&sm.a[wm * WM + i * 32 + (lane & 31)][kof]);
+        af[i] = *reinterpret_cast<const V8*>(&cur.a[wm * WM + i * 32 + (lane & 31)][kof]);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        bf[j] = *reinterpret_cast<const V8*>(&sm.b[wn * WN + j * 32 + (lane & 31)][kof]);
+        bf[j] = *reinterpret_cast<const V8*>(&cur.b[wn * WN + j * 32 + (lane & 31)][kof]);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = TypeTraits<T>::mfma32(af[i], bf[j], acc[i][j]);
     }
+    if (more) {                            // the other stage is free: nobody reads it until the barrier below
+      Smem& nxt = sm[(kt + 1) & 1];
+      sa.store(nxt.a, tid);
+      if (B_KN) sb_kn.store(nxt.b, tid);
+      else sb_kc.store(nxt.b, tid);
+    }
+    __syncthreads();
   }
 
   // D fragment: element e of lane l is row (e/4)*8 + (l/32)*4 + e%4, column l%32.
+  if (c_vec) {
+    // Stage the tile in LDS as [row][BN + 8] and write 16-byte row segments.
+    constexpr int CLD = BN + 8;
+    T* cs = reinterpret_cast<T*>(smem_raw);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        int col = wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          int row = wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          cs[row * CLD + col] = TypeTraits<T>::from_f32(acc[i][j][e]);
+        }
+      }
+    __syncthreads();
+    constexpr int VPR = BN / 8;                // 16-byte vectors per tile row
+    for (int v = tid; v < BM * VPR; v += 256) {
+      int row = v / VPR, cvec = (v - row * VPR) * 8;
+      int gr = m0 + row, gc = n0 + cvec;
+      if (gr < g.M && gc < g.N)
+        *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -258,22 +326,41 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) 
 template <typename T, int BM, int BN>
 static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
-  // 16-byte vector loads need every row start and every k (or n) offset to be 16-byte aligned.
+  // 16-byte vector accesses need every row start and every k (or n) offset to be 16-byte aligned.
   int a_vec = aligned(g.A, 16) && g.lda % 8 == 0 && g.sA % 8 == 0;
   int b_vec = aligned(g.B, 16) && g.ldb % 8 == 0 && g.sB % 8 == 0;
+  int c_vec = g.epi == EPI_PLAIN && g.cn == 1 && aligned(g.C, 16) && g.ldc % 8 == 0 && g.sC % 8 == 0 && g.N % 8 == 0;
+  size_t lds = 2 * sizeof(GemmSmem<T, BM, BN>);
+  void* fn = g.b_kn ? (void*)gemm_mfma_kernel<T, BM, BN, true> : (void*)gemm_mfma_kernel<T, BM, BN, false>;
+  static std::mutex mu;
+  static std::set<void*> raised;
+  {
+    std::lock_guard<std::mutex> lk(mu);
+    if (lds > 64 * 1024 && !raised.count(fn)) {
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) { set_error("gemm: cannot raise LDS limit: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+      raised.insert(fn);
+    }
+  }
   dim3 grid(tiles_m * tiles_n, g.batch);
-  if (g.b_kn) hipLaunchKernelGGL((gemm_mfma_kernel<T, BM, BN, true>), grid, dim3(256), 0, st, g, tiles_m, tiles_n, a_vec, b_vec);
-  else hipLaunchKernelGGL((gemm_mfma_kernel<T, BM, BN, false>), grid, dim3(256), 0, st, g, tiles_m, tiles_n, a_vec, b_vec);
-  BLR_CHECK_LAUNCH("gemm_mfma");
+  GemmArgs ga = g;
+  void* args[] = {&ga, &tiles_m, &tiles_n, &a_vec, &b_vec, &c_vec};
+  hipError_t e = hipLaunchKernel(fn, grid, dim3(256), args, lds, st);
+  if (e != hipSuccess) { set_error("gemm_mfma: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
 }
 
 template <typename T>
 static int pick_mfma(const GemmArgs& g, hipStream_t st) {
-  // Large problems take the 256x128 tile (more MFMA work per LDS byte); when that would leave
-  // most of the 256 CUs idle, or N is narrow, fall back to 128x128.
-  int64_t big_tiles = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
-  if (g.M >= 256 && big_tiles >= 2 * device_cus()) return launch_mfma<T, 256, 128>(g, st);
+  // Bigger tiles do more MFMA work per LDS byte (the 2x2 wave grid reads 0.5 fragments per MFMA at
+  // 256x256, 0.75 at 256x128, 1 at 128x128) but need enough tiles to fill the 256 CUs.
+  static const int force = [] { const char* e = getenv("BLR_GEMM_TILE"); return e ? atoi(e) : 0; }();
+  const int cus = device_cus() > 0 ? device_cus() : 256;
+  int64_t t256 = cdiv(g.M, 256) * cdiv(g.N, 256) * g.batch;
+  int64_t t128 = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
+  // 256x256 needs 256 accumulator registers per lane and currently spills: only on request (BLR_GEMM_TILE=256).
+  if (force == 256 && t256 > 0) return launch_mfma<T, 256, 256>(g, st);
+  if (force == 128256 || (force == 0 && g.M >= 256 && t128 >= cus)) return launch_mfma<T, 256, 128>(g, st);
   return launch_mfma<T, 128, 128>(g, st);
 }
 
@@ -348,11 +435,73 @@ static void mix_dispatch(dim3 grid, size_t lds, hipStream_t st, const void* Y, c
     hipLaunchKernelGGL((blast_mix_kernel<T, 0>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
 }
 
+// Vector variant for two-byte types, b <= 16, R % 8 == 0: thread = (8 consecutive r, one m); all
+// b vectors Y_j[m, r..r+7] are loaded (16 bytes each) before the b x b x 8 multiply-adds, S comes
+// from an LDS slab [j][i][64] staged once per workgroup and reused for 128 rows of m.
+template <typename T>
+__global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict__ Y, const T* __restrict__ S,
+                                                            T* __restrict__ Z, int M, int b, int R,
+                                                            int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg) {
+  using V8 = typename TypeTraits<T>::vec8;
+  extern __shared__ float s_lds[];
+  T* s_t = reinterpret_cast<T*>(s_lds);      // [b][b][64]  (j, i, r)
+  const int tid = threadIdx.x;
+  const int r0 = blockIdx.x * 64;
+  for (int idx = tid; idx < b * b * 64; idx += 256) {
+    int r = idx & 63, ji = idx >> 6;
+    int j = ji / b, i = ji - j * b;
+    T v = (T)0.0f;
+    if (r0 + r < R) v = S[(int64_t)i * s_si + (int64_t)j * s_sj + (int64_t)(r0 + r) * s_sr];
+    s_t[idx] = v;
+  }
+  __syncthreads();
+  const int rl = tid & 7, ms = tid >> 3;     // 8 r-vectors x 32 m slots
+  const int r = r0 + rl * 8;
+  if (r >= R) return;
+  const int m_begin = blockIdx.y * m_per_wg;
+  const int m_end = min(M, m_begin + m_per_wg);
+  for (int m = m_begin + ms; m < m_end; m += 32) {
+    V8 yv[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if (j < b) yv[j] = ldg16<V8>(&Y[((int64_t)j * M + m) * R + r]);
+    for (int i = 0; i < b; ++i) {
+      float acc[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        if (j < b) {
+          V8 sv = *reinterpret_cast<const V8*>(&s_t[(j * b + i) * 64 + rl * 8]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] = fmaf(TypeTraits<T>::to_f32(sv[e]), TypeTraits<T>::to_f32(yv[j][e]), acc[e]);
+        }
+      }
+      V8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = TypeTraits<T>::from_f32(acc[e]);
+      *reinterpret_cast<V8*>(&Z[((int64_t)i * M + m) * R + r]) = o;
+    }
+  }
+}
+
 int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
                      int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st) {
+  int r_chunks = (int)cdiv(R, 64);
+  if (dtype != BLR_F32 && b <= 16 && R % 8 == 0 && aligned(Y, 16) && aligned(Z, 16)) {
+    size_t lds = (size_t)b * b * 64 * 2;
+    int m_per_wg = 128;
+    while ((int64_t)r_chunks * cdiv(M, m_per_wg) < 512 && m_per_wg > 32) m_per_wg /= 2;
+    dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
+    if (dtype == BLR_F16)
+      hipLaunchKernelGGL(blast_mix_vec_kernel<f16>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+    else
+      hipLaunchKernelGGL(blast_mix_vec_kernel<bf16>, grid, dim3(256), lds, st, (const bf16*)Y, (const bf16*)S, (bf16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+    BLR_CHECK_LAUNCH("blast_mix_vec");
+    return BLR_OK;
+  }
   size_t lds = (size_t)b * b * 64 * sizeof(float);
   if (lds > 64 * 1024) { set_error("blast mix: b=%d too large for the LDS slab", b); return BLR_ERR_UNSUPPORTED; }
-  int r_chunks = (int)cdiv(R, 64);
   int m_per_wg = 64;
   while ((int64_t)r_chunks * cdiv(M, m_per_wg) < 1024 && m_per_wg > 4) m_per_wg /= 2;
   dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
