@@ -87,7 +87,7 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
  * and fp16 per-output-channel scales: U codes (b, q, r[/2]) + u_scales (b, q); V codes
  * (b, p, r[/2]) + v_scales (b, r); S (r, i, j) of dtype.  Served behind the name
  * triton_blast_bmm_int8_fp16 (reference triton_funcs/blast_sym_quant_kernels.py:558-580).
- * M <= 16, r % 32 == 0.                                                                      */
+  * r % 32 == 0.  M <= 16 streams the codes; larger M expands them to dtype in the workspace first.                                                                     */
 size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits);
 int blr_blast_q_fwd(const void* x, int64_t ldx,
                     const void* u_codes, const void* u_scales,

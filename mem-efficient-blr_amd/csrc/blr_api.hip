@@ -109,6 +109,26 @@ __global__ __launch_bounds__(256) void quant_cols_kernel(const T* __restrict__ w
   }
 }
 
+// codes (rows, cols) -> T; scale index = (row / rows_per_scale_block) * cols + col when per_col, else row.
+template <typename T>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ codes, const f16* __restrict__ scales,
+                                                      T* __restrict__ out, int64_t rows, int64_t cols, int bits,
+                                                      int per_col, int64_t rows_per_block) {
+  const int64_t total = rows * cols;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    const int64_t row = idx / cols, col = idx - row * cols;
+    int code;
+    if (bits == 8) code = reinterpret_cast<const int8_t*>(codes)[idx];
+    else {
+      uint8_t byte = codes[idx >> 1];
+      int nib = (idx & 1) ? (byte >> 4) : (byte & 0xF);
+      code = nib > 7 ? nib - 16 : nib;
+    }
+    const float sc = (float)scales[per_col ? (row / rows_per_block) * cols + col : row];
+    out[idx] = TypeTraits<T>::from_f32((float)code * sc);
+  }
+}
+
 template <typename T>
 static int quantize_t(const void* w, int64_t outer, int64_t reduce, int64_t inner, int bits, void* codes, void* scales, hipStream_t st) {
   if (inner == 1) {
@@ -218,7 +238,9 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
 // ---- quantized BLAST -----------------------------------------------------------------------------
 size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits) {
   if (M <= 0 || b <= 0 || r <= 0) return 0;
-  return stream_blast_workspace(M, in_f, out_f, b, r, bits);
+  if (M <= 16) return stream_blast_workspace(M, in_f, out_f, b, r, bits);
+  // larger M: factors are expanded to two-byte values once per call, then the tiled kernels run
+  return align_up((size_t)r * out_f * 2, 256) + align_up((size_t)r * in_f * 2, 256) + 2 * align_up((size_t)b * M * r * 2, 256);
 }
 
 int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void* u_scales,
@@ -230,16 +252,35 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   if (dtype != BLR_F16 && dtype != BLR_BF16) { set_error("blast_q: dtype must be f16 or bf16"); return BLR_ERR_UNSUPPORTED; }
   int rc = check_blast_shape("blast_q", M, in_f, out_f, b, r);
   if (rc) return rc;
-  if (M > 16) { set_error("blast_q: M=%d > 16 not served by the streaming kernel", M); return BLR_ERR_UNSUPPORTED; }
   if (r % 32) { set_error("blast_q: r=%d must be a multiple of 32", r); return BLR_ERR_BAD_SHAPE; }
   if (ldx < in_f || ldo < out_f) { set_error("blast_q: leading dimension too small"); return BLR_ERR_BAD_ARG; }
   if (!aligned(u_codes, 16) || !aligned(v_codes, 16)) { set_error("blast_q: code buffers must be 16-byte aligned"); return BLR_ERR_BAD_ARG; }
+  hipStream_t st = (hipStream_t)stream;
+  if (M > 16) {
+    if (algo == BLR_ALGO_STREAM || algo == BLR_ALGO_STREAM_SPLIT) { set_error("blast_q: M=%d > 16 not served by the streaming kernel", M); return BLR_ERR_UNSUPPORTED; }
+    size_t need = blr_blast_q_workspace_bytes(M, in_f, out_f, b, r, bits);
+    if (!ws || ws_bytes < need) { set_error("blast_q: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
+    char* wp = reinterpret_cast<char*>(ws);
+    void* Ud = wp; wp += align_up((size_t)r * out_f * 2, 256);
+    void* Vd = wp; wp += align_up((size_t)r * in_f * 2, 256);
+    const int64_t urows = out_f, vrows = in_f;
+    if (dtype == BLR_F16) {
+      hipLaunchKernelGGL(dequant_kernel<f16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)u_codes, (const f16*)u_scales, (f16*)Ud, urows, (int64_t)r, bits, 0, (int64_t)1);
+      hipLaunchKernelGGL(dequant_kernel<f16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)v_codes, (const f16*)v_scales, (f16*)Vd, vrows, (int64_t)r, bits, 1, (int64_t)(in_f / b));
+    } else {
+      hipLaunchKernelGGL(dequant_kernel<bf16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)u_codes, (const f16*)u_scales, (bf16*)Ud, urows, (int64_t)r, bits, 0, (int64_t)1);
+      hipLaunchKernelGGL(dequant_kernel<bf16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)v_codes, (const f16*)v_scales, (bf16*)Vd, vrows, (int64_t)r, bits, 1, (int64_t)(in_f / b));
+    }
+    BLR_CHECK_LAUNCH("dequant");
+    return blr_blast_fwd(x, ldx, Ud, Vd, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, BLR_U_QR, BLR_S_RIJ,
+                         BLR_ALGO_TILED, wp, ws_bytes - (size_t)(wp - reinterpret_cast<char*>(ws)), stream);
+  }
   StreamBlastArgs s = {};
   s.x = x; s.ldx = ldx; s.U = u_codes; s.V = v_codes; s.S = S; s.u_scales = u_scales; s.v_scales = v_scales;
   s.out = out; s.ldo = ldo; s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
   s.dtype = dtype; s.u_layout = BLR_U_QR; s.s_layout = BLR_S_RIJ; s.wbits = bits;
   s.ws = ws; s.ws_bytes = ws_bytes; s.split = (algo == BLR_ALGO_STREAM_SPLIT);
-  return stream_blast_launch(s, (hipStream_t)stream);
+  return stream_blast_launch(s, st);
 }
 
 int blr_quantize_sym(const void* w, int dtype, int64_t outer, int64_t reduce, int64_t inner,

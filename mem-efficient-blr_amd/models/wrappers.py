@@ -1,0 +1,147 @@
+"""nn.Module wrappers that own structured factors in the layout their forward function expects.
+
+Counterparts of the reference's models/wrappers.py:5-181.  The forward function is resolved from
+a dotted path string; the *name* of that function decides parameter layout and call convention,
+exactly as in the reference:
+  "triton" in name -> kernel layouts, function returns the output tensor;
+  "torch"  in name -> baseline layouts, function returns a tuple whose first item is the output;
+  BLAST   "bmm" in name  -> U (b, q, r), S (r, b, b), else U (b, r, q), S (b, b, r); V (b, p, r)
+  Monarch "left" in name -> w2 (b, r, s), else (b, s, r); w1 (b, p, r)
+The bias is added as `out += bias.to(x.dtype)` (reference wrappers.py:176-177).
+Factors are drawn with std 1/sqrt(fan-in of the factor) instead of the reference's std 1, so that
+fp16 activations stay in range at the ranks the networks use.
+"""
+import importlib
+import math
+
+import torch
+import torch.nn as nn
+
+
+def resolve(func_path):
+    module_name, func_name = func_path.rsplit(".", 1)
+    return func_name, getattr(importlib.import_module(module_name), func_name)
+
+
+class _StructuredLinear(nn.Module):
+    def __init__(self, in_features, out_features, func_path, device, dtype, bias, is_compiled):
+        super().__init__()
+        self.device, self.dtype = device, dtype
+        self.in_features, self.out_features = in_features, out_features
+        self.func_name, self.func = resolve(func_path)
+        self.is_compiled = is_compiled
+        if is_compiled:
+            self.func = torch.compile(self.func)
+        self.kind = "triton" if "triton" in self.func_name else "torch"
+        if bias:
+            self.bias = nn.Parameter(torch.randn(out_features, device=device, dtype=dtype))
+        else:
+            self.register_parameter("bias", None)
+
+    def _param(self, shape, fan_in):
+        return nn.Parameter(torch.randn(shape, device=self.device, dtype=torch.float32).mul_(1.0 / math.sqrt(fan_in)).to(self.dtype))
+
+    def _finish(self, out):
+        if self.kind == "torch" and isinstance(out, tuple):
+            out = out[0]
+        if self.bias is not None:
+            out += self.bias.to(out.dtype)
+        return out
+
+
+class BlastLinear(_StructuredLinear):
+    def __init__(self, in_features, out_features, b, rank, func_path, device, dtype, bias=True, is_compiled=False):
+        super().__init__(in_features, out_features, func_path, device, dtype, bias, is_compiled)
+        assert in_features % b == 0 and out_features % b == 0
+        self.b, self.rank = b, rank
+        p, q = in_features // b, out_features // b
+        if self.kind == "triton":
+            bmm = "bmm" in self.func_name
+            self.U = self._param((b, q, rank) if bmm else (b, rank, q), rank)
+            self.V = self._param((b, p, rank), rank)
+            self.S = self._param((rank, b, b) if bmm else (b, b, rank), 1)
+        else:
+            self.U = self._param((b, q, rank), rank)
+            self.V = self._param((b, rank, p), rank)
+            self.S = self._param((b, b, rank), 1)
+
+    def forward(self, x):
+        return self._finish(self.func(x, self.U, self.V, self.S))
+
+    def extra_repr(self):
+        return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
+                f"rank={self.rank}, b={self.b}, func={self.func_name}")
+
+
+class QuantBlastLinear(BlastLinear):
+    """BLAST with int8 / packed-int4 factors (method "blast_sym_quant"): quantized once at construction."""
+
+    def __init__(self, in_features, out_features, b, rank, func_path, device, dtype, bias=True, is_compiled=False, bits=8):
+        super().__init__(in_features, out_features, b, rank, func_path, device, dtype, bias, is_compiled)
+        from triton_funcs.blast_sym_quant_kernels import quantize_blast_factors
+        assert "bmm" in self.func_name, "the quantized kernel takes the bmm layouts"
+        self.bits = bits
+        self.Uq, self.Vq = quantize_blast_factors(self.U.detach().float(), self.V.detach().float(), bits)
+        del self.U, self.V
+
+    def forward(self, x):
+        return self._finish(self.func(x, self.Uq, self.Vq, self.S))
+
+
+class MonarchLinear(_StructuredLinear):
+    def __init__(self, in_features, out_features, b, rank, func_path, device, dtype, bias=True, is_compiled=False):
+        super().__init__(in_features, out_features, func_path, device, dtype, bias, is_compiled)
+        assert in_features % b == 0 and out_features % b == 0
+        assert rank % b == 0
+        self.b, self.rank = b, rank
+        p, s = in_features // b, out_features // b
+        if self.kind == "triton":
+            self.w1_bfly = self._param((b, p, rank), p)
+            self.w2_bfly = self._param((b, rank, s) if "left" in self.func_name else (b, s, rank), rank)
+        else:
+            self.w1_bfly = self._param((b, rank, p), p)
+            self.w2_bfly = self._param((b, s, rank), rank)
+
+    def forward(self, x):
+        return self._finish(self.func(x, self.w1_bfly, self.w2_bfly))
+
+    def extra_repr(self):
+        return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
+                f"rank={self.rank}, b={self.b}, func={self.func_name}")
+
+
+class LowRankLinear(_StructuredLinear):
+    def __init__(self, in_features, out_features, rank, func_path, device, dtype, bias=True, is_compiled=False):
+        super().__init__(in_features, out_features, func_path, device, dtype, bias, is_compiled)
+        self.rank = rank
+        if self.kind == "triton":
+            self.V = self._param((in_features, rank), rank)
+            self.U = self._param((rank, out_features), rank)
+        else:
+            self.V = self._param((rank, in_features), rank)
+            self.U = self._param((out_features, rank), rank)
+
+    def forward(self, x):
+        out = self.func(x, self.V, self.U)
+        if self.kind == "triton":                      # the kernel returns (N, out_f): restore the leading dims
+            out = out.reshape(*x.shape[:-1], self.out_features)
+        return self._finish(out)
+
+    def extra_repr(self):
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, rank={self.rank}, func={self.func_name}"
+
+
+class DenseLinear(_StructuredLinear):
+    def __init__(self, in_features, out_features, func_path, device, dtype, bias=True, is_compiled=False):
+        super().__init__(in_features, out_features, func_path, device, dtype, bias, is_compiled)
+        shape = (in_features, out_features) if self.kind == "triton" else (out_features, in_features)
+        self.W = self._param(shape, in_features)
+
+    def forward(self, x):
+        out = self.func(x, self.W)
+        if self.kind == "triton":
+            out = out.reshape(*x.shape[:-1], self.out_features)
+        return self._finish(out)
+
+    def extra_repr(self):
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, func={self.func_name}"

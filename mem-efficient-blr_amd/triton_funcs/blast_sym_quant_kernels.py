@@ -90,7 +90,7 @@ def triton_blast_bmm_int8_fp16(x, U, V, S, config=(None, None, None)):
     M, in_f, out_f = x2.shape[0], b1 * p, b2 * q
     out = torch.empty((M, out_f), device=x.device, dtype=x.dtype)
     lib = L.lib()
-    ws = L.workspace(x.device, lib.blr_blast_q_workspace_bytes(M, in_f, out_f, b1, r, U.bits), L.ALGO_STREAM)
+    ws = L.workspace(x.device, lib.blr_blast_q_workspace_bytes(M, in_f, out_f, b1, r, U.bits), L.ALGO_STREAM if M <= 16 else L.ALGO_TILED)
     rc = lib.blr_blast_q_fwd(x2.data_ptr(), x2.stride(0), U.codes.data_ptr(), U.scales.data_ptr(),
                              V.codes.data_ptr(), V.scales.data_ptr(), S.data_ptr(), out.data_ptr(), out.stride(0),
                              M, in_f, out_f, b1, r, dt, U.bits, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))

@@ -1,0 +1,82 @@
+"""GPU: the harness dispatches every configured function name to the HIP kernels and they verify."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import blr_oracle as O
+from gpu_util import assert_close, say
+
+pytestmark = pytest.mark.gpu
+PKG = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "mem-efficient-blr_amd")
+
+
+@pytest.mark.parametrize("cfg", ["gpt2s.mlp_c_fc", "dit_xl.fc1"])
+def test_layer_verify_all_match(cfg, tmp_path, monkeypatch):
+    from layer import Layer
+    from utils import VerificationStatus
+    monkeypatch.chdir(tmp_path)
+    l = Layer(os.path.join(PKG, "configs", "layers", cfg + ".yaml"))
+    l.num_seq = min(l.num_seq, 256)
+    say(f"[case] Layer.verify {cfg}")
+    l.verify("all")
+    for fam in ("blast", "monarch", "low_rank", "dense"):
+        assert l.status[fam] and all(s == VerificationStatus.MATCH for s in l.status[fam]), (fam, l.status[fam])
+    say(f"[case] Layer.benchmark {cfg}")
+    l.benchmark("all")
+    ms = l.measured_ms()
+    assert all(t > 0 for t in ms.values()), ms
+    l.summary()
+    assert os.path.exists(f"output/{l.network_name}/{l.layer_name}/triton_blast_full_fp16_best_config.pkl")
+    assert os.path.exists(f"output/{l.network_name}/{l.layer_name}/triton_blast_bmm_xv_fp16_best_config.pkl")
+
+
+@pytest.mark.parametrize("M", [1, 40])
+def test_wrappers_on_gpu_vs_oracle(M):
+    from models.wrappers import BlastLinear, MonarchLinear, LowRankLinear, DenseLinear, QuantBlastLinear
+    torch.manual_seed(0)
+    kw = dict(device="cuda", dtype=torch.float16)
+    x = torch.randn(1, M, 256, **kw)
+    f64 = lambda t: t.detach().double().cpu().numpy()
+    say(f"[case] wrappers M={M}")
+    m = BlastLinear(256, 384, b=4, rank=64, func_path="triton_funcs.blast_kernels.triton_blast_full_fp16", **kw)
+    Ut, Vt, St = f64(m.U).transpose(0, 2, 1), f64(m.V).transpose(0, 2, 1), f64(m.S).transpose(1, 0, 2)
+    assert_close(m(x), O.blast_forward(f64(x), Ut, Vt, St)[0] + f64(m.bias), torch.float16, "BlastLinear")
+    m = MonarchLinear(256, 384, b=4, rank=64, func_path="triton_funcs.monarch_kernels.triton_monarch_right_left_fp16", bias=False, **kw)
+    out = m(x)
+    assert out.shape == (1, M, 384) and torch.isfinite(out).all()
+    m = LowRankLinear(256, 384, rank=64, func_path="triton_funcs.low_rank_kernels.triton_low_rank_fp16", **kw)
+    assert_close(m(x), O.low_rank_forward(f64(x), f64(m.V).T, f64(m.U).T)[0] + f64(m.bias), torch.float16, "LowRankLinear")
+    m = DenseLinear(256, 384, func_path="triton_funcs.dense_kernels.triton_dense_fp16", **kw)
+    assert_close(m(x), O.dense_forward(f64(x), f64(m.W).T) + f64(m.bias), torch.float16, "DenseLinear")
+    if M <= 16:
+        m = QuantBlastLinear(256, 384, b=4, rank=64, func_path="triton_funcs.blast_sym_quant_kernels.triton_blast_bmm_int8_fp16", **kw)
+        out = m(x)
+        assert out.shape == (1, M, 384) and torch.isfinite(out).all()
+
+
+def test_dit_small_blast_matches_its_dense_assembly():
+    """2-block DiT with BLAST kernels vs the same model with each BlastLinear replaced by its dense matrix."""
+    from models.dit_xl import CustomDiT
+    torch.manual_seed(0)
+    cfg = {k: {"rank": r, "b": 16, "func": "triton_funcs.blast_kernels.triton_blast_bmm_fp16"}
+           for k, r in (("attn.qkv", 288), ("attn.proj", 288), ("mlp.fc1", 576), ("mlp.fc2", 576))}
+    say("[case] DiT depth 2, BLAST")
+    net = CustomDiT(layer_configs=cfg, method="blast", depth=2)
+    assert net.replaced == 8
+    x = torch.randn(4, 4, 32, 32, device="cuda", dtype=torch.float16)
+    t = torch.randint(0, 1000, (4,), device="cuda"); y = torch.randint(0, 1000, (4,), device="cuda")
+    with torch.no_grad():
+        out = net(x, t, y).float()
+        for blk in net.model.blocks:
+            for parent, name in ((blk.attn, "qkv"), (blk.attn, "proj"), (blk.mlp, "fc1"), (blk.mlp, "fc2")):
+                bl = getattr(parent, name)
+                S = bl.S.detach().double().cpu().numpy().transpose(1, 2, 0)            # (r,i,j) -> (i,j,r)
+                W = O.blast_dense_weight(bl.U.detach().double().cpu().numpy(), bl.V.detach().double().cpu().numpy().transpose(0, 2, 1), S)
+                lin = torch.nn.Linear(bl.in_features, bl.out_features).cuda().half()
+                lin.weight.copy_(torch.from_numpy(W)); lin.bias.copy_(bl.bias)
+                setattr(parent, name, lin)
+        ref = net(x, t, y).float()
+    assert out.shape == (4, 8, 32, 32)
+    assert (out - ref).abs().max() <= 2e-2 * ref.abs().max()

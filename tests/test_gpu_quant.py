@@ -44,7 +44,7 @@ def test_quantizer_half_inputs_and_ties():
     np.testing.assert_array_equal(c2.cpu().numpy(), r2)
 
 
-QSHAPES = [(2, 8, 8, 32, 1), (4, 16, 24, 64, 3), (16, 32, 40, 96, 16), (16, 256, 256, 512, 4)]
+QSHAPES = [(2, 8, 8, 32, 1), (4, 16, 24, 64, 3), (16, 32, 40, 96, 16), (16, 256, 256, 512, 4), (4, 32, 40, 96, 40), (16, 72, 288, 288, 300)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -67,7 +67,7 @@ def test_blast_q_vs_oracle_on_dequantized(shape, bits, dtype):
     np.testing.assert_array_equal(Uq.scales.cpu().numpy(), us); np.testing.assert_array_equal(Vq.scales.cpu().numpy(), vs)
     fn = Q.triton_blast_bmm_int8_fp16 if bits == 8 else Q.triton_blast_bmm_int4_fp16
     ref = O.blast_q_forward(rounded(x, dtype), uc, us, vc, vs, rounded(S, dtype))
-    for algo in (1, 4):
+    for algo in ((1, 4) if M <= 16 else (0,)):          # M > 16: codes are expanded, then the tiled kernels run
         out = fn(dev(x, dtype), Uq, Vq, dev(S, dtype), {"algo": algo})
         assert tuple(out.shape) == (1, M, b * q)
         assert_close(out, ref, dtype, f"blast_q bits={bits} algo={algo}")
