@@ -236,6 +236,25 @@ def main():
                     fl = 2 * m * r * (i_f + o_f + B * B)
                     row(f"blast_int{bits}/{lname}/M{m}", measure(lambda: mk_blast_q(m, i_f, o_f, r, bits), by), by, fl, m)
 
+    # ---- DiT-XL/2 end to end (BASELINE configs[4]): 16 latents [4,32,32], every qkv/proj/fc1/fc2 linear replaced ----
+    dit = None
+    if not args.no_table:
+        try:
+            import yaml
+            from models import dit_xl
+            ncfg = yaml.safe_load(open(os.path.join(PKG, "configs", "networks", "dit_xl.yaml")))
+            dit = {"batch": 16, "tokens_per_image": 256, "dtype": "f16"}
+            for method in ("blast", "low_rank", "dense"):
+                lc = {k: {"rank": v.get("rank"), "b": v.get("b"), "func": v["triton"]["func"]} for k, v in ncfg[method].items()}
+                ms = dit_xl.benchmark(method, "triton", lc, 256, 10, dev, f16, batch=16)
+                dit[f"{method}_img_per_s"] = round(16 / (ms * 1e-3), 1)
+                dit[f"{method}_ms"] = round(ms, 3)
+            ms = dit_xl.benchmark(None, None, None, 256, 10, dev, f16, batch=16)        # stock nn.Linear (hipBLASLt) for scale
+            dit["nn_linear_img_per_s"] = round(16 / (ms * 1e-3), 1)
+            torch.cuda.empty_cache()
+        except Exception as e:                       # the headline must still be printed
+            dit = {"error": str(e)}
+
     # ---- CPU baseline: the oracle's torch port of the same step, fp32, all host cores -----------------
     cpu = None
     if not args.no_cpu:
@@ -272,7 +291,7 @@ def main():
                                "triton_blast_full_fp16 layouts, HIP-graph replay, weight copies rotated past the Infinity Cache",
                    "weight_copies": ncopies, "algorithmic_bytes_per_step": step_bytes,
                    "pct_hbm_step": round(100 * step_bytes / (ms_per_step * 1e-3) / HBM_PEAK, 1)},
-        "roofline": roofline, "cpu_baseline": cpu, "layers": table,
+        "roofline": roofline, "cpu_baseline": cpu, "layers": table, "dit_xl": dit,
     }
     print(json.dumps(result))
 
