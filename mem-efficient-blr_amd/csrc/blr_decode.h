@@ -1,0 +1,16 @@
+// Two-stage BLAST decode kernel (blr_decode.hip), called from the streaming engine's BLAST entry.
+#pragma once
+#include "blr_common.h"
+
+namespace blr {
+
+// Bytes of the fixed-place workspace block that holds the tagged values exchanged by workgroups.
+size_t decode2_region_bytes();
+// Whether the call can be served by the two-stage decode kernel at all (layout, dtype, M).
+bool decode2_applicable(const StreamBlastArgs& a);
+// Returns BLR_OK, a negative blr_status, or 1 when the shape does not fit the kernel's tiling
+// (the caller then uses the phase engine).
+int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
+                         unsigned* err_word, hipStream_t st);
+
+}  // namespace blr

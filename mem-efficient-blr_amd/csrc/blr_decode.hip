@@ -1,0 +1,629 @@
+// Two-stage BLAST decode kernel for a handful of token rows (M <= 4), U (b, r, q) / V (b, p, r).
+//
+// The whole call is one short dependency chain, so the kernel is built around latency rather
+// than around phases:
+//   * every workgroup that owns a slab of U starts by asking for (up to) all of it: up to 32
+//     16-byte loads per lane go out before anything else is waited for, so HBM streams U while
+//     stage 1 and the hand-over of its result are still in progress;
+//   * there is no grid barrier.  Values that cross workgroups (stage-1 results y, split-k
+//     partial outputs) are stored as 8-byte {fp32 bits, epoch} pairs with device-scope stores;
+//     a consumer simply re-reads a pair until its tag equals the epoch of this call.  One store
+//     and one load make up a hand-over, instead of store - wait - count - poll - load;
+//   * the rank-space mix  z_i = sum_j S_ij * y_j  is a role of its own: a few of the first
+//     workgroups each take a handful of r, fetch the tagged y of every j once, and publish z as
+//     tagged pairs for the stage-2 slabs.
+// The epoch lives in the workspace.  Every workgroup reads it when it starts and then checks
+// in; the last one to check in advances it for the next call, which is safe because by then
+// every workgroup of this call holds its own copy.  Tag 0 is never used, so a zero-filled
+// workspace holds no valid pair.  Calls that share a workspace must be ordered on one stream.
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include "blr_common.h"
+#include "blr_decode.h"
+
+namespace blr {
+
+namespace {
+// 16-byte loads of the U slab held in registers per lane (fewer when the accumulators need the room)
+constexpr int d2_pf(int MT) { return MT <= 1 ? 32 : (MT <= 2 ? 24 : 16); }
+constexpr int D2_UNR = 8;             // loads in flight per lane while streaming the rest of a slab
+constexpr int d2_unr1(int MT) { return MT <= 2 ? 16 : 8; }   // loads in flight per lane in stage 1
+constexpr int D2_SHARDS = 16;         // check-in counters, 256 bytes apart
+constexpr int D2_AS = 4096;           // fp32 activations staged in LDS (MT * k-chunk <= this)
+constexpr int D2_NC_MAX = 512;
+constexpr unsigned D2_SPIN_LIMIT = 4000000u;
+}  // namespace
+
+#ifdef BLR_TRACE
+__device__ unsigned long long g_trace2[1024 * 16];
+#define TR2(i) do { if (threadIdx.x == 0 && blockIdx.x < 1024) g_trace2[blockIdx.x * 16 + (i)] = wall_clock64(); } while (0)
+#else
+#define TR2(i) do {} while (0)
+#endif
+
+struct Decode2Params {
+  const void* x; int64_t ldx;
+  const void* V; const void* U; const void* S;
+  void* out; int64_t ldo;
+  int M, b, P, R, Q;
+  int64_t s_si, s_sj, s_sr;
+  int lpr1_log2, nch1, ks1, kc1, items1;
+  int lpr2_log2, nch2, ks2, kc2, items2, pfn;
+  int itemsM, rch_log2, pf_wait;
+  unsigned long long* ypart;           // [ks1][b][M][R] tagged
+  unsigned long long* zt;              // [b][M][R] tagged
+  unsigned long long* opart;           // [ks2 - 1][b][M][Q] tagged
+  unsigned* epoch_word; unsigned* arrive_word; unsigned* err_word;
+};
+
+__device__ __forceinline__ unsigned long long ld_tag(const unsigned long long* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_tag(unsigned long long* p, float v, unsigned epoch) {
+  __hip_atomic_store(p, ((unsigned long long)epoch << 32) | (unsigned long long)__float_as_uint(v),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T>
+__device__ __forceinline__ void cvt8(const u32x4& r, float (&w)[8]) {
+  typename TypeTraits<T>::vec8 v = __builtin_bit_cast(typename TypeTraits<T>::vec8, r);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) w[e] = TypeTraits<T>::to_f32(v[e]);
+}
+__device__ __forceinline__ u32x4 ldw16(const void* W, int64_t eoff) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(W) + eoff));
+}
+
+// Sum of the row slots of a wave, then of the four waves; thread `col` < NC ends up with the
+// total of column `col` for each of the MT rows (returned through `tot`, valid for tid < NC).
+template <int MT>
+__device__ __forceinline__ void wg_reduce(float (&acc)[MT][8], int lpr, int cv, float* red, int NC, float (&tot)[MT][2]) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int o = lpr; o < 64; o <<= 1) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[m][e] += __shfl_xor(acc[m][e], o, 64);
+  }
+  __syncthreads();
+  if (lane < lpr) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) red[(wave * MT + m) * D2_NC_MAX + cv * 8 + e] = acc[m][e];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int col = tid + h * 256;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      float v = 0.0f;
+      if (col < NC)
+        v = red[(0 * MT + m) * D2_NC_MAX + col] + red[(1 * MT + m) * D2_NC_MAX + col] +
+            red[(2 * MT + m) * D2_NC_MAX + col] + red[(3 * MT + m) * D2_NC_MAX + col];
+      tot[m][h] = v;
+    }
+  }
+}
+
+// Workgroup 0, at its end: wait until every workgroup of the launch has checked in (each does so
+// once it holds its copy of the epoch), then clear the counters and publish the epoch of this call,
+// from which the next call derives its own.
+__device__ __forceinline__ void finish_epoch(const Decode2Params& p, unsigned epoch, int G) {
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    unsigned spins = 0;
+    while (true) {
+      unsigned v = (lane < D2_SHARDS) ? __hip_atomic_load(&p.arrive_word[lane * 64], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+#pragma unroll
+      for (int o = 1; o < D2_SHARDS; o <<= 1) v += __shfl_xor(v, o, 64);
+      if (__shfl(v, 0, 64) == (unsigned)G) break;
+      if (++spins > D2_SPIN_LIMIT) {
+        if (lane == 0) __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (lane < D2_SHARDS) __hip_atomic_store(&p.arrive_word[lane * 64], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(p.epoch_word, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <typename T, int MT>
+__global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
+  constexpr int D2_PF = d2_pf(MT);
+  constexpr int D2_UNR1 = d2_unr1(MT);
+  __shared__ float a_s[D2_AS];
+  __shared__ float red[4 * MT * D2_NC_MAX];
+  constexpr int KLD = D2_AS / MT;
+  const int tid = threadIdx.x;
+  const int w = blockIdx.x, G = gridDim.x;
+  const int M = p.M;
+
+  TR2(0);
+  // ---- epoch of this call ------------------------------------------------------------------
+  unsigned epoch = __hip_atomic_load(p.epoch_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  if (epoch == 0u) epoch = 1u;
+
+  // ---- stage-2 slab of this workgroup --------------------------------------------------------
+  const int item2 = G - 1 - w;
+  const bool has2 = item2 < p.items2;
+  const int lpr2 = 1 << p.lpr2_log2, rpp2 = 256 >> p.lpr2_log2;
+  const int cv2 = tid & (lpr2 - 1), rs2 = tid >> p.lpr2_log2;
+  const int nc2 = has2 ? item2 % p.nch2 : 0;
+  const int t2 = has2 ? item2 / p.nch2 : 0;
+  const int i2 = t2 % p.b, ksi2 = t2 / p.b;
+  const int k0_2 = ksi2 * p.kc2;
+  const int kcur2 = min(p.kc2, p.R - k0_2);
+  const int NC2 = lpr2 * 8;
+  const int n0_2 = nc2 * NC2;
+  const int n2 = n0_2 + cv2 * 8;
+  const bool col_ok2 = n2 < p.Q;
+  const int64_t wbase2 = ((int64_t)i2 * p.R + k0_2) * p.Q + (col_ok2 ? n2 : 0);
+
+  u32x4 pf[D2_PF];                                   // only slots below pfn are ever read after the prefetch
+  auto issue_prefetch = [&]() {
+#pragma unroll
+    for (int u = 0; u < D2_PF; ++u) {
+      if (u < p.pfn) pf[u] = ldw16(p.U, wbase2 + (int64_t)min(rs2 + u * rpp2, kcur2 - 1) * p.Q);
+    }
+  };
+
+  // Mix role (the first workgroups): its S values depend on nothing, so they are asked for first.
+  // S(i = g, j = u, r) for this thread's (g, r); indices are clamped so that every load is legal.
+  float sv[16];
+  if (w < p.itemsM) {
+    const int g = min(tid >> p.rch_log2, p.b - 1);
+    const int r = min(w * (1 << p.rch_log2) + (tid & ((1 << p.rch_log2) - 1)), p.R - 1);
+    const T* Sp = reinterpret_cast<const T*>(p.S);
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      sv[u] = TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]);
+  }
+
+  // Check-in: once the epoch has arrived this workgroup counts itself (no value comes back, so nothing
+  // waits on it).  Workgroup 0 advances the epoch word at its very end, after seeing every check-in.
+  auto check_in = [&]() {
+    if (tid == 0) {
+      asm volatile("" ::"v"(epoch) : "memory");
+      (void)__hip_atomic_fetch_add(&p.arrive_word[(w % D2_SHARDS) * 64], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+
+  // ---- stage 1: y[ks][j][m][n] = sum_k x[m, j P + k] V_j[k, n] over this workgroup's k-slice ----
+  if (w < p.items1) {
+    const int lpr1 = 1 << p.lpr1_log2, rpp1 = 256 >> p.lpr1_log2;
+    const int cv1 = tid & (lpr1 - 1), rs1 = tid >> p.lpr1_log2;
+    const int nc1 = w % p.nch1;
+    const int t1 = w / p.nch1;
+    const int j = t1 % p.b, ks = t1 / p.b;
+    const int k0 = ks * p.kc1, kc = min(p.kc1, p.P - k0);
+    const int NC1 = lpr1 * 8;
+    const int n0 = nc1 * NC1, n = n0 + cv1 * 8;
+    const bool col_ok = n < p.R;
+    const int64_t wbase = ((int64_t)j * p.P + k0) * p.R + (col_ok ? n : 0);
+
+    // The registers that will hold the slab of U serve as the load buffer of stage 1 first.  Batches
+    // are always full: rows past the end are clamped to the last one and meet a zero activation.
+    const int nbatch = ((kc + rpp1 - 1) / rpp1 + D2_UNR1 - 1) / D2_UNR1;
+#pragma unroll
+    for (int u = 0; u < D2_UNR1; ++u) pf[u] = ldw16(p.V, wbase + (int64_t)min(rs1 + u * rpp1, kc - 1) * p.R);
+    const T* xp = reinterpret_cast<const T*>(p.x);
+    for (int idx = tid; idx < MT * kc; idx += 256) {
+      const int m = idx / kc, ka = idx - m * kc;
+      a_s[m * KLD + ka] = (m < M) ? TypeTraits<T>::to_f32(xp[(int64_t)m * p.ldx + (int64_t)j * p.P + k0 + ka]) : 0.0f;
+    }
+    check_in();
+    __syncthreads();
+
+    float acc[MT][8];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[m][e] = 0.0f;
+    for (int bi = 0; bi < nbatch; ++bi) {
+#pragma unroll
+      for (int u = 0; u < D2_UNR1; ++u) {
+        float wv[8];
+        cvt8<T>(pf[u], wv);
+        const int k = rs1 + (bi * D2_UNR1 + u) * rpp1;
+        const bool kok = k < kc;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float a = kok ? a_s[m * KLD + min(k, kc - 1)] : 0.0f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
+        }
+      }
+      if (bi + 1 < nbatch) {                           // deeper slices than one batch: next batch, same registers
+#pragma unroll
+        for (int u = 0; u < D2_UNR1; ++u)
+          pf[u] = ldw16(p.V, wbase + (int64_t)min(rs1 + ((bi + 1) * D2_UNR1 + u) * rpp1, kc - 1) * p.R);
+      }
+    }
+    TR2(1);
+    // every stage-1 load has been consumed: the slab of U may now queue up behind nothing
+    if (has2) issue_prefetch();
+
+    float tot[MT][2];
+    wg_reduce<MT>(acc, lpr1, cv1, red, NC1, tot);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int col = tid + h * 256;
+      if (col < NC1 && n0 + col < p.R) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+          if (m < M) st_tag(&p.ypart[(((int64_t)ks * p.b + j) * M + m) * p.R + n0 + col], tot[m][h], epoch);
+      }
+    }
+    TR2(2);
+  } else {
+    // the loads of stage 1 head the dependency chain: let them reach memory first
+    if (p.pf_wait) asm volatile("" ::"v"(epoch) : "memory");
+    if (has2) issue_prefetch();
+    check_in();
+  }
+
+  // ---- mix role: z[i][m][r] = sum_j S(i, j, r) * sum_ks y[ks][j][m][r] for RCH values of r, every i ------
+  // Thread (g, rr): first g is the block column j whose y it fetches, then the block row i it emits.
+  if (w < p.itemsM) {
+    __syncthreads();                                   // the stage-1 use of a_s is over
+    TR2(8);
+    const int RCH = 1 << p.rch_log2;
+    const int g = tid >> p.rch_log2, rr = tid & (RCH - 1);
+    const int r = w * RCH + rr;
+    const bool live = g < p.b && r < p.R;
+    const T* Sp = reinterpret_cast<const T*>(p.S);
+    float ysum[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) ysum[m] = 0.0f;
+    if (live) {
+      unsigned long long yv[4][MT];
+      unsigned spins = 0;
+      while (true) {
+        bool ok = true;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            if (ks < p.ks1 && m < M) {
+              yv[ks][m] = ld_tag(&p.ypart[(((int64_t)ks * p.b + g) * M + m) * p.R + r]);
+              ok = ok && ((unsigned)(yv[ks][m] >> 32) == epoch);
+            } else {
+              yv[ks][m] = 0ull;
+            }
+          }
+        }
+        if (ok) break;
+        if (++spins > D2_SPIN_LIMIT) {
+          __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) ysum[m] += __uint_as_float((unsigned)yv[ks][m]);
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) a_s[m * 256 + tid] = ysum[m];     // [m][j][rr]
+    __syncthreads();
+    if (live) {
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        if (m < M) {
+          float z = 0.0f;
+#pragma unroll
+          for (int u = 0; u < 16; ++u) z = fmaf((u < p.b) ? sv[u] : 0.0f, a_s[m * 256 + min(u, p.b - 1) * RCH + rr], z);
+          for (int j = 16; j < p.b; ++j)
+            z = fmaf(TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)j * p.s_sj + (int64_t)r * p.s_sr]), a_s[m * 256 + j * RCH + rr], z);
+          st_tag(&p.zt[((int64_t)g * M + m) * p.R + r], z, epoch);
+        }
+      }
+    }
+    TR2(9);
+  }
+  if (!has2) {
+    if (w == 0) finish_epoch(p, epoch, G);
+    return;
+  }
+
+  // ---- stage-2 activations: this slab's slice of z, polled from the tagged pairs into LDS ---------------
+  __syncthreads();                                   // earlier uses of a_s and red are over
+  TR2(3);
+  {
+    const int pairs = kcur2 >> 1;
+    const int total = M * pairs;
+    __amdgpu_buffer_rsrc_t zr = __builtin_amdgcn_make_buffer_rsrc(p.zt, 0, 0x7fffffff, 0x00020000);
+    for (int base = 0; base < total; base += 256 * 4) {
+      u32x4 v[4];
+      unsigned spins = 0;
+      while (true) {
+        bool ok = true;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int idx = base + u * 256 + tid;
+          if (idx < total) {
+            const int m = idx / pairs, kp = idx - m * pairs;
+            const uint32_t off = (uint32_t)((((int64_t)i2 * M + m) * p.R + k0_2 + 2 * kp) * 8);
+            v[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(zr, off, 0, 17));
+            ok = ok && v[u][1] == epoch && v[u][3] == epoch;
+          } else {
+            v[u] = u32x4{0u, 0u, 0u, 0u};
+          }
+        }
+        if (ok) break;
+        if (++spins > D2_SPIN_LIMIT) {
+          __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * 256 + tid;
+        if (idx < total) {
+          const int m = idx / pairs, kp = idx - m * pairs;
+          a_s[m * KLD + 2 * kp] = __uint_as_float(v[u][0]);
+          a_s[m * KLD + 2 * kp + 1] = __uint_as_float(v[u][2]);
+        }
+      }
+    }
+    for (int idx = M * kcur2 + tid; idx < MT * kcur2; idx += 256) {   // rows beyond M contribute nothing
+      const int m = idx / kcur2;
+      a_s[m * KLD + (idx - m * kcur2)] = 0.0f;
+    }
+  }
+  __syncthreads();
+  TR2(4);
+
+  // ---- stage 2: out[m, i Q + n] = sum_k z[m][k] U_i[k, n] ---------------------------------------
+  float acc[MT][8];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[m][e] = 0.0f;
+#pragma unroll
+  for (int u = 0; u < D2_PF; ++u) {
+    const int k = rs2 + u * rpp2;
+    if (u < p.pfn) {
+      float wv[8];
+      cvt8<T>(pf[u], wv);
+      const bool kok = k < kcur2;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const float a = kok ? a_s[m * KLD + min(k, kcur2 - 1)] : 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  {
+    // rows the registers did not hold, in full batches (rows past the end: clamped, zero activation)
+    const int rows_left = kcur2 - p.pfn * rpp2;
+    const int nb = rows_left > 0 ? ((rows_left + rpp2 - 1) / rpp2 + D2_UNR - 1) / D2_UNR : 0;
+    for (int bi = 0; bi < nb; ++bi) {
+      u32x4 raw[D2_UNR];
+#pragma unroll
+      for (int u = 0; u < D2_UNR; ++u)
+        raw[u] = ldw16(p.U, wbase2 + (int64_t)min(rs2 + (p.pfn + bi * D2_UNR + u) * rpp2, kcur2 - 1) * p.Q);
+#pragma unroll
+      for (int u = 0; u < D2_UNR; ++u) {
+        float wv[8];
+        cvt8<T>(raw[u], wv);
+        const int k = rs2 + (p.pfn + bi * D2_UNR + u) * rpp2;
+        const bool kok = k < kcur2;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float a = kok ? a_s[m * KLD + k] : 0.0f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
+        }
+      }
+    }
+  }
+  TR2(5);
+  float tot[MT][2];
+  wg_reduce<MT>(acc, lpr2, cv2, red, NC2, tot);
+  TR2(6);
+  T* outp = reinterpret_cast<T*>(p.out);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int col = tid + h * 256;
+    const int gn = n0_2 + col;
+    if (col < NC2 && gn < p.Q) {
+      if (ksi2 != 0) {                                // a producer of partial sums
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+          if (m < M) st_tag(&p.opart[(((int64_t)(ksi2 - 1) * p.b + i2) * M + m) * p.Q + gn], tot[m][h], epoch);
+      } else {                                        // the slab of k-slice 0 adds the others in order
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          if (m < M) {
+            float v = tot[m][h];
+            for (int ks = 1; ks < p.ks2; ++ks) {
+              const unsigned long long* src = &p.opart[(((int64_t)(ks - 1) * p.b + i2) * M + m) * p.Q + gn];
+              unsigned long long pv;
+              unsigned spins = 0;
+              while (true) {
+                pv = ld_tag(src);
+                if ((unsigned)(pv >> 32) == epoch) break;
+                if (++spins > D2_SPIN_LIMIT) {
+                  __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                  break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+              }
+              v += __uint_as_float((unsigned)pv);
+            }
+            outp[(int64_t)m * p.ldo + (int64_t)i2 * p.Q + gn] = TypeTraits<T>::from_f32(v);
+          }
+        }
+      }
+    }
+  }
+  TR2(7);
+  if (w == 0) finish_epoch(p, epoch, G);
+}
+
+// ---- host side -----------------------------------------------------------------------------------
+namespace {
+
+int env_i(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+}
+int ilog2(int v) { int l = 0; while ((1 << l) < v) ++l; return l; }
+
+template <typename T>
+void* d2_kernel(int MT) {
+  switch (MT) {
+    case 1: return (void*)decode2_kernel<T, 1>;
+    case 2: return (void*)decode2_kernel<T, 2>;
+    default: return (void*)decode2_kernel<T, 4>;
+  }
+}
+
+}  // namespace
+
+size_t decode2_region_bytes() { return (size_t)16 << 20; }
+
+bool decode2_applicable(const StreamBlastArgs& a) {
+  static const int enabled = env_i("BLR_DECODE2", 1);
+  if (!enabled || a.split) return false;
+  if (a.wbits != 16 || a.u_layout != BLR_U_RQ) return false;
+  if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
+  if (a.M < 1 || a.M > 4) return false;
+  const int P = a.in_f / a.b, Q = a.out_f / a.b;
+  if (a.r % 8 || Q % 8 || P < 1) return false;
+  if (!aligned(a.U, 16) || !aligned(a.V, 16)) return false;
+  return true;
+}
+
+// region: the fixed-place 16 MiB block of the workspace reserved for tagged pairs; ctrl3: three
+// words on separate cache lines (epoch, arrivals, error).
+int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
+                         unsigned* err_word, hipStream_t st) {
+  const int P = a.in_f / a.b, Q = a.out_f / a.b, R = a.r, b = a.b, M = a.M;
+  const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
+  const int kc_cap = D2_AS / MT;
+  void* fn = a.dtype == BLR_F16 ? d2_kernel<f16>(MT) : d2_kernel<bf16>(MT);
+
+  static std::mutex mu;
+  static std::map<void*, int> occ_cache;
+  int occ = 0;
+  {
+    std::lock_guard<std::mutex> lk(mu);
+    auto it = occ_cache.find(fn);
+    if (it != occ_cache.end()) occ = it->second;
+    else {
+      hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, 256, 0);
+      if (e != hipSuccess || occ < 1) { (void)hipGetLastError(); set_error("decode2: occupancy query failed"); return BLR_ERR_LAUNCH; }
+      occ_cache[fn] = occ;
+    }
+  }
+  const int cus = device_cus() > 0 ? device_cus() : 256;
+  const int resident = (occ < 2 ? occ : 2) * cus;
+
+  Decode2Params p = {};
+  p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
+  p.M = M; p.b = b; p.P = P; p.R = R; p.Q = Q;
+  if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
+  else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
+  else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
+
+  // stage 1: column chunks of 8 * lpr1 ranks; k split only as far as needed to engage the chip
+  {
+    static const int e_lpr = env_i("BLR_D2_LPR1", 16), e_ks = env_i("BLR_D2_KS1", 0);
+    int lpr = e_lpr;
+    const int vecs = (R + 7) / 8;
+    while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
+    if (lpr > 64) lpr = 64;
+    if (lpr < 4) lpr = 4;
+    const int rpp = 256 / lpr;
+    const int nch = (vecs + lpr - 1) / lpr;
+    const int base = b * nch;
+    if (base > resident) return 1;
+    int ks = e_ks;
+    if (ks <= 0) {
+      const int loads = (P + rpp - 1) / rpp;          // per lane without a split
+      ks = (loads + 15) / 16;
+    }
+    if (ks > resident / base) ks = resident / base;
+    if (ks > 4) ks = 4;
+    if (ks < 1) ks = 1;
+    int kc = (P + ks - 1) / ks;
+    kc = (kc + rpp - 1) / rpp * rpp;
+    if (kc > kc_cap) kc = kc_cap / rpp * rpp;
+    if (kc < 1) return 1;
+    ks = (P + kc - 1) / kc;
+    if (ks > 4 || base * ks > resident) return 1;
+    p.lpr1_log2 = ilog2(lpr); p.nch1 = nch; p.ks1 = ks; p.kc1 = kc; p.items1 = base * ks;
+  }
+  // stage 2: column chunks of 8 * lpr2 outputs; k split so that the slabs cover the resident grid
+  {
+    static const int e_lpr = env_i("BLR_D2_LPR2", 16), e_ks = env_i("BLR_D2_KS2", 0), e_ksmax = env_i("BLR_D2_KS2_MAX", 4);
+    int lpr = e_lpr;
+    const int vecs = (Q + 7) / 8;
+    while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
+    if (lpr > 64) lpr = 64;
+    if (lpr < 4) lpr = 4;
+    const int rpp = 256 / lpr;
+    const int nch = (vecs + lpr - 1) / lpr;
+    const int base = b * nch;
+    if (base > resident) return 1;
+    int ks = e_ks > 0 ? e_ks : resident / base;
+    if (ks > e_ksmax) ks = e_ksmax;
+    if (ks > resident / base) ks = resident / base;
+    if (ks < 1) ks = 1;
+    int kc = (R + ks - 1) / ks;
+    kc = (kc + rpp - 1) / rpp * rpp;
+    if (kc > kc_cap) kc = kc_cap / rpp * rpp;
+    if (kc < 1) return 1;
+    ks = (R + kc - 1) / kc;
+    if (base * ks > resident) return 1;
+    int pfn = (kc + rpp - 1) / rpp;
+    if (pfn > d2_pf(MT)) pfn = d2_pf(MT);
+    p.lpr2_log2 = ilog2(lpr); p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn;
+  }
+  {
+    int bp2 = 1;
+    while (bp2 < b) bp2 <<= 1;
+    if (bp2 > 256) return 1;
+    const int rch = 256 / bp2;
+    p.rch_log2 = ilog2(rch);
+    p.itemsM = (R + rch - 1) / rch;
+    if (p.itemsM > resident) return 1;
+    static const int e_wait = env_i("BLR_D2_PF_WAIT", 1);
+    p.pf_wait = e_wait;
+  }
+  const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)b * M * R * 8, 256);
+  const size_t obytes = (size_t)(p.ks2 - 1) * b * M * Q * 8;
+  if (ybytes + zbytes + obytes > decode2_region_bytes()) return 1;
+  p.ypart = reinterpret_cast<unsigned long long*>(region);
+  p.zt = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes);
+  p.opart = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes + zbytes);
+  p.epoch_word = epoch_word; p.arrive_word = arrive_word; p.err_word = err_word;
+
+  int grid = p.items1 + p.items2;
+  if (grid > resident) grid = resident;
+  if (grid < p.items1) grid = p.items1;
+  if (grid < p.items2) grid = p.items2;
+  if (grid < p.itemsM) grid = p.itemsM;
+  void* args[] = {&p};
+  hipError_t e = hipLaunchKernel(fn, dim3(grid), dim3(256), args, 0, st);
+  if (e != hipSuccess) { set_error("decode2: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  return BLR_OK;
+}
+
+}  // namespace blr
+
+#ifdef BLR_TRACE
+extern "C" int blr_debug_trace2(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(blr::g_trace2), (size_t)n * 8, 0, hipMemcpyDeviceToHost);
+}
+#endif

@@ -23,6 +23,7 @@
 #include <mutex>
 #include <utility>
 #include "blr_common.h"
+#include "blr_decode.h"
 
 namespace blr {
 
@@ -87,6 +88,8 @@ constexpr int BAR_ERR = 2 * BAR_SHARDS * BAR_STRIDE;
 constexpr int BAR_GDONE = BAR_ERR + 64;           // shards that have fully finished (end-of-call bookkeeping)
 constexpr int Z_PARITY = BAR_ERR + 128;           // which Z buffer the current call accumulates into
 constexpr int Z_DIRTY = BAR_ERR + 192;            // [2] floats of each Z buffer that are not known to be zero
+constexpr int D2_EPOCH = BAR_ERR + 256;           // call counter of the two-stage decode kernel
+constexpr int D2_ARRIVE = BAR_ERR + 320;          // its check-in counter
 
 __device__ __forceinline__ unsigned shard_population(int shard) {   // workgroups whose index maps to `shard`
   return ((unsigned)gridDim.x + BAR_SHARDS - 1 - shard) / BAR_SHARDS;
@@ -930,7 +933,7 @@ constexpr size_t CTRL_BYTES = 16384;          // barrier shards, finished counte
 constexpr int MAX_COUNTERS = 8192;
 
 struct WsLayout {
-  unsigned* ctrl; unsigned* counters; float* zb0; float* zb1; float* buf0; float* buf1; float* part;
+  unsigned* ctrl; unsigned* counters; float* zb0; float* zb1; void* d2; float* buf0; float* buf1; float* part;
 };
 constexpr size_t ZCAP_FLOATS = 256 * 1024;    // capacity of each fixed-place Z accumulation buffer (1 MiB)
 
@@ -1123,10 +1126,11 @@ int launch(StreamParams& p, int dtype, int split, hipStream_t st) {
 
 int target_items() { return wgs_per_cu() * (device_cus() > 0 ? device_cus() : 256); }
 
-// Workspace: [ctrl][counters][Z ping][Z pong][buf0][buf1][partials]; everything before buf0 sits at fixed offsets
-// and must be zero before the first call (the kernels leave it consistent afterwards).
+// Workspace: [ctrl][counters][Z ping][Z pong][tagged pairs][buf0][buf1][partials]; everything before buf0 sits at
+// fixed offsets and must be zero before the first call (the kernels leave it consistent afterwards).
 size_t ws_total(size_t buf_elems, size_t part_elems) {
-  return CTRL_BYTES + MAX_COUNTERS * sizeof(unsigned) + 2 * ZCAP_FLOATS * 4 + align_up(buf_elems * 4, 256) * 2 + align_up(part_elems * 4, 256);
+  return CTRL_BYTES + MAX_COUNTERS * sizeof(unsigned) + 2 * ZCAP_FLOATS * 4 + decode2_region_bytes() +
+         align_up(buf_elems * 4, 256) * 2 + align_up(part_elems * 4, 256);
 }
 WsLayout ws_carve(void* ws, size_t buf_elems) {
   WsLayout l;
@@ -1135,6 +1139,7 @@ WsLayout ws_carve(void* ws, size_t buf_elems) {
   l.counters = reinterpret_cast<unsigned*>(p); p += MAX_COUNTERS * sizeof(unsigned);
   l.zb0 = reinterpret_cast<float*>(p); p += ZCAP_FLOATS * 4;
   l.zb1 = reinterpret_cast<float*>(p); p += ZCAP_FLOATS * 4;
+  l.d2 = p; p += decode2_region_bytes();
   l.buf0 = reinterpret_cast<float*>(p); p += align_up(buf_elems * 4, 256);
   l.buf1 = reinterpret_cast<float*>(p); p += align_up(buf_elems * 4, 256);
   l.part = reinterpret_cast<float*>(p);
@@ -1163,6 +1168,10 @@ int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st) {
   size_t need = stream_blast_workspace(a.M, a.in_f, a.out_f, a.b, a.r, a.wbits);
   if (!a.ws || a.ws_bytes < need) { set_error("blast stream: workspace %zu < %zu", a.ws_bytes, need); return BLR_ERR_WORKSPACE; }
   WsLayout w = ws_carve(a.ws, (size_t)a.b * a.M * a.r);
+  if (decode2_applicable(a)) {
+    int rc = decode2_blast_launch(a, w.d2, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
+    if (rc <= 0) return rc;                    // served (or failed); 1 = shape outside its tiling
+  }
   const int MT = mt_for(a.M), target = target_items();
   const bool zatom = a.M <= zatom_max_m() && (size_t)a.b * a.M * a.r <= ZCAP_FLOATS;
   const bool inline_mix = !zatom && a.M <= mix_inline_max_m();
