@@ -28,7 +28,8 @@ namespace {
 // 16-byte loads of the U slab held in registers per lane (fewer when the accumulators need the room)
 constexpr int d2_pf(int MT) { return MT <= 1 ? 32 : (MT <= 2 ? 24 : 16); }
 constexpr int D2_UNR = 8;             // loads in flight per lane while streaming the rest of a slab
-constexpr int d2_unr1(int MT) { return MT <= 2 ? 16 : 8; }   // loads in flight per lane in stage 1
+constexpr int d2_unr1(int) { return 8; }   // loads in flight per lane in stage 1
+constexpr int d2_ks1_max(int MT) { return MT <= 2 ? 8 : 4; } // most k-slices of stage 1 (the mix fetches them all at once)
 constexpr int D2_SHARDS = 16;         // check-in counters, 256 bytes apart
 constexpr int D2_AS = 4096;           // fp32 activations staged in LDS (MT * k-chunk <= this)
 constexpr int D2_NC_MAX = 512;
@@ -49,8 +50,8 @@ struct Decode2Params {
   int M, b, P, R, Q;
   int64_t s_si, s_sj, s_sr;
   int lpr1_log2, nch1, ks1, kc1, items1;
-  int lpr2_log2, nch2, ks2, kc2, items2, pfn;
-  int itemsM, rch_log2, pf_wait;
+  int lpr2_log2, nch2, ks2, kc2, items2, pfn, kpad2;
+  int itemsM, rch_log2, pf_depth;
   unsigned long long* ypart;           // [ks1][b][M][R] tagged
   unsigned long long* zt;              // [b][M][R] tagged
   unsigned long long* opart;           // [ks2 - 1][b][M][Q] tagged
@@ -71,8 +72,14 @@ __device__ __forceinline__ void cvt8(const u32x4& r, float (&w)[8]) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) w[e] = TypeTraits<T>::to_f32(v[e]);
 }
-__device__ __forceinline__ u32x4 ldw16(const void* W, int64_t eoff) {
-  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(W) + eoff));
+// 16-byte streaming load through a buffer descriptor that spans the whole factor: the per-lane
+// byte offset sits in one register, the per-load row offset is uniform (scalar), and a row past
+// the end of the factor reads as zero instead of faulting - no clamping, no 64-bit addresses.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wbuf(const void* W, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(W), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 ldw16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 2));   // nt
 }
 
 // Sum of the row slots of a wave, then of the four waves; thread `col` < NC ends up with the
@@ -135,6 +142,7 @@ template <typename T, int MT>
 __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   constexpr int D2_PF = d2_pf(MT);
   constexpr int D2_UNR1 = d2_unr1(MT);
+  constexpr int D2_KS1_MAX = d2_ks1_max(MT);
   __shared__ float a_s[D2_AS];
   __shared__ float red[4 * MT * D2_NC_MAX];
   constexpr int KLD = D2_AS / MT;
@@ -161,13 +169,26 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   const int n0_2 = nc2 * NC2;
   const int n2 = n0_2 + cv2 * 8;
   const bool col_ok2 = n2 < p.Q;
-  const int64_t wbase2 = ((int64_t)i2 * p.R + k0_2) * p.Q + (col_ok2 ? n2 : 0);
+  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.b * p.R * p.Q * 2u);
+  const uint32_t uoff = (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs2) * p.Q + (col_ok2 ? n2 : 0)) * 2);   // bytes, row rs2 of the slab
+  const uint32_t ustep = (uint32_t)rpp2 * p.Q * 2u;                                                       // bytes between a lane's loads
 
   u32x4 pf[D2_PF];                                   // only slots below pfn are ever read after the prefetch
   auto issue_prefetch = [&]() {
 #pragma unroll
     for (int u = 0; u < D2_PF; ++u) {
-      if (u < p.pfn) pf[u] = ldw16(p.U, wbase2 + (int64_t)min(rs2 + u * rpp2, kcur2 - 1) * p.Q);
+      if (u < p.pfn) {
+        // pacing: at most pf_depth of this lane's loads in flight, so that the queues of the memory
+        // system stay short enough for the small hand-over accesses of other workgroups to get through
+        if (u >= 2 && p.pf_depth == 2) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+        else if (u >= 3 && p.pf_depth == 3) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else if (u >= 4 && p.pf_depth == 4) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+        else if (u >= 6 && p.pf_depth == 6) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+        else if (u >= 8 && p.pf_depth == 8) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+        else if (u >= 12 && p.pf_depth == 12) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
+        else if (u >= 16 && p.pf_depth == 16) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
+        pf[u] = ldw16(ubuf, uoff, (uint32_t)u * ustep);
+      }
     }
   };
 
@@ -203,17 +224,37 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     const int NC1 = lpr1 * 8;
     const int n0 = nc1 * NC1, n = n0 + cv1 * 8;
     const bool col_ok = n < p.R;
-    const int64_t wbase = ((int64_t)j * p.P + k0) * p.R + (col_ok ? n : 0);
+    const __amdgpu_buffer_rsrc_t vbuf = wbuf(p.V, (uint32_t)p.b * p.P * p.R * 2u);
+    const uint32_t voff = (uint32_t)((((int64_t)j * p.P + k0 + rs1) * p.R + (col_ok ? n : 0)) * 2);
+    const uint32_t vstep = (uint32_t)rpp1 * p.R * 2u;
 
-    // The registers that will hold the slab of U serve as the load buffer of stage 1 first.  Batches
-    // are always full: rows past the end are clamped to the last one and meet a zero activation.
+    // Batches are always full: rows past the end of the slice meet a zero activation.
     const int nbatch = ((kc + rpp1 - 1) / rpp1 + D2_UNR1 - 1) / D2_UNR1;
-#pragma unroll
-    for (int u = 0; u < D2_UNR1; ++u) pf[u] = ldw16(p.V, wbase + (int64_t)min(rs1 + u * rpp1, kc - 1) * p.R);
+    const int kpad = nbatch * D2_UNR1 * rpp1;          // rows the batches touch (the host keeps this within KLD)
+    // The activations go first of all (loads come back in order, and they are needed first).
     const T* xp = reinterpret_cast<const T*>(p.x);
-    for (int idx = tid; idx < MT * kc; idx += 256) {
-      const int m = idx / kc, ka = idx - m * kc;
-      a_s[m * KLD + ka] = (m < M) ? TypeTraits<T>::to_f32(xp[(int64_t)m * p.ldx + (int64_t)j * p.P + k0 + ka]) : 0.0f;
+    constexpr int XR = 4;
+    T xr[XR];
+#pragma unroll
+    for (int q = 0; q < XR; ++q) {
+      const int idx = tid + q * 256;
+      const int m = min(idx / kpad, M - 1), ka = min(idx % kpad, kc - 1);
+      xr[q] = xp[(int64_t)m * p.ldx + (int64_t)j * p.P + k0 + ka];
+    }
+    u32x4 raw[D2_UNR1];
+#pragma unroll
+    for (int u = 0; u < D2_UNR1; ++u) raw[u] = ldw16(vbuf, voff, (uint32_t)u * vstep);
+#pragma unroll
+    for (int q = 0; q < XR; ++q) {
+      const int idx = tid + q * 256;
+      if (idx < MT * kpad) {
+        const int m = idx / kpad, ka = idx - m * kpad;
+        a_s[m * KLD + ka] = (m < M && ka < kc) ? TypeTraits<T>::to_f32(xr[q]) : 0.0f;
+      }
+    }
+    for (int idx = tid + XR * 256; idx < MT * kpad; idx += 256) {   // long slices only
+      const int m = idx / kpad, ka = idx - m * kpad;
+      a_s[m * KLD + ka] = (m < M && ka < kc) ? TypeTraits<T>::to_f32(xp[(int64_t)m * p.ldx + (int64_t)j * p.P + k0 + ka]) : 0.0f;
     }
     check_in();
     __syncthreads();
@@ -227,25 +268,22 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
 #pragma unroll
       for (int u = 0; u < D2_UNR1; ++u) {
         float wv[8];
-        cvt8<T>(pf[u], wv);
+        cvt8<T>(raw[u], wv);
         const int k = rs1 + (bi * D2_UNR1 + u) * rpp1;
-        const bool kok = k < kc;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-          const float a = kok ? a_s[m * KLD + min(k, kc - 1)] : 0.0f;
+          const float a = a_s[m * KLD + k];            // zero beyond the slice
 #pragma unroll
           for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
         }
       }
-      if (bi + 1 < nbatch) {                           // deeper slices than one batch: next batch, same registers
+      if (bi + 1 < nbatch) {                           // deeper slices than one batch (the planner avoids them)
 #pragma unroll
         for (int u = 0; u < D2_UNR1; ++u)
-          pf[u] = ldw16(p.V, wbase + (int64_t)min(rs1 + ((bi + 1) * D2_UNR1 + u) * rpp1, kc - 1) * p.R);
+          raw[u] = ldw16(vbuf, voff, (uint32_t)((bi + 1) * D2_UNR1 + u) * vstep);
       }
     }
     TR2(1);
-    // every stage-1 load has been consumed: the slab of U may now queue up behind nothing
-    if (has2) issue_prefetch();
 
     float tot[MT][2];
     wg_reduce<MT>(acc, lpr1, cv1, red, NC1, tot);
@@ -260,9 +298,6 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     }
     TR2(2);
   } else {
-    // the loads of stage 1 head the dependency chain: let them reach memory first
-    if (p.pf_wait) asm volatile("" ::"v"(epoch) : "memory");
-    if (has2) issue_prefetch();
     check_in();
   }
 
@@ -280,12 +315,12 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) ysum[m] = 0.0f;
     if (live) {
-      unsigned long long yv[4][MT];
+      unsigned long long yv[D2_KS1_MAX][MT];
       unsigned spins = 0;
       while (true) {
         bool ok = true;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < D2_KS1_MAX; ++ks) {
 #pragma unroll
           for (int m = 0; m < MT; ++m) {
             if (ks < p.ks1 && m < M) {
@@ -304,7 +339,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
         __builtin_amdgcn_s_sleep(1);
       }
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
+      for (int ks = 0; ks < D2_KS1_MAX; ++ks)
 #pragma unroll
         for (int m = 0; m < MT; ++m) ysum[m] += __uint_as_float((unsigned)yv[ks][m]);
     }
@@ -330,6 +365,11 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     if (w == 0) finish_epoch(p, epoch, G);
     return;
   }
+
+  // The slab of U: asked for only now, after this workgroup's share of stage 1 (and of the mix), because
+  // a wave that queues this many loads is held up until most of them have been accepted, and the
+  // work heading the dependency chain must not sit behind that.
+  issue_prefetch();
 
   // ---- stage-2 activations: this slab's slice of z, polled from the tagged pairs into LDS ---------------
   __syncthreads();                                   // earlier uses of a_s and red are over
@@ -372,9 +412,11 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
         }
       }
     }
-    for (int idx = M * kcur2 + tid; idx < MT * kcur2; idx += 256) {   // rows beyond M contribute nothing
-      const int m = idx / kcur2;
-      a_s[m * KLD + (idx - m * kcur2)] = 0.0f;
+    // zero what the products below touch beyond the real data: rows m >= M and k in [kcur2, kpad2)
+    const int kpad2 = p.kpad2;
+    for (int idx = tid; idx < MT * kpad2; idx += 256) {
+      const int m = idx / kpad2, k = idx - m * kpad2;
+      if (m >= M || k >= kcur2) a_s[m * KLD + k] = 0.0f;
     }
   }
   __syncthreads();
@@ -392,10 +434,9 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     if (u < p.pfn) {
       float wv[8];
       cvt8<T>(pf[u], wv);
-      const bool kok = k < kcur2;
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
-        const float a = kok ? a_s[m * KLD + min(k, kcur2 - 1)] : 0.0f;
+        const float a = a_s[m * KLD + k];              // zero beyond the slice
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
       }
@@ -403,23 +444,22 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     }
   }
   {
-    // rows the registers did not hold, in full batches (rows past the end: clamped, zero activation)
+    // rows the registers did not hold, in full batches (rows past the end meet a zero activation)
     const int rows_left = kcur2 - p.pfn * rpp2;
     const int nb = rows_left > 0 ? ((rows_left + rpp2 - 1) / rpp2 + D2_UNR - 1) / D2_UNR : 0;
     for (int bi = 0; bi < nb; ++bi) {
       u32x4 raw[D2_UNR];
 #pragma unroll
       for (int u = 0; u < D2_UNR; ++u)
-        raw[u] = ldw16(p.U, wbase2 + (int64_t)min(rs2 + (p.pfn + bi * D2_UNR + u) * rpp2, kcur2 - 1) * p.Q);
+        raw[u] = ldw16(ubuf, uoff, (uint32_t)(p.pfn + bi * D2_UNR + u) * ustep);
 #pragma unroll
       for (int u = 0; u < D2_UNR; ++u) {
         float wv[8];
         cvt8<T>(raw[u], wv);
         const int k = rs2 + (p.pfn + bi * D2_UNR + u) * rpp2;
-        const bool kok = k < kcur2;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-          const float a = kok ? a_s[m * KLD + k] : 0.0f;
+          const float a = a_s[m * KLD + k];
 #pragma unroll
           for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
         }
@@ -501,6 +541,7 @@ bool decode2_applicable(const StreamBlastArgs& a) {
   const int P = a.in_f / a.b, Q = a.out_f / a.b;
   if (a.r % 8 || Q % 8 || P < 1) return false;
   if (!aligned(a.U, 16) || !aligned(a.V, 16)) return false;
+  if ((int64_t)a.r * a.out_f * 2 >= (1ll << 31) || (int64_t)a.r * a.in_f * 2 >= (1ll << 31)) return false;   // 32-bit buffer offsets
   return true;
 }
 
@@ -510,7 +551,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
                          unsigned* err_word, hipStream_t st) {
   const int P = a.in_f / a.b, Q = a.out_f / a.b, R = a.r, b = a.b, M = a.M;
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
-  const int kc_cap = D2_AS / MT;
+  const int kc_cap = D2_AS / MT - 256;           // the kernels pad a slice up to 255 rows with zeros
   void* fn = a.dtype == BLR_F16 ? d2_kernel<f16>(MT) : d2_kernel<bf16>(MT);
 
   static std::mutex mu;
@@ -548,20 +589,21 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     const int nch = (vecs + lpr - 1) / lpr;
     const int base = b * nch;
     if (base > resident) return 1;
-    int ks = e_ks;
-    if (ks <= 0) {
-      const int loads = (P + rpp - 1) / rpp;          // per lane without a split
-      ks = (loads + 15) / 16;
-    }
+    // split k just far enough that a lane's share of a slice is one batch of loads
+    const int ks_max = d2_ks1_max(MT);
+    int ks = e_ks > 0 ? e_ks : ((P + rpp - 1) / rpp + d2_unr1(MT) - 1) / d2_unr1(MT);
     if (ks > resident / base) ks = resident / base;
-    if (ks > 4) ks = 4;
+    if (ks > ks_max) ks = ks_max;
+    if (ks > (P + rpp - 1) / rpp) ks = (P + rpp - 1) / rpp;     // at least one load per lane
     if (ks < 1) ks = 1;
     int kc = (P + ks - 1) / ks;
     kc = (kc + rpp - 1) / rpp * rpp;
     if (kc > kc_cap) kc = kc_cap / rpp * rpp;
     if (kc < 1) return 1;
     ks = (P + kc - 1) / kc;
-    if (ks > 4 || base * ks > resident) return 1;
+    if (ks > ks_max || base * ks > resident) return 1;
+    const int unr1 = d2_unr1(MT);
+    if (((kc + rpp - 1) / rpp + unr1 - 1) / unr1 * unr1 * rpp > D2_AS / MT) return 1;   // zero padding must fit too
     p.lpr1_log2 = ilog2(lpr); p.nch1 = nch; p.ks1 = ks; p.kc1 = kc; p.items1 = base * ks;
   }
   // stage 2: column chunks of 8 * lpr2 outputs; k split so that the slabs cover the resident grid
@@ -588,7 +630,10 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     if (base * ks > resident) return 1;
     int pfn = (kc + rpp - 1) / rpp;
     if (pfn > d2_pf(MT)) pfn = d2_pf(MT);
-    p.lpr2_log2 = ilog2(lpr); p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn;
+    const int left = (kc + rpp - 1) / rpp - pfn;     // loads per lane beyond the register-resident ones
+    const int kpad2 = (pfn + (left > 0 ? (left + D2_UNR - 1) / D2_UNR * D2_UNR : 0)) * rpp;
+    if (kpad2 > D2_AS / MT) return 1;
+    p.lpr2_log2 = ilog2(lpr); p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn; p.kpad2 = kpad2;
   }
   {
     int bp2 = 1;
@@ -598,8 +643,8 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     p.rch_log2 = ilog2(rch);
     p.itemsM = (R + rch - 1) / rch;
     if (p.itemsM > resident) return 1;
-    static const int e_wait = env_i("BLR_D2_PF_WAIT", 1);
-    p.pf_wait = e_wait;
+    static const int e_depth = env_i("BLR_D2_PF_DEPTH", 4);
+    p.pf_depth = e_depth;
   }
   const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)b * M * R * 8, 256);
   const size_t obytes = (size_t)(p.ks2 - 1) * b * M * Q * 8;
