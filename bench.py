@@ -34,8 +34,8 @@ LAYERS = {"qkvo": (4096, 4096, 512), "gate_up": (4096, 22016, 1024), "down": (11
 B = 16
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE), scaled
-# by the same counters over a copy kernel of known size; None until measured.
-TRAFFIC_BYTES = None
+# by the same counters over a copy kernel of known size (1 FETCH_SIZE unit = 1.99978 KiB, 1 WRITE_SIZE unit = 1 KiB).
+TRAFFIC_BYTES = 70.96e6   # 70.33 MB fetched + 0.63 MB written (profiles/decode2_kernel_blast_llama7b_decode_m1.txt)
 
 
 def blast_bytes_flops(n, i, r, o, b=B, elt=2):
@@ -49,6 +49,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-table", action="store_true", help="skip the per-layer table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--pmc", choices=["dominant", "calib"], default=None,
+                    help="counter-collection helper: launch only the dominant kernel (dominant) or only copy/probe kernels "
+                         "of known size (calib), eagerly, and print nothing but a note")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -173,6 +176,27 @@ def main():
         torch.cuda.empty_cache()
         return us
 
+    # ---- counter-collection helper (run under rocprofv3 --pmc) ---------------------------------------
+    if args.pmc == "calib":
+        nbytes = 256 << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        words = torch.zeros(lib.blr_probe_dst_words(), dtype=torch.int32, device=dev)
+        for _ in range(4):
+            dst.copy_(src)                                                   # reads 256 MiB, writes 256 MiB
+            L.check(lib.blr_stream_probe(src.data_ptr(), nbytes, words.data_ptr(), torch.cuda.current_stream().cuda_stream), "probe")
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc": "calib", "copy_bytes_read": nbytes, "copy_bytes_written": nbytes, "probe_bytes_read": nbytes}))
+        return
+    if args.pmc == "dominant":
+        gu = [mk_blast(1, *LAYERS["gate_up"][:2], LAYERS["gate_up"][2], L.U_RQ, L.S_JIR) for _ in range(12)]
+        st = torch.cuda.current_stream().cuda_stream
+        for i in range(36):
+            gu[i % 12][0](st)
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc": "dominant", "launches": 36, "algorithmic_bytes": blast_bytes_flops(1, 4096, 1024, 22016)[0]}))
+        return
+
     # ---- headline: one decoder layer's six BLAST linears at M = 1 ---------------------------------
     M = 1
     step_bytes = 4 * blast_bytes_flops(M, *LAYERS["qkvo"][:1], LAYERS["qkvo"][2], LAYERS["qkvo"][1])[0] \
@@ -203,7 +227,7 @@ def main():
     gu_us = time_graph(g_gu, n_l)
     gu_bytes, gu_flops = blast_bytes_flops(M, LAYERS["gate_up"][0], LAYERS["gate_up"][2], LAYERS["gate_up"][1])
     achieved = gu_bytes / (gu_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "stream_kernel<f16,1> (BLAST gate_up 4096->22016 r=1024 b=16, M=1)",
+    roofline = {"bound": "hbm", "kernel": "decode2_kernel<f16,1> (BLAST gate_up 4096->22016 r=1024 b=16, M=1)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": round(achieved * 1e9 / HBM_PEAK, 4),
                 "us_per_launch": round(gu_us, 3), "algorithmic_bytes": gu_bytes, "traffic": TRAFFIC_BYTES}
     del g_gu, step_graphs, sets
@@ -272,7 +296,7 @@ def main():
             for x, U, Vt, S in ops:
                 T.blast(x, U, Vt, S)
         reps, t_used, times = 0, 0.0, []
-        while t_used < 10.0 and reps < 2000:
+        while t_used < 12.0 and reps < 100000:
             c0 = time.perf_counter()
             for x, U, Vt, S in ops:
                 T.blast(x, U, Vt, S)
