@@ -51,7 +51,7 @@ struct Decode2Params {
   int64_t s_si, s_sj, s_sr;
   int lpr1_log2, nch1, ks1, kc1, items1;
   int lpr2_log2, nch2, ks2, kc2, items2, pfn, kpad2;
-  int itemsM, rch_log2, pf_depth;
+  int itemsM, rch_log2, pf_depth, x_vec;
   unsigned long long* ypart;           // [ks1][b][M][R] tagged
   unsigned long long* zt;              // [b][M][R] tagged
   unsigned long long* opart;           // [ks2 - 1][b][M][Q] tagged
@@ -510,6 +510,395 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   if (w == 0) finish_epoch(p, epoch, G);
 }
 
+
+// ---- matrix-core variant: up to 16 token rows --------------------------------------------------
+// Same roles and hand-overs as decode2_kernel; the products run on v_mfma_f32_16x16x32.  Column
+// chunks are 128 wide (16 lanes x 8), a lane loads 8 consecutive rows of its 8 columns per batch
+// (a batch of a workgroup = 128 rows), transposes the 8x8 block in registers into eight B
+// fragments, and the activations - staged in LDS as [16][k] of T - are the A fragment.  z crosses
+// workgroups as {two T values, epoch} pairs (half the bytes of fp32 pairs: a slab's slice of z
+// is 16 x 512 values at M = 16).
+constexpr int DM_ROWS = 128;          // rows per batch of a workgroup
+constexpr int DM_PF = 32;             // loads of the U slab kept in registers (4 batches)
+constexpr int DM_KMAX = 1024;         // deepest staged slice
+constexpr int DM_MC = 4;              // token rows per mix item
+
+template <typename T>
+__device__ __forceinline__ void dm_batch(const u32x4 (&cur)[8], const T* a_s, int ald, int cv, int rs, int kbase, f32x4 (&acc)[8]) {
+  using V8 = typename TypeTraits<T>::vec8;
+  const V8 af = *reinterpret_cast<const V8*>(&a_s[cv * ald + kbase + rs * 8]);     // row m = lane % 16, k = 8 (lane / 16) ..
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    u32x4 bb;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      bb[q] = __builtin_amdgcn_perm(cur[2 * q + 1][e >> 1], cur[2 * q][e >> 1], (e & 1) ? 0x07060302u : 0x05040100u);
+    acc[e] = TypeTraits<T>::mfma16(af, __builtin_bit_cast(V8, bb), acc[e]);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  typedef T T2 __attribute__((ext_vector_type(2)));
+  T2 v = {TypeTraits<T>::from_f32(a), TypeTraits<T>::from_f32(b)};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
+  __shared__ __attribute__((aligned(16))) T a_s[16 * (DM_KMAX + 8)];
+  __shared__ __attribute__((aligned(16))) float red[4 * 4 * 64 * 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int cv = lane & 15, kg = lane >> 4, rs = wave * 4 + kg;
+  const int w = blockIdx.x, G = gridDim.x;
+  const int M = p.M;
+  TR2(0);
+
+  unsigned epoch = __hip_atomic_load(p.epoch_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  if (epoch == 0u) epoch = 1u;
+  auto check_in = [&]() {
+    if (tid == 0) {
+      asm volatile("" ::"v"(epoch) : "memory");
+      (void)__hip_atomic_fetch_add(&p.arrive_word[(w % D2_SHARDS) * 64], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+
+  // ---- stage-2 slab -------------------------------------------------------------------------------
+  const int item2 = G - 1 - w;
+  const bool has2 = item2 < p.items2;
+  const int nc2 = has2 ? item2 % p.nch2 : 0;
+  const int t2 = has2 ? item2 / p.nch2 : 0;
+  const int i2 = t2 % p.b, ksi2 = t2 / p.b;
+  const int k0_2 = ksi2 * p.kc2;
+  const int kcur2 = min(p.kc2, p.R - k0_2);
+  const int n0_2 = nc2 * 128;
+  const int n2 = n0_2 + cv * 8;
+  const bool col_ok2 = n2 < p.Q;
+  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.b * p.R * p.Q * 2u);
+  const uint32_t uoff = (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs * 8) * p.Q + (col_ok2 ? n2 : 0)) * 2);
+  const uint32_t urow = (uint32_t)p.Q * 2u;
+  u32x4 pf[DM_PF];
+  auto issue_prefetch = [&]() {
+#pragma unroll
+    for (int u = 0; u < DM_PF; ++u) {
+      if (u < p.pfn) {
+        if (u >= 4 && p.pf_depth == 4) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+        else if (u >= 8 && p.pf_depth == 8) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+        else if (u >= 16 && p.pf_depth == 16) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
+        pf[u] = ldw16(ubuf, uoff, (uint32_t)((u >> 3) * DM_ROWS + (u & 7)) * urow);
+      }
+    }
+  };
+
+  // Reduction of the four waves' fragments and hand-out of the totals: emit(h, e, l, v) receives,
+  // for half h and fragment e, the four rows m = 4 (l / 16) + i of column 8 (l % 16) + 4 h + e.
+  auto reduce_emit = [&](f32x4 (&acc)[8], auto&& emit) {
+    f32x4 vh[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < 4; ++e) *reinterpret_cast<f32x4*>(&red[((wave * 4 + e) * 64 + lane) * 4]) = acc[h * 4 + e];
+      __syncthreads();
+      const int e = tid >> 6, l = tid & 63;
+      f32x4 v = *reinterpret_cast<const f32x4*>(&red[((0 * 4 + e) * 64 + l) * 4]);
+      v += *reinterpret_cast<const f32x4*>(&red[((1 * 4 + e) * 64 + l) * 4]);
+      v += *reinterpret_cast<const f32x4*>(&red[((2 * 4 + e) * 64 + l) * 4]);
+      v += *reinterpret_cast<const f32x4*>(&red[((3 * 4 + e) * 64 + l) * 4]);
+      vh[h] = v;
+    }
+    const int e = tid >> 6, l = tid & 63;
+    emit((l & 15) * 8 + e, (l >> 4) * 4, vh);                       // columns col and col + 4
+  };
+
+  // ---- mix role: S of this thread's (i, r), asked for first -------------------------------------------
+  const int nrc = (p.R + (1 << p.rch_log2) - 1) >> p.rch_log2;
+  float sv[16];
+  if (w < p.itemsM) {
+    const int g = min(tid >> p.rch_log2, p.b - 1);
+    const int r = min((w % nrc) * (1 << p.rch_log2) + (tid & ((1 << p.rch_log2) - 1)), p.R - 1);
+    const T* Sp = reinterpret_cast<const T*>(p.S);
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      sv[u] = TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]);
+  }
+
+  // ---- stage 1 -----------------------------------------------------------------------------------
+  if (w < p.items1) {
+    const int nc1 = w % p.nch1;
+    const int t1 = w / p.nch1;
+    const int j = t1 % p.b, ks = t1 / p.b;
+    const int k0 = ks * p.kc1, kc = min(p.kc1, p.P - k0);
+    const int n0 = nc1 * 128, n = n0 + cv * 8;
+    const bool col_ok = n < p.R;
+    const __amdgpu_buffer_rsrc_t vbuf = wbuf(p.V, (uint32_t)p.b * p.P * p.R * 2u);
+    const uint32_t voff = (uint32_t)((((int64_t)j * p.P + k0 + rs * 8) * p.R + (col_ok ? n : 0)) * 2);
+    const uint32_t vrow = (uint32_t)p.R * 2u;
+    const int nbatch = (kc + DM_ROWS - 1) / DM_ROWS;
+    const int kpad = nbatch * DM_ROWS, ald = kpad + 8;
+    u32x4 raw[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) raw[u] = ldw16(vbuf, voff, (uint32_t)u * vrow);
+    // activations straight into LDS as T (zero outside the slice and beyond M)
+    const T* xp = reinterpret_cast<const T*>(p.x);
+    if (p.x_vec) {                                               // 16-byte pieces: one or two per thread
+      const int pieces = kpad >> 3;
+      for (int idx = tid; idx < 16 * pieces; idx += 256) {
+        const int m = idx / pieces, ka = (idx - m * pieces) * 8;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (m < M && ka < kc) v = *reinterpret_cast<const u32x4*>(&xp[(int64_t)m * p.ldx + (int64_t)j * p.P + k0 + ka]);
+        if (m < M && ka + 8 > kc && ka < kc) {                   // piece straddling the end of the slice
+          uint16_t* h = reinterpret_cast<uint16_t*>(&v);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) if (ka + e >= kc) h[e] = 0;
+        }
+        *reinterpret_cast<u32x4*>(&a_s[m * ald + ka]) = v;
+      }
+    } else {
+      for (int idx = tid; idx < 16 * kpad; idx += 256) {
+        const int m = idx / kpad, ka = idx - m * kpad;
+        T v = TypeTraits<T>::from_f32(0.0f);
+        if (m < M && ka < kc) v = xp[(int64_t)m * p.ldx + (int64_t)j * p.P + k0 + ka];
+        a_s[m * ald + ka] = v;
+      }
+    }
+    check_in();
+    __syncthreads();
+    f32x4 acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int bi = 0; bi < nbatch; ++bi) {
+      u32x4 cur[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) cur[u] = raw[u];
+      if (bi + 1 < nbatch) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) raw[u] = ldw16(vbuf, voff, (uint32_t)((bi + 1) * DM_ROWS + u) * vrow);
+      }
+      dm_batch<T>(cur, a_s, ald, cv, rs, bi * DM_ROWS, acc);
+    }
+    TR2(1);
+    reduce_emit(acc, [&](int col, int m0, const f32x4 (&vh)[2]) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int gn = n0 + col + 4 * h;
+        if (gn < p.R) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (m0 + i < M) st_tag(&p.ypart[(((int64_t)ks * p.b + j) * M + m0 + i) * p.R + gn], vh[h][i], epoch);
+        }
+      }
+    });
+    TR2(2);
+  } else {
+    check_in();
+  }
+
+  // ---- mix role: item = (chunk of RCH ranks, DM_MC token rows); z goes out as tagged pairs of T -----------
+  if (w < p.itemsM) {
+    __syncthreads();
+    TR2(8);
+    float* ys = reinterpret_cast<float*>(a_s);                  // [DM_MC][256]
+    const int RCH = 1 << p.rch_log2;
+    const int g = tid >> p.rch_log2, rr = tid & (RCH - 1);
+    const int r = (w % nrc) * RCH + rr;
+    const int mbase = (w / nrc) * DM_MC;
+    const bool live = g < p.b && r < p.R;
+    const T* Sp = reinterpret_cast<const T*>(p.S);
+    float ysum[DM_MC];
+#pragma unroll
+    for (int m = 0; m < DM_MC; ++m) ysum[m] = 0.0f;
+    if (live) {
+      unsigned long long yv[4][DM_MC];
+      unsigned spins = 0;
+      while (true) {
+        bool ok = true;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+          for (int m = 0; m < DM_MC; ++m) {
+            if (ks < p.ks1 && mbase + m < M) {
+              yv[ks][m] = ld_tag(&p.ypart[(((int64_t)ks * p.b + g) * M + mbase + m) * p.R + r]);
+              ok = ok && ((unsigned)(yv[ks][m] >> 32) == epoch);
+            } else {
+              yv[ks][m] = 0ull;
+            }
+          }
+        }
+        if (ok) break;
+        if (++spins > D2_SPIN_LIMIT) {
+          __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int m = 0; m < DM_MC; ++m) ysum[m] += __uint_as_float((unsigned)yv[ks][m]);
+    }
+#pragma unroll
+    for (int m = 0; m < DM_MC; ++m) ys[m * 256 + tid] = ysum[m];
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < DM_MC; ++m) {
+      float z = 0.0f;
+      if (live) {
+#pragma unroll
+        for (int u = 0; u < 16; ++u) z = fmaf((u < p.b) ? sv[u] : 0.0f, ys[m * 256 + min(u, p.b - 1) * RCH + rr], z);
+        for (int jx = 16; jx < p.b; ++jx)
+          z = fmaf(TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)jx * p.s_sj + (int64_t)r * p.s_sr]), ys[m * 256 + jx * RCH + rr], z);
+      }
+      const float zn = __shfl_down(z, 1, 64);                    // rank r + 1 (same i: RCH is even)
+      if (live && (rr & 1) == 0 && mbase + m < M) {
+        const unsigned long long v = ((unsigned long long)epoch << 32) | pack2<T>(z, (r + 1 < p.R) ? zn : 0.0f);
+        __hip_atomic_store(&p.zt[((int64_t)g * M + mbase + m) * (p.R >> 1) + (r >> 1)], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    TR2(9);
+  }
+  if (!has2) {
+    if (w == 0) finish_epoch(p, epoch, G);
+    return;
+  }
+
+  issue_prefetch();
+
+  // ---- stage-2 activations: z slice -> LDS as T ----------------------------------------------------------
+  __syncthreads();
+  TR2(3);
+  const int kpad2 = p.kpad2, ald2 = kpad2 + 8;
+  {
+    const int quads = kcur2 >> 2;                                 // 16-byte units (4 ranks) per token row
+    const int total = M * quads;
+    __amdgpu_buffer_rsrc_t zr = __builtin_amdgcn_make_buffer_rsrc(p.zt, 0, 0x7fffffff, 0x00020000);
+    for (int base = 0; base < total; base += 256 * 8) {
+      u32x4 v[8];
+      unsigned spins = 0;
+      while (true) {
+        bool ok = true;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int idx = base + u * 256 + tid;
+          if (idx < total) {
+            const int m = idx / quads, kq = idx - m * quads;
+            const uint32_t off = (uint32_t)((((int64_t)i2 * M + m) * (p.R >> 1) + ((k0_2 + 4 * kq) >> 1)) * 8);
+            v[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(zr, off, 0, 17));
+            ok = ok && v[u][1] == epoch && v[u][3] == epoch;
+          } else {
+            v[u] = u32x4{0u, 0u, 0u, 0u};
+          }
+        }
+        if (ok) break;
+        if (++spins > D2_SPIN_LIMIT) {
+          __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int idx = base + u * 256 + tid;
+        if (idx < total) {
+          const int m = idx / quads, kq = idx - m * quads;
+          uint32_t* dst = reinterpret_cast<uint32_t*>(&a_s[m * ald2 + 4 * kq]);
+          dst[0] = v[u][0];
+          dst[1] = v[u][2];
+        }
+      }
+    }
+    for (int idx = tid; idx < 16 * kpad2; idx += 256) {           // zero rows beyond M and ranks beyond the slice
+      const int m = idx / kpad2, k = idx - m * kpad2;
+      if (m >= M || k >= kcur2) a_s[m * ald2 + k] = TypeTraits<T>::from_f32(0.0f);
+    }
+  }
+  __syncthreads();
+  TR2(4);
+
+  // ---- stage 2 --------------------------------------------------------------------------------------
+  f32x4 acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int bq = 0; bq < DM_PF / 8; ++bq) {
+    if (bq * 8 < p.pfn) {
+      u32x4 cur[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) cur[u] = pf[bq * 8 + u];
+      dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+    }
+  }
+  for (int bq = p.pfn / 8; bq * DM_ROWS < kcur2; ++bq) {          // deeper slabs: stream the rest
+    u32x4 cur[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) cur[u] = ldw16(ubuf, uoff, (uint32_t)(bq * DM_ROWS + u) * urow);
+    dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+  }
+  TR2(5);
+  T* outp = reinterpret_cast<T*>(p.out);
+  reduce_emit(acc, [&](int col, int m0, const f32x4 (&vh)[2]) {
+    if (ksi2 != 0) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int gn = n0_2 + col + 4 * h;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (gn < p.Q && m0 + i < M) st_tag(&p.opart[(((int64_t)(ksi2 - 1) * p.b + i2) * M + m0 + i) * p.Q + gn], vh[h][i], epoch);
+      }
+      return;
+    }
+    float tot[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) tot[h][i] = vh[h][i];
+    if (p.ks2 > 1) {                                                // all partial sums of this thread's 8 outputs in one go
+      unsigned long long pv[3][2][4];
+      unsigned spins = 0;
+      while (true) {
+        bool ok = true;
+#pragma unroll
+        for (int ks = 1; ks < 4; ++ks) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int gn = n0_2 + col + 4 * h;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              if (ks < p.ks2 && gn < p.Q && m0 + i < M) {
+                pv[ks - 1][h][i] = ld_tag(&p.opart[(((int64_t)(ks - 1) * p.b + i2) * M + m0 + i) * p.Q + gn]);
+                ok = ok && ((unsigned)(pv[ks - 1][h][i] >> 32) == epoch);
+              } else {
+                pv[ks - 1][h][i] = 0ull;
+              }
+            }
+          }
+        }
+        if (ok) break;
+        if (++spins > D2_SPIN_LIMIT) {
+          __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 3; ++ks)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) tot[h][i] += __uint_as_float((unsigned)pv[ks][h][i]);
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int gn = n0_2 + col + 4 * h;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (gn < p.Q && m0 + i < M) outp[(int64_t)(m0 + i) * p.ldo + (int64_t)i2 * p.Q + gn] = TypeTraits<T>::from_f32(tot[h][i]);
+    }
+  });
+  TR2(7);
+  if (w == 0) finish_epoch(p, epoch, G);
+}
+
 // ---- host side -----------------------------------------------------------------------------------
 namespace {
 
@@ -537,7 +926,7 @@ bool decode2_applicable(const StreamBlastArgs& a) {
   if (!enabled || a.split) return false;
   if (a.wbits != 16 || a.u_layout != BLR_U_RQ) return false;
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
-  if (a.M < 1 || a.M > 4) return false;
+  if (a.M < 1 || a.M > 16) return false;
   const int P = a.in_f / a.b, Q = a.out_f / a.b;
   if (a.r % 8 || Q % 8 || P < 1) return false;
   if (!aligned(a.U, 16) || !aligned(a.V, 16)) return false;
@@ -545,11 +934,17 @@ bool decode2_applicable(const StreamBlastArgs& a) {
   return true;
 }
 
+int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
+                          unsigned* err_word, hipStream_t st);
+
 // region: the fixed-place 16 MiB block of the workspace reserved for tagged pairs; ctrl3: three
 // words on separate cache lines (epoch, arrivals, error).
 int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
                          unsigned* err_word, hipStream_t st) {
   const int P = a.in_f / a.b, Q = a.out_f / a.b, R = a.r, b = a.b, M = a.M;
+  static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
+  if (M >= mfma_min_m) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
+  if (M > 4) return 1;
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int kc_cap = D2_AS / MT - 256;           // the kernels pad a slice up to 255 rows with zeros
   void* fn = a.dtype == BLR_F16 ? d2_kernel<f16>(MT) : d2_kernel<bf16>(MT);
@@ -662,6 +1057,99 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   void* args[] = {&p};
   hipError_t e = hipLaunchKernel(fn, dim3(grid), dim3(256), args, 0, st);
   if (e != hipSuccess) { set_error("decode2: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  return BLR_OK;
+}
+
+// Matrix-core variant of the launch (any M <= 16).
+int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
+                          unsigned* err_word, hipStream_t st) {
+  const int P = a.in_f / a.b, Q = a.out_f / a.b, R = a.r, b = a.b, M = a.M;
+  void* fn = a.dtype == BLR_F16 ? (void*)decode2m_kernel<f16> : (void*)decode2m_kernel<bf16>;
+  static std::mutex mu;
+  static std::map<void*, int> occ_cache;
+  int occ = 0;
+  {
+    std::lock_guard<std::mutex> lk(mu);
+    auto it = occ_cache.find(fn);
+    if (it != occ_cache.end()) occ = it->second;
+    else {
+      hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, 256, 0);
+      if (e != hipSuccess || occ < 1) { (void)hipGetLastError(); set_error("decode2m: occupancy query failed"); return BLR_ERR_LAUNCH; }
+      occ_cache[fn] = occ;
+    }
+  }
+  const int cus = device_cus() > 0 ? device_cus() : 256;
+  const int resident = (occ < 2 ? occ : 2) * cus;
+  if (R % 4) return 1;
+
+  Decode2Params p = {};
+  p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
+  p.M = M; p.b = b; p.P = P; p.R = R; p.Q = Q;
+  if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
+  else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
+  else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
+  {
+    static const int e_ks = env_i("BLR_DM_KS1", 0);
+    const int nch = (R + 127) / 128, base = b * nch;
+    if (base > resident) return 1;
+    int ks = e_ks > 0 ? e_ks : (P + DM_ROWS - 1) / DM_ROWS;       // one batch per slice if the grid allows
+    if (ks > resident / base) ks = resident / base;
+    if (ks > 4) ks = 4;
+    if (ks < 1) ks = 1;
+    int kc = (P + ks - 1) / ks;
+    kc = (kc + 7) / 8 * 8;
+    if (kc > DM_KMAX) kc = DM_KMAX;
+    ks = (P + kc - 1) / kc;
+    if (ks > 4 || base * ks > resident) return 1;
+    p.lpr1_log2 = 4; p.nch1 = nch; p.ks1 = ks; p.kc1 = kc; p.items1 = base * ks;
+    // a slice of x may be fetched in 16-byte pieces if every piece is aligned and inside the row
+    p.x_vec = aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0 && kc % 8 == 0;
+  }
+  {
+    static const int e_ks = env_i("BLR_DM_KS2", 0), e_ksmax = env_i("BLR_DM_KS2_MAX", 4);
+    const int nch = (Q + 127) / 128, base = b * nch;
+    if (base > resident) return 1;
+    int ks = e_ks > 0 ? e_ks : resident / base;
+    if (ks > e_ksmax) ks = e_ksmax;
+    if (ks > 4) ks = 4;
+    if (ks > resident / base) ks = resident / base;
+    if (ks < 1) ks = 1;
+    int kc = (R + ks - 1) / ks;
+    kc = (kc + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
+    if (kc > DM_KMAX) kc = DM_KMAX;
+    ks = (R + kc - 1) / kc;
+    if (ks > 4 || base * ks > resident) return 1;
+    int pfn = (kc + DM_ROWS - 1) / DM_ROWS * 8;
+    if (pfn > DM_PF) pfn = DM_PF;
+    p.lpr2_log2 = 4; p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn;
+    p.kpad2 = (kc + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
+  }
+  {
+    int bp2 = 2;                                   // at least two ranks per mix thread row: z goes out in pairs
+    while (bp2 < b) bp2 <<= 1;
+    if (bp2 > 128) return 1;
+    const int rch = 256 / bp2;
+    p.rch_log2 = ilog2(rch);
+    p.itemsM = ((R + rch - 1) / rch) * ((M + DM_MC - 1) / DM_MC);
+    if (p.itemsM > resident) return 1;
+    static const int e_depth = env_i("BLR_DM_PF_DEPTH", 4);
+    p.pf_depth = e_depth;
+  }
+  const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)b * M * (R / 2) * 8, 256);
+  const size_t obytes = (size_t)(p.ks2 - 1) * b * M * Q * 8;
+  if (ybytes + zbytes + obytes > decode2_region_bytes()) return 1;
+  p.ypart = reinterpret_cast<unsigned long long*>(region);
+  p.zt = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes);
+  p.opart = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes + zbytes);
+  p.epoch_word = epoch_word; p.arrive_word = arrive_word; p.err_word = err_word;
+  int grid = p.items1 + p.items2;
+  if (grid > resident) grid = resident;
+  if (grid < p.items1) grid = p.items1;
+  if (grid < p.items2) grid = p.items2;
+  if (grid < p.itemsM) grid = p.itemsM;
+  void* args[] = {&p};
+  hipError_t e = hipLaunchKernel(fn, dim3(grid), dim3(256), args, 0, st);
+  if (e != hipSuccess) { set_error("decode2m: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
 }
 
