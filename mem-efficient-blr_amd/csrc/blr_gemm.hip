@@ -35,7 +35,7 @@ template <typename T, int ROWS>
 struct KcStage {
   static constexpr int NV = ROWS * 8 / 256;
   using V8 = typename TypeTraits<T>::vec8;
-  V8 v[NV];
+  struct Vals { V8 v[NV]; };
   const T* p[NV];
 
   __device__ __forceinline__ void init(const T* base, int64_t ld, int row0, int nrows, int tid) {
@@ -46,10 +46,10 @@ struct KcStage {
       p[i] = base + (int64_t)min(row0 + row, nrows - 1) * ld + kv;
     }
   }
-  __device__ __forceinline__ void load(int k0, int K, bool vec_ok, int tid) {
+  __device__ __forceinline__ void load(Vals& r, int k0, int K, bool vec_ok, int tid) const {
     if (vec_ok && k0 + BK <= K) {
 #pragma unroll
-      for (int i = 0; i < NV; ++i) v[i] = ldg16<V8>(p[i] + k0);
+      for (int i = 0; i < NV; ++i) r.v[i] = ldg16<V8>(p[i] + k0);
       return;
     }
 #pragma unroll
@@ -59,15 +59,15 @@ struct KcStage {
       V8 val;
 #pragma unroll
       for (int e = 0; e < 8; ++e) val[e] = (gk + e < K) ? p[i][k0 + e] : (T)0.0f;
-      v[i] = val;
+      r.v[i] = val;
     }
   }
-  __device__ __forceinline__ void store(T (*s)[LDS_LD], int tid) const {
+  __device__ __forceinline__ void store(const Vals& r, T (*s)[LDS_LD], int tid) const {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       int vi = tid + i * 256;
       int row = vi >> 3, kv = (vi & 7) * 8;
-      *reinterpret_cast<V8*>(&s[row][kv]) = v[i];
+      *reinterpret_cast<V8*>(&s[row][kv]) = r.v[i];
     }
   }
 };
@@ -80,7 +80,7 @@ template <typename T, int COLS>
 struct KnStage {
   static constexpr int NP = COLS / 128;
   using V8 = typename TypeTraits<T>::vec8;
-  V8 v[NP][4];
+  struct Vals { V8 v[NP][4]; };
   const T* p[NP];
   int64_t ld;
   int nvalid[NP];                           // columns of this thread's vector that exist (0..8)
@@ -99,12 +99,12 @@ struct KnStage {
       p[ps] = base + (int64_t)(kq * 4) * ld + gn;
     }
   }
-  __device__ __forceinline__ void load(int k0, int K, bool vec_ok, int tid) {
+  __device__ __forceinline__ void load(Vals& r, int k0, int K, bool vec_ok, int tid) const {
     if (vec_ok && k0 + BK <= K) {
 #pragma unroll
       for (int ps = 0; ps < NP; ++ps)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[ps][i] = ldg16<V8>(p[ps] + (int64_t)(k0 + i) * ld);
+        for (int i = 0; i < 4; ++i) r.v[ps][i] = ldg16<V8>(p[ps] + (int64_t)(k0 + i) * ld);
       return;
     }
     int kq = tid & 15;
@@ -125,10 +125,10 @@ struct KnStage {
               if (e < nvalid[ps]) val[e] = q[e];
           }
         }
-        v[ps][i] = val;
+        r.v[ps][i] = val;
       }
   }
-  __device__ __forceinline__ void store(T (*s)[LDS_LD], int tid) const {
+  __device__ __forceinline__ void store(const Vals& r, T (*s)[LDS_LD], int tid) const {
     int lane = tid & 63, wave = tid >> 6;
     int kq = lane & 15;
 #pragma unroll
@@ -137,7 +137,7 @@ struct KnStage {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         typename TypeTraits<T>::vec4 w;
-        w[0] = v[ps][0][e]; w[1] = v[ps][1][e]; w[2] = v[ps][2][e]; w[3] = v[ps][3][e];
+        w[0] = r.v[ps][0][e]; w[1] = r.v[ps][1][e]; w[2] = r.v[ps][2][e]; w[3] = r.v[ps][3][e];
         *reinterpret_cast<typename TypeTraits<T>::vec4*>(&s[nv * 8 + e][kq * 4]) = w;
       }
     }
@@ -152,7 +152,7 @@ __device__ __forceinline__ int64_t epi_offset(const GemmArgs& g, int bt, int m, 
   return (int64_t)bt * g.sC + (int64_t)m * g.ldc + (int64_t)n * g.cn;
 }
 
-template <typename T, int BM, int BN, bool B_KN>
+template <typename T, int BM, int BN, bool B_KN, int PD>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int a_vec, int b_vec, int c_vec) {
   constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;    // 32x32 MFMA tiles per wave
@@ -185,50 +185,63 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
   KcStage<T, BM> sa;
   KcStage<T, BN> sb_kc;
   KnStage<T, BN> sb_kn;
+  // PD register sets of staged tiles: global loads run PD k-tiles ahead of the multiplication.
+  // One set measured fastest on MI355X (deeper prefetch only added register pressure).
+  typename KcStage<T, BM>::Vals ra[PD];
+  typename KcStage<T, BN>::Vals rb_kc[B_KN ? 1 : PD];
+  typename KnStage<T, BN>::Vals rb_kn[B_KN ? PD : 1];
 
   const int KT = (g.K + BK - 1) / BK;
   sa.init(A, g.lda, m0, g.M, tid);
   if (B_KN) sb_kn.init(B, g.ldb, n0, g.N, tid, b_vec);
   else sb_kc.init(B, g.ldb, n0, g.N, tid);
-  sa.load(0, g.K, a_vec, tid);
-  if (B_KN) sb_kn.load(0, g.K, b_vec, tid);
-  else sb_kc.load(0, g.K, b_vec, tid);
-  sa.store(sm[0].a, tid);
-  if (B_KN) sb_kn.store(sm[0].b, tid);
-  else sb_kc.store(sm[0].b, tid);
+  auto load_tile = [&](int d, int t) {
+    sa.load(ra[d], t * BK, g.K, a_vec, tid);
+    if (B_KN) sb_kn.load(rb_kn[B_KN ? d : 0], t * BK, g.K, b_vec, tid);
+    else sb_kc.load(rb_kc[B_KN ? 0 : d], t * BK, g.K, b_vec, tid);
+  };
+  auto store_tile = [&](int d, Smem& dst) {
+    sa.store(ra[d], dst.a, tid);
+    if (B_KN) sb_kn.store(rb_kn[B_KN ? d : 0], dst.b, tid);
+    else sb_kc.store(rb_kc[B_KN ? 0 : d], dst.b, tid);
+  };
+#pragma unroll
+  for (int d = 0; d < PD; ++d)
+    if (d < KT) load_tile(d, d);
+  store_tile(0, sm[0]);
   __syncthreads();
 
-  for (int kt = 0; kt < KT; ++kt) {
-    Smem& cur = sm[kt & 1];
-    const bool more = kt + 1 < KT;
-    if (more) {                            // next tile's global loads fly while this one is multiplied
-      int k0 = (kt + 1) * BK;
-      sa.load(k0, g.K, a_vec, tid);
-      if (B_KN) sb_kn.load(k0, g.K, b_vec, tid);
-      else sb_kc.load(k0, g.K, b_vec, tid);
+  for (int kt0 = 0; kt0 < KT; kt0 += PD) {
+#pragma unroll
+    for (int d = 0; d < PD; ++d) {
+      const int kt = kt0 + d;
+      if (kt < KT) {
+        Smem& cur = sm[kt & 1];
+        if (kt + PD < KT) load_tile(d, kt + PD);   // set d went to LDS one step ago: free again
+        // fragments of step kk + 1 are fetched from LDS before the matrix instructions of step kk are issued
+        V8 af[2][TM], bf[2][TN];
+        auto frags = [&](int kk, int set) {
+          const int kof = kk * 16 + (lane >> 5) * 8;
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            af[set][i] = *reinterpret_cast<const V8*>(&cur.a[wm * WM + i * 32 + (lane & 31)][kof]);
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            bf[set][j] = *reinterpret_cast<const V8*>(&cur.b[wn * WN + j * 32 + (lane & 31)][kof]);
+        };
+        frags(0, 0);
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+          if (kk + 1 < BK / 16) frags(kk + 1, (kk + 1) & 1);
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = TypeTraits<T>::mfma32(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
+        }
+        if (kt + 1 < KT) store_tile((d + 1) % PD, sm[(kt + 1) & 1]);   // nobody reads that stage until the barrier
+        __syncthreads();
+      }
     }
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      const int kof = kk * 16 + (lane >> 5) * 8;
-      V8 af[TM], bf[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        af[i] = *reinterpret_cast<const V8*>(&cur.a[wm * WM + i * 32 + (lane & 31)][kof]);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        bf[j] = *reinterpret_cast<const V8*>(&cur.b[wn * WN + j * 32 + (lane & 31)][kof]);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = TypeTraits<T>::mfma32(af[i], bf[j], acc[i][j]);
-    }
-    if (more) {                            // the other stage is free: nobody reads it until the barrier below
-      Smem& nxt = sm[(kt + 1) & 1];
-      sa.store(nxt.a, tid);
-      if (B_KN) sb_kn.store(nxt.b, tid);
-      else sb_kc.store(nxt.b, tid);
-    }
-    __syncthreads();
   }
 
   // D fragment: element e of lane l is row (e/4)*8 + (l/32)*4 + e%4, column l%32.
@@ -323,6 +336,14 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) 
     }
 }
 
+template <typename T, int BM, int BN, bool B_KN>
+static void* mfma_kernel_ptr(int pd) {
+  switch (pd) {
+    case 2: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 2>;
+    default: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 1>;
+  }
+}
+
 template <typename T, int BM, int BN>
 static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
@@ -331,7 +352,9 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   int b_vec = aligned(g.B, 16) && g.ldb % 8 == 0 && g.sB % 8 == 0;
   int c_vec = g.epi == EPI_PLAIN && g.cn == 1 && aligned(g.C, 16) && g.ldc % 8 == 0 && g.sC % 8 == 0 && g.N % 8 == 0;
   size_t lds = 2 * sizeof(GemmSmem<T, BM, BN>);
-  void* fn = g.b_kn ? (void*)gemm_mfma_kernel<T, BM, BN, true> : (void*)gemm_mfma_kernel<T, BM, BN, false>;
+  // k-tiles of global loads kept in flight (tuning aid: BLR_GEMM_PD = 1, 2 or 3)
+  static const int pd = [] { const char* e = getenv("BLR_GEMM_PD"); return e ? atoi(e) : 1; }();
+  void* fn = g.b_kn ? mfma_kernel_ptr<T, BM, BN, true>(pd) : mfma_kernel_ptr<T, BM, BN, false>(pd);
   static std::mutex mu;
   static std::set<void*> raised;
   {
@@ -485,6 +508,53 @@ __global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict_
   }
 }
 
+// fp16 only: the same mix with packed half-precision multiply-adds (two per lane and instruction).
+// The b <= 16 products of one output are accumulated in fp16; Z is stored as fp16 anyway and the
+// reference rounds it to 16 bits as well, so this costs about one extra rounding of the result.
+__global__ __launch_bounds__(256) void blast_mix_h2_kernel(const f16* __restrict__ Y, const f16* __restrict__ S,
+                                                           f16* __restrict__ Z, int M, int b, int R,
+                                                           int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  struct H8 { h2 v[4]; };
+  extern __shared__ float s_lds[];
+  f16* s_t = reinterpret_cast<f16*>(s_lds);      // [b][b][64]  (j, i, r)
+  const int tid = threadIdx.x;
+  const int r0 = blockIdx.x * 64;
+  for (int idx = tid; idx < b * b * 64; idx += 256) {
+    int r = idx & 63, ji = idx >> 6;
+    int j = ji / b, i = ji - j * b;
+    f16 v = (f16)0.0f;
+    if (r0 + r < R) v = S[(int64_t)i * s_si + (int64_t)j * s_sj + (int64_t)(r0 + r) * s_sr];
+    s_t[idx] = v;
+  }
+  __syncthreads();
+  const int rl = tid & 7, ms = tid >> 3;     // 8 r-vectors x 32 m slots
+  const int r = r0 + rl * 8;
+  if (r >= R) return;
+  const int m_begin = blockIdx.y * m_per_wg;
+  const int m_end = min(M, m_begin + m_per_wg);
+  for (int m = m_begin + ms; m < m_end; m += 32) {
+    H8 yv[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if (j < b) yv[j] = *reinterpret_cast<const H8*>(&Y[((int64_t)j * M + m) * R + r]);
+    for (int i = 0; i < b; ++i) {
+      H8 acc;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc.v[e] = h2{(_Float16)0.0f, (_Float16)0.0f};
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        if (j < b) {
+          const H8 sv = *reinterpret_cast<const H8*>(&s_t[(j * b + i) * 64 + rl * 8]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc.v[e] = sv.v[e] * yv[j].v[e] + acc.v[e];
+        }
+      }
+      *reinterpret_cast<H8*>(&Z[((int64_t)i * M + m) * R + r]) = acc;
+    }
+  }
+}
+
 int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
                      int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st) {
   int r_chunks = (int)cdiv(R, 64);
@@ -493,7 +563,10 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
     int m_per_wg = 128;
     while ((int64_t)r_chunks * cdiv(M, m_per_wg) < 512 && m_per_wg > 32) m_per_wg /= 2;
     dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
-    if (dtype == BLR_F16)
+    static const bool h2 = [] { const char* e = getenv("BLR_MIX_H2"); return e ? atoi(e) != 0 : true; }();
+    if (dtype == BLR_F16 && h2)
+      hipLaunchKernelGGL(blast_mix_h2_kernel, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+    else if (dtype == BLR_F16)
       hipLaunchKernelGGL(blast_mix_vec_kernel<f16>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
     else
       hipLaunchKernelGGL(blast_mix_vec_kernel<bf16>, grid, dim3(256), lds, st, (const bf16*)Y, (const bf16*)S, (bf16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
