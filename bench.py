@@ -91,12 +91,12 @@ def main():
     def mk_blast_q(M, in_f, out_f, r, bits):
         p, q = in_f // B, out_f // B
         x = randn(M, in_f)
-        U = randn(B, q, r, std=r ** -0.5, dtype=torch.float32)
+        U = randn(B, r, q, std=r ** -0.5, dtype=torch.float32)          # (k, n)-ordered like V
         V = randn(B, p, r, std=r ** -0.5, dtype=torch.float32)
         S = randn(r, B, B)
-        uc = torch.empty((B, q, r * bits // 8), dtype=torch.uint8, device=dev); us = torch.empty((B, q), dtype=f16, device=dev)
+        uc = torch.empty((B, r, q * bits // 8), dtype=torch.uint8, device=dev); us = torch.empty((B, q), dtype=f16, device=dev)
         vc = torch.empty((B, p, r * bits // 8), dtype=torch.uint8, device=dev); vs = torch.empty((B, r), dtype=f16, device=dev)
-        L.check(lib.blr_quantize_sym(U.data_ptr(), L.F32, B * q, r, 1, bits, uc.data_ptr(), us.data_ptr(), None), "quantize U")
+        L.check(lib.blr_quantize_sym(U.data_ptr(), L.F32, B, r, q, bits, uc.data_ptr(), us.data_ptr(), None), "quantize U")
         L.check(lib.blr_quantize_sym(V.data_ptr(), L.F32, B, p, r, bits, vc.data_ptr(), vs.data_ptr(), None), "quantize V")
         torch.cuda.synchronize()
         del U, V

@@ -84,10 +84,11 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
 
 /* ---- weight-quantized BLAST ---------------------------------------------------------------
  * Same product with U and V stored as symmetric int8 (bits = 8) or packed int4 (bits = 4) codes
- * and fp16 per-output-channel scales: U codes (b, q, r[/2]) + u_scales (b, q); V codes
- * (b, p, r[/2]) + v_scales (b, r); S (r, i, j) of dtype.  Served behind the name
- * triton_blast_bmm_int8_fp16 (reference triton_funcs/blast_sym_quant_kernels.py:558-580).
-  * r % 32 == 0.  M <= 16 streams the codes; larger M expands them to dtype in the workspace first.                                                                     */
+ * and fp16 per-output-channel scales.  Both factors are stored (k, n)-ordered, the order in which
+ * the kernels stream them: U codes (b, r, q[/2]) + u_scales (b, q); V codes (b, p, r[/2]) +
+ * v_scales (b, r); S (r, i, j) of dtype.  Served behind the name triton_blast_bmm_int8_fp16
+ * (reference triton_funcs/blast_sym_quant_kernels.py:558-580).  r % 32 == 0 and q % 8 == 0.
+ * M <= 16 streams the codes; larger M expands them to dtype in the workspace first.           */
 size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits);
 int blr_blast_q_fwd(const void* x, int64_t ldx,
                     const void* u_codes, const void* u_scales,
@@ -100,7 +101,8 @@ int blr_blast_q_fwd(const void* x, int64_t ldx,
 /* Symmetric per-channel quantizer producing the codes/scales consumed above.  w is viewed as
  * (outer, reduce, inner) contiguous; the max-abs runs over `reduce`.  scales: fp16 (outer, inner).
  * codes: int8 (outer, reduce, inner), or for bits = 4 two codes per byte along the flattened
- * last axis (low nibble = even index).  No reference counterpart (the reference has no weight
+ * last axis (low nibble = even index).  U (b, r, q): outer = b, reduce = r, inner = q; V (b, p, r):
+ * outer = b, reduce = p, inner = r.  No reference counterpart (the reference has no weight
  * quantizer).                                                                                */
 int blr_quantize_sym(const void* w, int dtype, int64_t outer, int64_t reduce, int64_t inner,
                      int bits, void* codes, void* scales, void* stream);

@@ -253,6 +253,7 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   int rc = check_blast_shape("blast_q", M, in_f, out_f, b, r);
   if (rc) return rc;
   if (r % 32) { set_error("blast_q: r=%d must be a multiple of 32", r); return BLR_ERR_BAD_SHAPE; }
+  if ((out_f / b) % 8) { set_error("blast_q: out_f / b = %d must be a multiple of 8", out_f / b); return BLR_ERR_BAD_SHAPE; }
   if (ldx < in_f || ldo < out_f) { set_error("blast_q: leading dimension too small"); return BLR_ERR_BAD_ARG; }
   if (!aligned(u_codes, 16) || !aligned(v_codes, 16)) { set_error("blast_q: code buffers must be 16-byte aligned"); return BLR_ERR_BAD_ARG; }
   hipStream_t st = (hipStream_t)stream;
@@ -263,22 +264,23 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
     char* wp = reinterpret_cast<char*>(ws);
     void* Ud = wp; wp += align_up((size_t)r * out_f * 2, 256);
     void* Vd = wp; wp += align_up((size_t)r * in_f * 2, 256);
-    const int64_t urows = out_f, vrows = in_f;
+    // both factors are (k, n)-ordered with one scale per column of their block: U (b, r, q), V (b, p, r)
+    const int64_t urows = (int64_t)b * r, vrows = in_f, q = out_f / b;
     if (dtype == BLR_F16) {
-      hipLaunchKernelGGL(dequant_kernel<f16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)u_codes, (const f16*)u_scales, (f16*)Ud, urows, (int64_t)r, bits, 0, (int64_t)1);
+      hipLaunchKernelGGL(dequant_kernel<f16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)u_codes, (const f16*)u_scales, (f16*)Ud, urows, q, bits, 1, (int64_t)r);
       hipLaunchKernelGGL(dequant_kernel<f16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)v_codes, (const f16*)v_scales, (f16*)Vd, vrows, (int64_t)r, bits, 1, (int64_t)(in_f / b));
     } else {
-      hipLaunchKernelGGL(dequant_kernel<bf16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)u_codes, (const f16*)u_scales, (bf16*)Ud, urows, (int64_t)r, bits, 0, (int64_t)1);
+      hipLaunchKernelGGL(dequant_kernel<bf16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)u_codes, (const f16*)u_scales, (bf16*)Ud, urows, q, bits, 1, (int64_t)r);
       hipLaunchKernelGGL(dequant_kernel<bf16>, dim3(2048), dim3(256), 0, st, (const uint8_t*)v_codes, (const f16*)v_scales, (bf16*)Vd, vrows, (int64_t)r, bits, 1, (int64_t)(in_f / b));
     }
     BLR_CHECK_LAUNCH("dequant");
-    return blr_blast_fwd(x, ldx, Ud, Vd, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, BLR_U_QR, BLR_S_RIJ,
+    return blr_blast_fwd(x, ldx, Ud, Vd, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, BLR_U_RQ, BLR_S_RIJ,
                          BLR_ALGO_TILED, wp, ws_bytes - (size_t)(wp - reinterpret_cast<char*>(ws)), stream);
   }
   StreamBlastArgs s = {};
   s.x = x; s.ldx = ldx; s.U = u_codes; s.V = v_codes; s.S = S; s.u_scales = u_scales; s.v_scales = v_scales;
   s.out = out; s.ldo = ldo; s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
-  s.dtype = dtype; s.u_layout = BLR_U_QR; s.s_layout = BLR_S_RIJ; s.wbits = bits;
+  s.dtype = dtype; s.u_layout = BLR_U_RQ; s.s_layout = BLR_S_RIJ; s.wbits = bits;
   s.ws = ws; s.ws_bytes = ws_bytes; s.split = (algo == BLR_ALGO_STREAM_SPLIT);
   return stream_blast_launch(s, st);
 }

@@ -9,8 +9,9 @@ the scale of V is folded into S, the scale of U is applied to the output row.
 
 The reference has no weight quantizer; the scheme is this library's own: symmetric, per output
 channel, scale = fp16(max|w| / Qmax) (1 for an all-zero channel), code = clamp(rne(w / scale),
--Qmax, Qmax) with Qmax = 127 (int8) or 7 (int4); int4 codes are packed two per byte along r,
-low nibble = even r.
+-Qmax, Qmax) with Qmax = 127 (int8) or 7 (int4).  Codes are stored (k, n)-ordered - U as
+(b, r, q), V as (b, p, r) - and int4 codes are packed two per byte along the last axis, low
+nibble = even index.
 """
 from __future__ import annotations
 
@@ -28,7 +29,7 @@ _last_config = {}
 
 
 class QuantFactor(NamedTuple):
-    codes: torch.Tensor      # int8 (…, r) or uint8 (…, r/2) when bits == 4
+    codes: torch.Tensor      # int8, or uint8 with the last axis halved when bits == 4 (U: (b, r, q), V: (b, p, r))
     scales: torch.Tensor     # float16
     bits: int
     shape: tuple             # logical (unpacked) shape of the factor
@@ -63,8 +64,11 @@ def quantize_sym(w, reduce_dim, bits=8):
 
 
 def quantize_blast_factors(U, V, bits=8):
-    """U (b, q, r) -> per-(b, q) scales; V (b, p, r) -> per-(b, r) scales (V maps p -> r)."""
-    uc, us = quantize_sym(U, 2, bits)
+    """U (b, q, r) -> per-(b, q) scales; V (b, p, r) -> per-(b, r) scales (V maps p -> r).
+
+    The codes of U are stored transposed, (b, r, q[/2]) - the order the kernels stream them in
+    (output channel contiguous, like V); ``QuantFactor.shape`` keeps the logical (b, q, r)."""
+    uc, us = quantize_sym(U.transpose(1, 2).contiguous(), 1, bits)
     vc, vs = quantize_sym(V, 1, bits)
     return QuantFactor(uc, us, bits, tuple(U.shape)), QuantFactor(vc, vs, bits, tuple(V.shape))
 

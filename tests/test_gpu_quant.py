@@ -63,7 +63,8 @@ def test_blast_q_vs_oracle_on_dequantized(shape, bits, dtype):
     uc, us = O.quantize_sym(U, 2, bits); vc, vs = O.quantize_sym(V, 1, bits)
     got_uc = Uq.codes.cpu().numpy() if bits == 8 else O.unpack_int4(Uq.codes.cpu().numpy())
     got_vc = Vq.codes.cpu().numpy() if bits == 8 else O.unpack_int4(Vq.codes.cpu().numpy())
-    np.testing.assert_array_equal(got_uc, uc); np.testing.assert_array_equal(got_vc, vc)
+    np.testing.assert_array_equal(got_uc.transpose(0, 2, 1), uc)      # U codes are stored (b, r, q)
+    np.testing.assert_array_equal(got_vc, vc)
     np.testing.assert_array_equal(Uq.scales.cpu().numpy(), us); np.testing.assert_array_equal(Vq.scales.cpu().numpy(), vs)
     fn = Q.triton_blast_bmm_int8_fp16 if bits == 8 else Q.triton_blast_bmm_int4_fp16
     ref = O.blast_q_forward(rounded(x, dtype), uc, us, vc, vs, rounded(S, dtype))
@@ -90,7 +91,8 @@ def test_blast_q_llama7b(layer, bits, M):
     Uq, Vq = Q.quantize_blast_factors(torch.from_numpy(U).cuda(), torch.from_numpy(V).cuda(), bits)
     uc, us = O.quantize_sym(U, 2, bits); vc, vs = O.quantize_sym(V, 1, bits)
     got_uc = Uq.codes.cpu().numpy() if bits == 8 else O.unpack_int4(Uq.codes.cpu().numpy())
-    np.testing.assert_array_equal(got_uc, uc)
+    np.testing.assert_array_equal(got_uc.transpose(0, 2, 1), uc)      # U codes are stored (b, r, q)
+    np.testing.assert_array_equal(Uq.scales.cpu().numpy(), us)
     np.testing.assert_array_equal(Vq.scales.cpu().numpy(), vs)
     out = Q.triton_blast_bmm_int8_fp16(dev(x, torch.float16), Uq, Vq, dev(S, torch.float16))
     ref = O.blast_q_forward(rounded(x, torch.float16), uc, us, vc, vs, rounded(S, torch.float16))
