@@ -26,7 +26,7 @@ namespace blr {
 
 namespace {
 // 16-byte loads of the U slab held in registers per lane (fewer when the accumulators need the room)
-constexpr int d2_pf(int MT) { return MT <= 1 ? 32 : (MT <= 2 ? 24 : 16); }
+constexpr int d2_pf(int MT, int WB = 16) { return MT * (128 / WB) >= 64 ? 16 : (MT <= 1 ? 32 : (MT <= 2 ? 24 : 16)); }
 constexpr int D2_UNR = 8;             // loads in flight per lane while streaming the rest of a slab
 constexpr int d2_unr1(int) { return 8; }   // loads in flight per lane in stage 1
 constexpr int d2_ks1_max(int MT) { return MT <= 2 ? 8 : 4; } // most k-slices of stage 1 (the mix fetches them all at once)
@@ -46,6 +46,7 @@ __device__ unsigned long long g_trace2[1024 * 16];
 struct Decode2Params {
   const void* x; int64_t ldx;
   const void* V; const void* U; const void* S;
+  const f16* u_scales; const f16* v_scales;      // quantized weights only
   void* out; int64_t ldo;
   int M, b, P, R, Q;
   int64_t s_si, s_sj, s_sr;
@@ -66,11 +67,20 @@ __device__ __forceinline__ void st_tag(unsigned long long* p, float v, unsigned 
                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <typename T>
-__device__ __forceinline__ void cvt8(const u32x4& r, float (&w)[8]) {
-  typename TypeTraits<T>::vec8 v = __builtin_bit_cast(typename TypeTraits<T>::vec8, r);
+// 16 bytes of weights -> fp32: 8 two-byte elements, 16 int8 codes or 32 int4 codes (low nibble first).
+template <typename T, int WB>
+__device__ __forceinline__ void cvtw(const u32x4& r, float (&w)[128 / WB]) {
+  if constexpr (WB == 16) {
+    typename TypeTraits<T>::vec8 v = __builtin_bit_cast(typename TypeTraits<T>::vec8, r);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) w[e] = TypeTraits<T>::to_f32(v[e]);
+    for (int e = 0; e < 8; ++e) w[e] = TypeTraits<T>::to_f32(v[e]);
+  } else if constexpr (WB == 8) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) w[e] = (float)(int8_t)((r[e >> 2] >> ((e & 3) * 8)) & 0xFF);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 32; ++e) w[e] = (float)(((int32_t)(r[e >> 3] << (28 - 4 * (e & 7)))) >> 28);
+  }
 }
 // 16-byte streaming load through a buffer descriptor that spans the whole factor: the per-lane
 // byte offset sits in one register, the per-load row offset is uniform (scalar), and a row past
@@ -84,21 +94,21 @@ __device__ __forceinline__ u32x4 ldw16(__amdgpu_buffer_rsrc_t r, uint32_t voff, 
 
 // Sum of the row slots of a wave, then of the four waves; thread `col` < NC ends up with the
 // total of column `col` for each of the MT rows (returned through `tot`, valid for tid < NC).
-template <int MT>
-__device__ __forceinline__ void wg_reduce(float (&acc)[MT][8], int lpr, int cv, float* red, int NC, float (&tot)[MT][2]) {
+template <int MT, int EPL>
+__device__ __forceinline__ void wg_reduce(float (&acc)[MT][EPL], int lpr, int cv, float* red, int NC, float (&tot)[MT][2]) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int o = lpr; o < 64; o <<= 1) {
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[m][e] += __shfl_xor(acc[m][e], o, 64);
+      for (int e = 0; e < EPL; ++e) acc[m][e] += __shfl_xor(acc[m][e], o, 64);
   }
   __syncthreads();
   if (lane < lpr) {
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) red[(wave * MT + m) * D2_NC_MAX + cv * 8 + e] = acc[m][e];
+      for (int e = 0; e < EPL; ++e) red[(wave * MT + m) * D2_NC_MAX + cv * EPL + e] = acc[m][e];
   }
   __syncthreads();
 #pragma unroll
@@ -138,9 +148,10 @@ __device__ __forceinline__ void finish_epoch(const Decode2Params& p, unsigned ep
   }
 }
 
-template <typename T, int MT>
+template <typename T, int MT, int WB>
 __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
-  constexpr int D2_PF = d2_pf(MT);
+  constexpr int EPL = 128 / WB;                      // weights per 16-byte load
+  constexpr int D2_PF = d2_pf(MT, WB);
   constexpr int D2_UNR1 = d2_unr1(MT);
   constexpr int D2_KS1_MAX = d2_ks1_max(MT);
   __shared__ float a_s[D2_AS];
@@ -165,13 +176,13 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   const int i2 = t2 % p.b, ksi2 = t2 / p.b;
   const int k0_2 = ksi2 * p.kc2;
   const int kcur2 = min(p.kc2, p.R - k0_2);
-  const int NC2 = lpr2 * 8;
+  const int NC2 = lpr2 * EPL;
   const int n0_2 = nc2 * NC2;
-  const int n2 = n0_2 + cv2 * 8;
+  const int n2 = n0_2 + cv2 * EPL;
   const bool col_ok2 = n2 < p.Q;
-  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.b * p.R * p.Q * 2u);
-  const uint32_t uoff = (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs2) * p.Q + (col_ok2 ? n2 : 0)) * 2);   // bytes, row rs2 of the slab
-  const uint32_t ustep = (uint32_t)rpp2 * p.Q * 2u;                                                       // bytes between a lane's loads
+  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)((int64_t)p.b * p.R * p.Q * WB / 8));
+  const uint32_t uoff = (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs2) * p.Q + (col_ok2 ? n2 : 0)) * WB / 8);   // bytes, row rs2 of the slab
+  const uint32_t ustep = (uint32_t)((int64_t)rpp2 * p.Q * WB / 8);                                            // bytes between a lane's loads
 
   u32x4 pf[D2_PF];                                   // only slots below pfn are ever read after the prefetch
   auto issue_prefetch = [&]() {
@@ -221,12 +232,12 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     const int t1 = w / p.nch1;
     const int j = t1 % p.b, ks = t1 / p.b;
     const int k0 = ks * p.kc1, kc = min(p.kc1, p.P - k0);
-    const int NC1 = lpr1 * 8;
-    const int n0 = nc1 * NC1, n = n0 + cv1 * 8;
+    const int NC1 = lpr1 * EPL;
+    const int n0 = nc1 * NC1, n = n0 + cv1 * EPL;
     const bool col_ok = n < p.R;
-    const __amdgpu_buffer_rsrc_t vbuf = wbuf(p.V, (uint32_t)p.b * p.P * p.R * 2u);
-    const uint32_t voff = (uint32_t)((((int64_t)j * p.P + k0 + rs1) * p.R + (col_ok ? n : 0)) * 2);
-    const uint32_t vstep = (uint32_t)rpp1 * p.R * 2u;
+    const __amdgpu_buffer_rsrc_t vbuf = wbuf(p.V, (uint32_t)((int64_t)p.b * p.P * p.R * WB / 8));
+    const uint32_t voff = (uint32_t)((((int64_t)j * p.P + k0 + rs1) * p.R + (col_ok ? n : 0)) * WB / 8);
+    const uint32_t vstep = (uint32_t)((int64_t)rpp1 * p.R * WB / 8);
 
     // Batches are always full: rows past the end of the slice meet a zero activation.
     const int nbatch = ((kc + rpp1 - 1) / rpp1 + D2_UNR1 - 1) / D2_UNR1;
@@ -259,22 +270,22 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     check_in();
     __syncthreads();
 
-    float acc[MT][8];
+    float acc[MT][EPL];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[m][e] = 0.0f;
+      for (int e = 0; e < EPL; ++e) acc[m][e] = 0.0f;
     for (int bi = 0; bi < nbatch; ++bi) {
 #pragma unroll
       for (int u = 0; u < D2_UNR1; ++u) {
-        float wv[8];
-        cvt8<T>(raw[u], wv);
+        float wv[EPL];
+        cvtw<T, WB>(raw[u], wv);
         const int k = rs1 + (bi * D2_UNR1 + u) * rpp1;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
           const float a = a_s[m * KLD + k];            // zero beyond the slice
 #pragma unroll
-          for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
+          for (int e = 0; e < EPL; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
         }
       }
       if (bi + 1 < nbatch) {                           // deeper slices than one batch (the planner avoids them)
@@ -286,14 +297,15 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     TR2(1);
 
     float tot[MT][2];
-    wg_reduce<MT>(acc, lpr1, cv1, red, NC1, tot);
+    wg_reduce<MT, EPL>(acc, lpr1, cv1, red, NC1, tot);
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int col = tid + h * 256;
       if (col < NC1 && n0 + col < p.R) {
+        const float vsc = (WB != 16) ? (float)p.v_scales[(int64_t)j * p.R + n0 + col] : 1.0f;   // per-rank scale of the codes of V
 #pragma unroll
         for (int m = 0; m < MT; ++m)
-          if (m < M) st_tag(&p.ypart[(((int64_t)ks * p.b + j) * M + m) * p.R + n0 + col], tot[m][h], epoch);
+          if (m < M) st_tag(&p.ypart[(((int64_t)ks * p.b + j) * M + m) * p.R + n0 + col], tot[m][h] * vsc, epoch);
       }
     }
     TR2(2);
@@ -423,22 +435,22 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   TR2(4);
 
   // ---- stage 2: out[m, i Q + n] = sum_k z[m][k] U_i[k, n] ---------------------------------------
-  float acc[MT][8];
+  float acc[MT][EPL];
 #pragma unroll
   for (int m = 0; m < MT; ++m)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[m][e] = 0.0f;
+    for (int e = 0; e < EPL; ++e) acc[m][e] = 0.0f;
 #pragma unroll
   for (int u = 0; u < D2_PF; ++u) {
     const int k = rs2 + u * rpp2;
     if (u < p.pfn) {
-      float wv[8];
-      cvt8<T>(pf[u], wv);
+      float wv[EPL];
+      cvtw<T, WB>(pf[u], wv);
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         const float a = a_s[m * KLD + k];              // zero beyond the slice
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
+        for (int e = 0; e < EPL; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -454,21 +466,21 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
         raw[u] = ldw16(ubuf, uoff, (uint32_t)(p.pfn + bi * D2_UNR + u) * ustep);
 #pragma unroll
       for (int u = 0; u < D2_UNR; ++u) {
-        float wv[8];
-        cvt8<T>(raw[u], wv);
+        float wv[EPL];
+        cvtw<T, WB>(raw[u], wv);
         const int k = rs2 + (p.pfn + bi * D2_UNR + u) * rpp2;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
           const float a = a_s[m * KLD + k];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
+          for (int e = 0; e < EPL; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
         }
       }
     }
   }
   TR2(5);
   float tot[MT][2];
-  wg_reduce<MT>(acc, lpr2, cv2, red, NC2, tot);
+  wg_reduce<MT, EPL>(acc, lpr2, cv2, red, NC2, tot);
   TR2(6);
   T* outp = reinterpret_cast<T*>(p.out);
 #pragma unroll
@@ -500,6 +512,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
               }
               v += __uint_as_float((unsigned)pv);
             }
+            if (WB != 16) v *= (float)p.u_scales[(int64_t)i2 * p.Q + gn];                      // per-output scale of the codes of U
             outp[(int64_t)m * p.ldo + (int64_t)i2 * p.Q + gn] = TypeTraits<T>::from_f32(v);
           }
         }
@@ -908,13 +921,19 @@ int env_i(const char* name, int dflt) {
 }
 int ilog2(int v) { int l = 0; while ((1 << l) < v) ++l; return l; }
 
-template <typename T>
-void* d2_kernel(int MT) {
+template <typename T, int WB>
+void* d2_kernel_mt(int MT) {
   switch (MT) {
-    case 1: return (void*)decode2_kernel<T, 1>;
-    case 2: return (void*)decode2_kernel<T, 2>;
-    default: return (void*)decode2_kernel<T, 4>;
+    case 1: return (void*)decode2_kernel<T, 1, WB>;
+    case 2: return (void*)decode2_kernel<T, 2, WB>;
+    default: return (void*)decode2_kernel<T, 4, WB>;
   }
+}
+template <typename T>
+void* d2_kernel(int MT, int wbits) {
+  if (wbits == 8) return d2_kernel_mt<T, 8>(MT);
+  if (wbits == 4) return d2_kernel_mt<T, 4>(MT);
+  return d2_kernel_mt<T, 16>(MT);
 }
 
 }  // namespace
@@ -924,7 +943,9 @@ size_t decode2_region_bytes() { return (size_t)16 << 20; }
 bool decode2_applicable(const StreamBlastArgs& a) {
   static const int enabled = env_i("BLR_DECODE2", 1);
   if (!enabled || a.split) return false;
-  if (a.wbits != 16 || a.u_layout != BLR_U_RQ) return false;
+  if (a.u_layout != BLR_U_RQ) return false;
+  if (a.wbits != 16 && (a.wbits != 8 && a.wbits != 4)) return false;
+  if (a.wbits != 16 && (a.M > 4 || !a.u_scales || !a.v_scales)) return false;   // the matrix-core variant takes two-byte weights only
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
   if (a.M < 1 || a.M > 16) return false;
   const int P = a.in_f / a.b, Q = a.out_f / a.b;
@@ -946,8 +967,9 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   if (M >= mfma_min_m) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
   if (M > 4) return 1;
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
+  const int WBITS = a.wbits, EPL = 128 / WBITS;  // weights per 16-byte load
   const int kc_cap = D2_AS / MT - 256;           // the kernels pad a slice up to 255 rows with zeros
-  void* fn = a.dtype == BLR_F16 ? d2_kernel<f16>(MT) : d2_kernel<bf16>(MT);
+  void* fn = a.dtype == BLR_F16 ? d2_kernel<f16>(MT, WBITS) : d2_kernel<bf16>(MT, WBITS);
 
   static std::mutex mu;
   static std::map<void*, int> occ_cache;
@@ -967,18 +989,21 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
 
   Decode2Params p = {};
   p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
+  p.u_scales = (const f16*)a.u_scales; p.v_scales = (const f16*)a.v_scales;
   p.M = M; p.b = b; p.P = P; p.R = R; p.Q = Q;
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
+  const int lpr_cap = D2_NC_MAX / EPL;           // widest column chunk the reduction buffer holds
 
-  // stage 1: column chunks of 8 * lpr1 ranks; k split only as far as needed to engage the chip
+  // stage 1: column chunks of EPL * lpr1 ranks; k split only as far as needed to engage the chip
   {
     static const int e_lpr = env_i("BLR_D2_LPR1", 16), e_ks = env_i("BLR_D2_KS1", 0);
-    int lpr = e_lpr;
-    const int vecs = (R + 7) / 8;
+    int lpr = e_lpr < lpr_cap ? e_lpr : lpr_cap;
+    const int vecs = (R + EPL - 1) / EPL;
     while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
     if (lpr > 64) lpr = 64;
+    if (lpr > lpr_cap) lpr = lpr_cap;
     if (lpr < 4) lpr = 4;
     const int rpp = 256 / lpr;
     const int nch = (vecs + lpr - 1) / lpr;
@@ -1004,8 +1029,8 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   // stage 2: column chunks of 8 * lpr2 outputs; k split so that the slabs cover the resident grid
   {
     static const int e_lpr = env_i("BLR_D2_LPR2", 16), e_ks = env_i("BLR_D2_KS2", 0), e_ksmax = env_i("BLR_D2_KS2_MAX", 4);
-    int lpr = e_lpr;
-    const int vecs = (Q + 7) / 8;
+    int lpr = e_lpr < lpr_cap ? e_lpr : lpr_cap;
+    const int vecs = (Q + EPL - 1) / EPL;
     while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
     if (lpr > 64) lpr = 64;
     if (lpr < 4) lpr = 4;
@@ -1024,7 +1049,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     ks = (R + kc - 1) / kc;
     if (base * ks > resident) return 1;
     int pfn = (kc + rpp - 1) / rpp;
-    if (pfn > d2_pf(MT)) pfn = d2_pf(MT);
+    if (pfn > d2_pf(MT, WBITS)) pfn = d2_pf(MT, WBITS);
     const int left = (kc + rpp - 1) / rpp - pfn;     // loads per lane beyond the register-resident ones
     const int kpad2 = (pfn + (left > 0 ? (left + D2_UNR - 1) / D2_UNR * D2_UNR : 0)) * rpp;
     if (kpad2 > D2_AS / MT) return 1;
