@@ -107,6 +107,7 @@ struct StreamBlastArgs {
   const void* u_scales; const void* v_scales;   // quantized only (fp16)
   void* out; int64_t ldo;
   int M, in_f, out_f, b, r;
+  int bo;                                       // output blocks when they differ from b (0: same); S may then be null (all ones)
   int dtype, u_layout, s_layout;
   int wbits;                                    // 16 = floating weights, 8 / 4 = codes
   void* ws; size_t ws_bytes;

@@ -16,6 +16,7 @@
 // in; the last one to check in advances it for the next call, which is safe because by then
 // every workgroup of this call holds its own copy.  Tag 0 is never used, so a zero-filled
 // workspace holds no valid pair.  Calls that share a workspace must be ordered on one stream.
+#include <cstdio>
 #include <cstdlib>
 #include <map>
 #include <mutex>
@@ -48,7 +49,8 @@ struct Decode2Params {
   const void* V; const void* U; const void* S;
   const f16* u_scales; const f16* v_scales;      // quantized weights only
   void* out; int64_t ldo;
-  int M, b, P, R, Q;
+  int zrep;                                      // bo == 1: z is published in zrep copies so that the slabs do not all poll one address range
+  int M, b, bo, P, R, Q;                         // b blocks of the input (stage 1), bo blocks of the output (stage 2)
   int64_t s_si, s_sj, s_sr;
   int lpr1_log2, nch1, ks1, kc1, items1;
   int lpr2_log2, nch2, ks2, kc2, items2, pfn, kpad2;
@@ -173,14 +175,15 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   const int cv2 = tid & (lpr2 - 1), rs2 = tid >> p.lpr2_log2;
   const int nc2 = has2 ? item2 % p.nch2 : 0;
   const int t2 = has2 ? item2 / p.nch2 : 0;
-  const int i2 = t2 % p.b, ksi2 = t2 / p.b;
+  const int i2 = t2 % p.bo, ksi2 = t2 / p.bo;
+  const int zi = p.zrep > 1 ? nc2 % p.zrep : i2;     // which published copy of z this slab reads
   const int k0_2 = ksi2 * p.kc2;
   const int kcur2 = min(p.kc2, p.R - k0_2);
   const int NC2 = lpr2 * EPL;
   const int n0_2 = nc2 * NC2;
   const int n2 = n0_2 + cv2 * EPL;
   const bool col_ok2 = n2 < p.Q;
-  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)((int64_t)p.b * p.R * p.Q * WB / 8));
+  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)((int64_t)p.bo * p.R * p.Q * WB / 8));
   const uint32_t uoff = (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs2) * p.Q + (col_ok2 ? n2 : 0)) * WB / 8);   // bytes, row rs2 of the slab
   const uint32_t ustep = (uint32_t)((int64_t)rpp2 * p.Q * WB / 8);                                            // bytes between a lane's loads
 
@@ -207,12 +210,12 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   // S(i = g, j = u, r) for this thread's (g, r); indices are clamped so that every load is legal.
   float sv[16];
   if (w < p.itemsM) {
-    const int g = min(tid >> p.rch_log2, p.b - 1);
+    const int g = min(tid >> p.rch_log2, p.bo - 1);   // (replicas of a single output block all use S of block 0)
     const int r = min(w * (1 << p.rch_log2) + (tid & ((1 << p.rch_log2) - 1)), p.R - 1);
     const T* Sp = reinterpret_cast<const T*>(p.S);
 #pragma unroll
     for (int u = 0; u < 16; ++u)
-      sv[u] = TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]);
+      sv[u] = Sp ? TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]) : 1.0f;
   }
 
   // Check-in: once the epoch has arrived this workgroup counts itself (no value comes back, so nothing
@@ -321,7 +324,8 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     const int RCH = 1 << p.rch_log2;
     const int g = tid >> p.rch_log2, rr = tid & (RCH - 1);
     const int r = w * RCH + rr;
-    const bool live = g < p.b && r < p.R;
+    const bool live = g < p.b && r < p.R;              // fetches y of input block g
+    const bool live_o = g < (p.zrep > 1 ? p.zrep : p.bo) && r < p.R;   // emits z of output block (or replica) g
     const T* Sp = reinterpret_cast<const T*>(p.S);
     float ysum[MT];
 #pragma unroll
@@ -358,7 +362,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) a_s[m * 256 + tid] = ysum[m];     // [m][j][rr]
     __syncthreads();
-    if (live) {
+    if (live_o) {
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         if (m < M) {
@@ -366,7 +370,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
 #pragma unroll
           for (int u = 0; u < 16; ++u) z = fmaf((u < p.b) ? sv[u] : 0.0f, a_s[m * 256 + min(u, p.b - 1) * RCH + rr], z);
           for (int j = 16; j < p.b; ++j)
-            z = fmaf(TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)j * p.s_sj + (int64_t)r * p.s_sr]), a_s[m * 256 + j * RCH + rr], z);
+            z = fmaf(Sp ? TypeTraits<T>::to_f32(Sp[(int64_t)min(g, p.bo - 1) * p.s_si + (int64_t)j * p.s_sj + (int64_t)r * p.s_sr]) : 1.0f, a_s[m * 256 + j * RCH + rr], z);
           st_tag(&p.zt[((int64_t)g * M + m) * p.R + r], z, epoch);
         }
       }
@@ -400,7 +404,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
           const int idx = base + u * 256 + tid;
           if (idx < total) {
             const int m = idx / pairs, kp = idx - m * pairs;
-            const uint32_t off = (uint32_t)((((int64_t)i2 * M + m) * p.R + k0_2 + 2 * kp) * 8);
+            const uint32_t off = (uint32_t)((((int64_t)zi * M + m) * p.R + k0_2 + 2 * kp) * 8);
             v[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(zr, off, 0, 17));
             ok = ok && v[u][1] == epoch && v[u][3] == epoch;
           } else {
@@ -491,14 +495,14 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
       if (ksi2 != 0) {                                // a producer of partial sums
 #pragma unroll
         for (int m = 0; m < MT; ++m)
-          if (m < M) st_tag(&p.opart[(((int64_t)(ksi2 - 1) * p.b + i2) * M + m) * p.Q + gn], tot[m][h], epoch);
+          if (m < M) st_tag(&p.opart[(((int64_t)(ksi2 - 1) * p.bo + i2) * M + m) * p.Q + gn], tot[m][h], epoch);
       } else {                                        // the slab of k-slice 0 adds the others in order
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
           if (m < M) {
             float v = tot[m][h];
             for (int ks = 1; ks < p.ks2; ++ks) {
-              const unsigned long long* src = &p.opart[(((int64_t)(ks - 1) * p.b + i2) * M + m) * p.Q + gn];
+              const unsigned long long* src = &p.opart[(((int64_t)(ks - 1) * p.bo + i2) * M + m) * p.Q + gn];
               unsigned long long pv;
               unsigned spins = 0;
               while (true) {
@@ -581,13 +585,14 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   const bool has2 = item2 < p.items2;
   const int nc2 = has2 ? item2 % p.nch2 : 0;
   const int t2 = has2 ? item2 / p.nch2 : 0;
-  const int i2 = t2 % p.b, ksi2 = t2 / p.b;
+  const int i2 = t2 % p.bo, ksi2 = t2 / p.bo;
+  const int zi = p.zrep > 1 ? nc2 % p.zrep : i2;     // which published copy of z this slab reads
   const int k0_2 = ksi2 * p.kc2;
   const int kcur2 = min(p.kc2, p.R - k0_2);
   const int n0_2 = nc2 * 128;
   const int n2 = n0_2 + cv * 8;
   const bool col_ok2 = n2 < p.Q;
-  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.b * p.R * p.Q * 2u);
+  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.bo * p.R * p.Q * 2u);
   const uint32_t uoff = (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs * 8) * p.Q + (col_ok2 ? n2 : 0)) * 2);
   const uint32_t urow = (uint32_t)p.Q * 2u;
   u32x4 pf[DM_PF];
@@ -628,12 +633,12 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   const int nrc = (p.R + (1 << p.rch_log2) - 1) >> p.rch_log2;
   float sv[16];
   if (w < p.itemsM) {
-    const int g = min(tid >> p.rch_log2, p.b - 1);
+    const int g = min(tid >> p.rch_log2, p.bo - 1);   // (replicas of a single output block all use S of block 0)
     const int r = min((w % nrc) * (1 << p.rch_log2) + (tid & ((1 << p.rch_log2) - 1)), p.R - 1);
     const T* Sp = reinterpret_cast<const T*>(p.S);
 #pragma unroll
     for (int u = 0; u < 16; ++u)
-      sv[u] = TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]);
+      sv[u] = Sp ? TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]) : 1.0f;
   }
 
   // ---- stage 1 -----------------------------------------------------------------------------------
@@ -716,7 +721,8 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     const int g = tid >> p.rch_log2, rr = tid & (RCH - 1);
     const int r = (w % nrc) * RCH + rr;
     const int mbase = (w / nrc) * DM_MC;
-    const bool live = g < p.b && r < p.R;
+    const bool live = g < p.b && r < p.R;              // fetches y of input block g
+    const bool live_o = g < (p.zrep > 1 ? p.zrep : p.bo) && r < p.R;   // emits z of output block (or replica) g
     const T* Sp = reinterpret_cast<const T*>(p.S);
     float ysum[DM_MC];
 #pragma unroll
@@ -756,14 +762,14 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
     for (int m = 0; m < DM_MC; ++m) {
       float z = 0.0f;
-      if (live) {
+      if (live_o) {
 #pragma unroll
         for (int u = 0; u < 16; ++u) z = fmaf((u < p.b) ? sv[u] : 0.0f, ys[m * 256 + min(u, p.b - 1) * RCH + rr], z);
         for (int jx = 16; jx < p.b; ++jx)
-          z = fmaf(TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)jx * p.s_sj + (int64_t)r * p.s_sr]), ys[m * 256 + jx * RCH + rr], z);
+          z = fmaf(Sp ? TypeTraits<T>::to_f32(Sp[(int64_t)min(g, p.bo - 1) * p.s_si + (int64_t)jx * p.s_sj + (int64_t)r * p.s_sr]) : 1.0f, ys[m * 256 + jx * RCH + rr], z);
       }
       const float zn = __shfl_down(z, 1, 64);                    // rank r + 1 (same i: RCH is even)
-      if (live && (rr & 1) == 0 && mbase + m < M) {
+      if (live_o && (rr & 1) == 0 && mbase + m < M) {
         const unsigned long long v = ((unsigned long long)epoch << 32) | pack2<T>(z, (r + 1 < p.R) ? zn : 0.0f);
         __hip_atomic_store(&p.zt[((int64_t)g * M + mbase + m) * (p.R >> 1) + (r >> 1)], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
@@ -795,7 +801,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
           const int idx = base + u * 256 + tid;
           if (idx < total) {
             const int m = idx / quads, kq = idx - m * quads;
-            const uint32_t off = (uint32_t)((((int64_t)i2 * M + m) * (p.R >> 1) + ((k0_2 + 4 * kq) >> 1)) * 8);
+            const uint32_t off = (uint32_t)((((int64_t)zi * M + m) * (p.R >> 1) + ((k0_2 + 4 * kq) >> 1)) * 8);
             v[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(zr, off, 0, 17));
             ok = ok && v[u][1] == epoch && v[u][3] == epoch;
           } else {
@@ -856,7 +862,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
         const int gn = n0_2 + col + 4 * h;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (gn < p.Q && m0 + i < M) st_tag(&p.opart[(((int64_t)(ksi2 - 1) * p.b + i2) * M + m0 + i) * p.Q + gn], vh[h][i], epoch);
+          if (gn < p.Q && m0 + i < M) st_tag(&p.opart[(((int64_t)(ksi2 - 1) * p.bo + i2) * M + m0 + i) * p.Q + gn], vh[h][i], epoch);
       }
       return;
     }
@@ -878,7 +884,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               if (ks < p.ks2 && gn < p.Q && m0 + i < M) {
-                pv[ks - 1][h][i] = ld_tag(&p.opart[(((int64_t)(ks - 1) * p.b + i2) * M + m0 + i) * p.Q + gn]);
+                pv[ks - 1][h][i] = ld_tag(&p.opart[(((int64_t)(ks - 1) * p.bo + i2) * M + m0 + i) * p.Q + gn]);
                 ok = ok && ((unsigned)(pv[ks - 1][h][i] >> 32) == epoch);
               } else {
                 pv[ks - 1][h][i] = 0ull;
@@ -919,6 +925,12 @@ int env_i(const char* name, int dflt) {
   const char* e = getenv(name);
   return e ? atoi(e) : dflt;
 }
+// "this shape is not for me": 1, with the place reported when BLR_D2_DEBUG is set
+int d2_bail(int line) {
+  static const int dbg = env_i("BLR_D2_DEBUG", 0);
+  if (dbg) fprintf(stderr, "decode2: falling back (blr_decode.hip:%d)\n", line);
+  return 1;
+}
 int ilog2(int v) { int l = 0; while ((1 << l) < v) ++l; return l; }
 
 template <typename T, int WB>
@@ -948,7 +960,7 @@ bool decode2_applicable(const StreamBlastArgs& a) {
   if (a.wbits != 16 && (a.M > 4 || !a.u_scales || !a.v_scales)) return false;   // the matrix-core variant takes two-byte weights only
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
   if (a.M < 1 || a.M > 16) return false;
-  const int P = a.in_f / a.b, Q = a.out_f / a.b;
+  const int P = a.in_f / a.b, Q = a.out_f / (a.bo > 0 ? a.bo : a.b);
   if (a.r % 8 || Q % 8 || P < 1) return false;
   if (!aligned(a.U, 16) || !aligned(a.V, 16)) return false;
   if ((int64_t)a.r * a.out_f * 2 >= (1ll << 31) || (int64_t)a.r * a.in_f * 2 >= (1ll << 31)) return false;   // 32-bit buffer offsets
@@ -962,10 +974,11 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
 // words on separate cache lines (epoch, arrivals, error).
 int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
                          unsigned* err_word, hipStream_t st) {
-  const int P = a.in_f / a.b, Q = a.out_f / a.b, R = a.r, b = a.b, M = a.M;
+  const int bo = a.bo > 0 ? a.bo : a.b;
+  const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
   static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
   if (M >= mfma_min_m) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
-  if (M > 4) return 1;
+  if (M > 4) return d2_bail(__LINE__);
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int WBITS = a.wbits, EPL = 128 / WBITS;  // weights per 16-byte load
   const int kc_cap = D2_AS / MT - 256;           // the kernels pad a slice up to 255 rows with zeros
@@ -990,7 +1003,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   Decode2Params p = {};
   p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
   p.u_scales = (const f16*)a.u_scales; p.v_scales = (const f16*)a.v_scales;
-  p.M = M; p.b = b; p.P = P; p.R = R; p.Q = Q;
+  p.M = M; p.b = b; p.bo = bo; p.P = P; p.R = R; p.Q = Q;
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
@@ -1008,7 +1021,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     const int rpp = 256 / lpr;
     const int nch = (vecs + lpr - 1) / lpr;
     const int base = b * nch;
-    if (base > resident) return 1;
+    if (base > resident) return d2_bail(__LINE__);
     // split k just far enough that a lane's share of a slice is one batch of loads
     const int ks_max = d2_ks1_max(MT);
     int ks = e_ks > 0 ? e_ks : ((P + rpp - 1) / rpp + d2_unr1(MT) - 1) / d2_unr1(MT);
@@ -1019,11 +1032,11 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     int kc = (P + ks - 1) / ks;
     kc = (kc + rpp - 1) / rpp * rpp;
     if (kc > kc_cap) kc = kc_cap / rpp * rpp;
-    if (kc < 1) return 1;
+    if (kc < 1) return d2_bail(__LINE__);
     ks = (P + kc - 1) / kc;
-    if (ks > ks_max || base * ks > resident) return 1;
+    if (ks > ks_max || base * ks > resident) return d2_bail(__LINE__);
     const int unr1 = d2_unr1(MT);
-    if (((kc + rpp - 1) / rpp + unr1 - 1) / unr1 * unr1 * rpp > D2_AS / MT) return 1;   // zero padding must fit too
+    if (((kc + rpp - 1) / rpp + unr1 - 1) / unr1 * unr1 * rpp > D2_AS / MT) return d2_bail(__LINE__);   // zero padding must fit too
     p.lpr1_log2 = ilog2(lpr); p.nch1 = nch; p.ks1 = ks; p.kc1 = kc; p.items1 = base * ks;
   }
   // stage 2: column chunks of 8 * lpr2 outputs; k split so that the slabs cover the resident grid
@@ -1036,8 +1049,8 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     if (lpr < 4) lpr = 4;
     const int rpp = 256 / lpr;
     const int nch = (vecs + lpr - 1) / lpr;
-    const int base = b * nch;
-    if (base > resident) return 1;
+    const int base = bo * nch;
+    if (base > resident) return d2_bail(__LINE__);
     int ks = e_ks > 0 ? e_ks : resident / base;
     if (ks > e_ksmax) ks = e_ksmax;
     if (ks > resident / base) ks = resident / base;
@@ -1045,30 +1058,31 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     int kc = (R + ks - 1) / ks;
     kc = (kc + rpp - 1) / rpp * rpp;
     if (kc > kc_cap) kc = kc_cap / rpp * rpp;
-    if (kc < 1) return 1;
+    if (kc < 1) return d2_bail(__LINE__);
     ks = (R + kc - 1) / kc;
-    if (base * ks > resident) return 1;
+    if (base * ks > resident) return d2_bail(__LINE__);
     int pfn = (kc + rpp - 1) / rpp;
     if (pfn > d2_pf(MT, WBITS)) pfn = d2_pf(MT, WBITS);
     const int left = (kc + rpp - 1) / rpp - pfn;     // loads per lane beyond the register-resident ones
     const int kpad2 = (pfn + (left > 0 ? (left + D2_UNR - 1) / D2_UNR * D2_UNR : 0)) * rpp;
-    if (kpad2 > D2_AS / MT) return 1;
+    if (kpad2 > D2_AS / MT) return d2_bail(__LINE__);
     p.lpr2_log2 = ilog2(lpr); p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn; p.kpad2 = kpad2;
   }
   {
+    p.zrep = bo == 1 ? 16 : 1;
     int bp2 = 1;
-    while (bp2 < b) bp2 <<= 1;
-    if (bp2 > 256) return 1;
+    while (bp2 < b || bp2 < bo || bp2 < p.zrep) bp2 <<= 1;
+    if (bp2 > 256) return d2_bail(__LINE__);
     const int rch = 256 / bp2;
     p.rch_log2 = ilog2(rch);
     p.itemsM = (R + rch - 1) / rch;
-    if (p.itemsM > resident) return 1;
+    if (p.itemsM > resident) return d2_bail(__LINE__);
     static const int e_depth = env_i("BLR_D2_PF_DEPTH", 4);
     p.pf_depth = e_depth;
   }
-  const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)b * M * R * 8, 256);
-  const size_t obytes = (size_t)(p.ks2 - 1) * b * M * Q * 8;
-  if (ybytes + zbytes + obytes > decode2_region_bytes()) return 1;
+  const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)(p.zrep > 1 ? p.zrep : bo) * M * R * 8, 256);
+  const size_t obytes = (size_t)(p.ks2 - 1) * bo * M * Q * 8;
+  if (ybytes + zbytes + obytes > decode2_region_bytes()) return d2_bail(__LINE__);
   p.ypart = reinterpret_cast<unsigned long long*>(region);
   p.zt = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes);
   p.opart = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes + zbytes);
@@ -1088,7 +1102,8 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
 // Matrix-core variant of the launch (any M <= 16).
 int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
                           unsigned* err_word, hipStream_t st) {
-  const int P = a.in_f / a.b, Q = a.out_f / a.b, R = a.r, b = a.b, M = a.M;
+  const int bo = a.bo > 0 ? a.bo : a.b;
+  const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
   void* fn = a.dtype == BLR_F16 ? (void*)decode2m_kernel<f16> : (void*)decode2m_kernel<bf16>;
   static std::mutex mu;
   static std::map<void*, int> occ_cache;
@@ -1105,18 +1120,18 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
   }
   const int cus = device_cus() > 0 ? device_cus() : 256;
   const int resident = (occ < 2 ? occ : 2) * cus;
-  if (R % 4) return 1;
+  if (R % 4) return d2_bail(__LINE__);
 
   Decode2Params p = {};
   p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
-  p.M = M; p.b = b; p.P = P; p.R = R; p.Q = Q;
+  p.M = M; p.b = b; p.bo = bo; p.P = P; p.R = R; p.Q = Q;
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
   {
     static const int e_ks = env_i("BLR_DM_KS1", 0);
     const int nch = (R + 127) / 128, base = b * nch;
-    if (base > resident) return 1;
+    if (base > resident) return d2_bail(__LINE__);
     int ks = e_ks > 0 ? e_ks : (P + DM_ROWS - 1) / DM_ROWS;       // one batch per slice if the grid allows
     if (ks > resident / base) ks = resident / base;
     if (ks > 4) ks = 4;
@@ -1125,15 +1140,15 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     kc = (kc + 7) / 8 * 8;
     if (kc > DM_KMAX) kc = DM_KMAX;
     ks = (P + kc - 1) / kc;
-    if (ks > 4 || base * ks > resident) return 1;
+    if (ks > 4 || base * ks > resident) return d2_bail(__LINE__);
     p.lpr1_log2 = 4; p.nch1 = nch; p.ks1 = ks; p.kc1 = kc; p.items1 = base * ks;
     // a slice of x may be fetched in 16-byte pieces if every piece is aligned and inside the row
     p.x_vec = aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0 && kc % 8 == 0;
   }
   {
     static const int e_ks = env_i("BLR_DM_KS2", 0), e_ksmax = env_i("BLR_DM_KS2_MAX", 4);
-    const int nch = (Q + 127) / 128, base = b * nch;
-    if (base > resident) return 1;
+    const int nch = (Q + 127) / 128, base = bo * nch;
+    if (base > resident) return d2_bail(__LINE__);
     int ks = e_ks > 0 ? e_ks : resident / base;
     if (ks > e_ksmax) ks = e_ksmax;
     if (ks > 4) ks = 4;
@@ -1143,26 +1158,27 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     kc = (kc + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
     if (kc > DM_KMAX) kc = DM_KMAX;
     ks = (R + kc - 1) / kc;
-    if (ks > 4 || base * ks > resident) return 1;
+    if (ks > 4 || base * ks > resident) return d2_bail(__LINE__);
     int pfn = (kc + DM_ROWS - 1) / DM_ROWS * 8;
     if (pfn > DM_PF) pfn = DM_PF;
     p.lpr2_log2 = 4; p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn;
     p.kpad2 = (kc + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
   }
   {
+    p.zrep = bo == 1 ? 16 : 1;
     int bp2 = 2;                                   // at least two ranks per mix thread row: z goes out in pairs
-    while (bp2 < b) bp2 <<= 1;
-    if (bp2 > 128) return 1;
+    while (bp2 < b || bp2 < bo || bp2 < p.zrep) bp2 <<= 1;
+    if (bp2 > 128) return d2_bail(__LINE__);
     const int rch = 256 / bp2;
     p.rch_log2 = ilog2(rch);
     p.itemsM = ((R + rch - 1) / rch) * ((M + DM_MC - 1) / DM_MC);
-    if (p.itemsM > resident) return 1;
+    if (p.itemsM > resident) return d2_bail(__LINE__);
     static const int e_depth = env_i("BLR_DM_PF_DEPTH", 4);
     p.pf_depth = e_depth;
   }
-  const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)b * M * (R / 2) * 8, 256);
-  const size_t obytes = (size_t)(p.ks2 - 1) * b * M * Q * 8;
-  if (ybytes + zbytes + obytes > decode2_region_bytes()) return 1;
+  const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)(p.zrep > 1 ? p.zrep : bo) * M * (R / 2) * 8, 256);
+  const size_t obytes = (size_t)(p.ks2 - 1) * bo * M * Q * 8;
+  if (ybytes + zbytes + obytes > decode2_region_bytes()) return d2_bail(__LINE__);
   p.ypart = reinterpret_cast<unsigned long long*>(region);
   p.zt = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes);
   p.opart = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes + zbytes);

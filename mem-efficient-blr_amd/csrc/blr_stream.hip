@@ -1256,6 +1256,23 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
   }
   if (a.op == 1) {                             // low rank: z = x A (in, r); out = z B (r, out)
     WsLayout w = ws_carve(a.ws, (size_t)a.M * a.r);
+    if (!a.split) {
+      // The two-stage decode kernel sees a low-rank layer as a BLAST layer with the input cut into
+      // blocks of rows of A, a single output block and S = 1.
+      int bi = 0;
+      for (int c = 16; c >= 2 && !bi; c >>= 1)
+        if (a.in_f % c == 0 && (a.in_f / c) % 8 == 0) bi = c;
+      if (bi) {
+        StreamBlastArgs bl = {};
+        bl.x = a.x; bl.ldx = a.ldx; bl.U = a.W2; bl.V = a.W1; bl.S = nullptr; bl.out = a.out; bl.ldo = a.ldo;
+        bl.M = a.M; bl.in_f = a.in_f; bl.out_f = a.out_f; bl.b = bi; bl.bo = 1; bl.r = a.r;
+        bl.dtype = a.dtype; bl.u_layout = BLR_U_RQ; bl.s_layout = BLR_S_IJR; bl.wbits = 16;
+        if (decode2_applicable(bl)) {
+          int rc = decode2_blast_launch(bl, w.d2, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
+          if (rc <= 0) return rc;
+        }
+      }
+    }
     p.ctrl = w.ctrl; p.nph = 2;
     PhaseDesc& d = p.ph[0];
     d.kind = PH_KN; d.wbits = 16; d.W = a.W1; d.ldw = a.r; d.batch = 1; d.K = a.in_f; d.N = a.r;
