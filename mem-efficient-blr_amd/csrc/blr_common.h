@@ -108,6 +108,8 @@ struct StreamBlastArgs {
   void* out; int64_t ldo;
   int M, in_f, out_f, b, r;
   int bo;                                       // output blocks when they differ from b (0: same); S may then be null (all ones)
+  int perm_per;                                 // > 0: Monarch - the mix is the permutation with this period, S is unused
+  int64_t out_bs, out_ns;                       // output strides of (block, column); out_ns == 0: blocked (bs = q, ns = 1)
   int dtype, u_layout, s_layout;
   int wbits;                                    // 16 = floating weights, 8 / 4 = codes
   void* ws; size_t ws_bytes;

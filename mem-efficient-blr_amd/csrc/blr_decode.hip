@@ -49,6 +49,7 @@ struct Decode2Params {
   const void* V; const void* U; const void* S;
   const f16* u_scales; const f16* v_scales;      // quantized weights only
   void* out; int64_t ldo;
+  int perm_per; int64_t o_bs, o_ns;              // Monarch permutation period; output strides of (block, column)
   int zrep;                                      // bo == 1: z is published in zrep copies so that the slabs do not all poll one address range
   int M, b, bo, P, R, Q;                         // b blocks of the input (stage 1), bo blocks of the output (stage 2)
   int64_t s_si, s_sj, s_sr;
@@ -324,7 +325,11 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     const int RCH = 1 << p.rch_log2;
     const int g = tid >> p.rch_log2, rr = tid & (RCH - 1);
     const int r = w * RCH + rr;
-    const bool live = g < p.b && r < p.R;              // fetches y of input block g
+    // Monarch: the "mix" is a permutation - z[l][r] is the single value y[r / per][l * per + r % per]
+    const bool perm = p.perm_per > 0;
+    const int yj = perm ? r / p.perm_per : g;
+    const int yr = perm ? g * p.perm_per + r % p.perm_per : r;
+    const bool live = (perm ? g < p.bo : g < p.b) && r < p.R;          // fetches y of input block yj
     const bool live_o = g < (p.zrep > 1 ? p.zrep : p.bo) && r < p.R;   // emits z of output block (or replica) g
     const T* Sp = reinterpret_cast<const T*>(p.S);
     float ysum[MT];
@@ -340,7 +345,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
 #pragma unroll
           for (int m = 0; m < MT; ++m) {
             if (ks < p.ks1 && m < M) {
-              yv[ks][m] = ld_tag(&p.ypart[(((int64_t)ks * p.b + g) * M + m) * p.R + r]);
+              yv[ks][m] = ld_tag(&p.ypart[(((int64_t)ks * p.b + yj) * M + m) * p.R + yr]);
               ok = ok && ((unsigned)(yv[ks][m] >> 32) == epoch);
             } else {
               yv[ks][m] = 0ull;
@@ -366,10 +371,10 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         if (m < M) {
-          float z = 0.0f;
+          float z = perm ? ysum[m] : 0.0f;
 #pragma unroll
-          for (int u = 0; u < 16; ++u) z = fmaf((u < p.b) ? sv[u] : 0.0f, a_s[m * 256 + min(u, p.b - 1) * RCH + rr], z);
-          for (int j = 16; j < p.b; ++j)
+          for (int u = 0; u < 16; ++u) z = fmaf((u < p.b && !perm) ? sv[u] : 0.0f, a_s[m * 256 + min(u, p.b - 1) * RCH + rr], z);
+          for (int j = 16; j < p.b && !perm; ++j)
             z = fmaf(Sp ? TypeTraits<T>::to_f32(Sp[(int64_t)min(g, p.bo - 1) * p.s_si + (int64_t)j * p.s_sj + (int64_t)r * p.s_sr]) : 1.0f, a_s[m * 256 + j * RCH + rr], z);
           st_tag(&p.zt[((int64_t)g * M + m) * p.R + r], z, epoch);
         }
@@ -517,7 +522,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
               v += __uint_as_float((unsigned)pv);
             }
             if (WB != 16) v *= (float)p.u_scales[(int64_t)i2 * p.Q + gn];                      // per-output scale of the codes of U
-            outp[(int64_t)m * p.ldo + (int64_t)i2 * p.Q + gn] = TypeTraits<T>::from_f32(v);
+            outp[(int64_t)m * p.ldo + (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns] = TypeTraits<T>::from_f32(v);
           }
         }
       }
@@ -721,7 +726,10 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     const int g = tid >> p.rch_log2, rr = tid & (RCH - 1);
     const int r = (w % nrc) * RCH + rr;
     const int mbase = (w / nrc) * DM_MC;
-    const bool live = g < p.b && r < p.R;              // fetches y of input block g
+    const bool perm = p.perm_per > 0;                  // Monarch: z[l][r] = y[r / per][l * per + r % per]
+    const int yj = perm ? r / p.perm_per : g;
+    const int yr = perm ? g * p.perm_per + r % p.perm_per : r;
+    const bool live = (perm ? g < p.bo : g < p.b) && r < p.R;          // fetches y of input block yj
     const bool live_o = g < (p.zrep > 1 ? p.zrep : p.bo) && r < p.R;   // emits z of output block (or replica) g
     const T* Sp = reinterpret_cast<const T*>(p.S);
     float ysum[DM_MC];
@@ -737,7 +745,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
           for (int m = 0; m < DM_MC; ++m) {
             if (ks < p.ks1 && mbase + m < M) {
-              yv[ks][m] = ld_tag(&p.ypart[(((int64_t)ks * p.b + g) * M + mbase + m) * p.R + r]);
+              yv[ks][m] = ld_tag(&p.ypart[(((int64_t)ks * p.b + yj) * M + mbase + m) * p.R + yr]);
               ok = ok && ((unsigned)(yv[ks][m] >> 32) == epoch);
             } else {
               yv[ks][m] = 0ull;
@@ -761,8 +769,8 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     __syncthreads();
 #pragma unroll
     for (int m = 0; m < DM_MC; ++m) {
-      float z = 0.0f;
-      if (live_o) {
+      float z = perm ? ysum[m] : 0.0f;
+      if (live_o && !perm) {
 #pragma unroll
         for (int u = 0; u < 16; ++u) z = fmaf((u < p.b) ? sv[u] : 0.0f, ys[m * 256 + min(u, p.b - 1) * RCH + rr], z);
         for (int jx = 16; jx < p.b; ++jx)
@@ -911,7 +919,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
       const int gn = n0_2 + col + 4 * h;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (gn < p.Q && m0 + i < M) outp[(int64_t)(m0 + i) * p.ldo + (int64_t)i2 * p.Q + gn] = TypeTraits<T>::from_f32(tot[h][i]);
+        if (gn < p.Q && m0 + i < M) outp[(int64_t)(m0 + i) * p.ldo + (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns] = TypeTraits<T>::from_f32(tot[h][i]);
     }
   });
   TR2(7);
@@ -1004,6 +1012,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
   p.u_scales = (const f16*)a.u_scales; p.v_scales = (const f16*)a.v_scales;
   p.M = M; p.b = b; p.bo = bo; p.P = P; p.R = R; p.Q = Q;
+  p.perm_per = a.perm_per; p.o_bs = a.out_ns ? a.out_bs : Q; p.o_ns = a.out_ns ? a.out_ns : 1;
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
@@ -1125,6 +1134,7 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
   Decode2Params p = {};
   p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
   p.M = M; p.b = b; p.bo = bo; p.P = P; p.R = R; p.Q = Q;
+  p.perm_per = a.perm_per; p.o_bs = a.out_ns ? a.out_bs : Q; p.o_ns = a.out_ns ? a.out_ns : 1;
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }

@@ -1293,6 +1293,20 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
   // Monarch: out1 = scatter(x_k w1_k); out = out1_l w2_l
   const int P = a.in_f / a.b, S = a.out_f / a.b, per = a.r / a.b;
   WsLayout w = ws_carve(a.ws, (size_t)a.b * a.M * a.r);
+  if (!a.split && a.w2_layout == BLR_W2_RS && a.b >= 2 && a.r % a.b == 0) {
+    // Two-stage decode kernel: a BLAST-shaped call whose mix is the Monarch permutation.
+    StreamBlastArgs bl = {};
+    bl.x = a.x; bl.ldx = a.ldx; bl.U = a.W2; bl.V = a.W1; bl.S = nullptr; bl.out = a.out; bl.ldo = a.ldo;
+    bl.M = a.M; bl.in_f = a.in_f; bl.out_f = a.out_f; bl.b = a.b; bl.bo = a.b; bl.r = a.r;
+    bl.dtype = a.dtype; bl.u_layout = BLR_U_RQ; bl.s_layout = BLR_S_IJR; bl.wbits = 16;
+    bl.perm_per = per;
+    if (a.out_order == BLR_OUT_INTERLEAVED) { bl.out_bs = 1; bl.out_ns = a.b; }
+    else { bl.out_bs = S; bl.out_ns = 1; }
+    if (decode2_applicable(bl)) {
+      int rc = decode2_blast_launch(bl, w.d2, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
+      if (rc <= 0) return rc;
+    }
+  }
   p.ctrl = w.ctrl; p.nph = 2;
   PhaseDesc& d = p.ph[0];
   d.kind = PH_KN; d.wbits = 16; d.W = a.W1; d.w_bs = (int64_t)P * a.r; d.ldw = a.r; d.batch = a.b; d.K = P; d.N = a.r;
