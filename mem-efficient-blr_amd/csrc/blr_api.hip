@@ -110,22 +110,37 @@ __global__ __launch_bounds__(256) void quant_cols_kernel(const T* __restrict__ w
 }
 
 // codes (rows, cols) -> T; scale index = (row / rows_per_scale_block) * cols + col when per_col, else row.
+// cols % 8 == 0: a thread expands 8 consecutive codes (8 or 4 bytes in, 16 bytes out).
 template <typename T>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ codes, const f16* __restrict__ scales,
                                                       T* __restrict__ out, int64_t rows, int64_t cols, int bits,
                                                       int per_col, int64_t rows_per_block) {
-  const int64_t total = rows * cols;
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+  using V8 = typename TypeTraits<T>::vec8;
+  const int64_t total = rows * cols / 8;
+  for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < total; v += (int64_t)gridDim.x * 256) {
+    const int64_t idx = v * 8;
     const int64_t row = idx / cols, col = idx - row * cols;
-    int code;
-    if (bits == 8) code = reinterpret_cast<const int8_t*>(codes)[idx];
-    else {
-      uint8_t byte = codes[idx >> 1];
-      int nib = (idx & 1) ? (byte >> 4) : (byte & 0xF);
-      code = nib > 7 ? nib - 16 : nib;
+    int c[8];
+    if (bits == 8) {
+      const u32x2 w = *reinterpret_cast<const u32x2*>(codes + idx);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) c[e] = (int)(int8_t)((w[e >> 2] >> ((e & 3) * 8)) & 0xFF);
+    } else {
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(codes + (idx >> 1));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) c[e] = ((int32_t)(w << (28 - 4 * e))) >> 28;
     }
-    const float sc = (float)scales[per_col ? (row / rows_per_block) * cols + col : row];
-    out[idx] = TypeTraits<T>::from_f32((float)code * sc);
+    V8 o;
+    if (per_col) {
+      const f16x8 sc = *reinterpret_cast<const f16x8*>(&scales[(row / rows_per_block) * cols + col]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = TypeTraits<T>::from_f32((float)c[e] * (float)sc[e]);
+    } else {
+      const float sc = (float)scales[row];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = TypeTraits<T>::from_f32((float)c[e] * sc);
+    }
+    *reinterpret_cast<V8*>(&out[idx]) = o;
   }
 }
 
@@ -238,9 +253,13 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
 // ---- quantized BLAST -----------------------------------------------------------------------------
 size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits) {
   if (M <= 0 || b <= 0 || r <= 0) return 0;
-  if (M <= 16) return stream_blast_workspace(M, in_f, out_f, b, r, bits);
-  // larger M: factors are expanded to two-byte values once per call, then the tiled kernels run
-  return align_up((size_t)r * out_f * 2, 256) + align_up((size_t)r * in_f * 2, 256) + 2 * align_up((size_t)b * M * r * 2, 256);
+  // M <= 4 streams the codes.  Above that the factors are expanded to two-byte values once per call
+  // ([kernel workspace][U][V]) and the two-byte kernels run: the matrix-core decode kernel up to 16 rows,
+  // the tiled kernels beyond.  Requests for the phase engine (BLR_ALGO_STREAM*) stream codes up to M = 16.
+  size_t s = stream_blast_workspace(M <= 16 ? M : 16, in_f, out_f, b, r, bits);
+  if (M <= 4) return s;
+  size_t sub = M <= 16 ? s : 2 * align_up((size_t)b * M * r * 2, 256);
+  return align_up(sub, 256) + align_up((size_t)r * out_f * 2, 256) + align_up((size_t)r * in_f * 2, 256);
 }
 
 int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void* u_scales,
@@ -257,13 +276,15 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   if (ldx < in_f || ldo < out_f) { set_error("blast_q: leading dimension too small"); return BLR_ERR_BAD_ARG; }
   if (!aligned(u_codes, 16) || !aligned(v_codes, 16)) { set_error("blast_q: code buffers must be 16-byte aligned"); return BLR_ERR_BAD_ARG; }
   hipStream_t st = (hipStream_t)stream;
-  if (M > 16) {
-    if (algo == BLR_ALGO_STREAM || algo == BLR_ALGO_STREAM_SPLIT) { set_error("blast_q: M=%d > 16 not served by the streaming kernel", M); return BLR_ERR_UNSUPPORTED; }
+  const bool phase_engine = algo == BLR_ALGO_STREAM || algo == BLR_ALGO_STREAM_SPLIT;
+  if (M > 16 && phase_engine) { set_error("blast_q: M=%d > 16 not served by the streaming kernel", M); return BLR_ERR_UNSUPPORTED; }
+  if (M > 4 && !phase_engine) {
     size_t need = blr_blast_q_workspace_bytes(M, in_f, out_f, b, r, bits);
     if (!ws || ws_bytes < need) { set_error("blast_q: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
-    char* wp = reinterpret_cast<char*>(ws);
+    const size_t sub = align_up(M <= 16 ? stream_blast_workspace(M, in_f, out_f, b, r, bits) : 2 * align_up((size_t)b * M * r * 2, 256), 256);
+    char* wp = reinterpret_cast<char*>(ws) + sub;
     void* Ud = wp; wp += align_up((size_t)r * out_f * 2, 256);
-    void* Vd = wp; wp += align_up((size_t)r * in_f * 2, 256);
+    void* Vd = wp;
     // both factors are (k, n)-ordered with one scale per column of their block: U (b, r, q), V (b, p, r)
     const int64_t urows = (int64_t)b * r, vrows = in_f, q = out_f / b;
     if (dtype == BLR_F16) {
@@ -275,7 +296,7 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
     }
     BLR_CHECK_LAUNCH("dequant");
     return blr_blast_fwd(x, ldx, Ud, Vd, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, BLR_U_RQ, BLR_S_RIJ,
-                         BLR_ALGO_TILED, wp, ws_bytes - (size_t)(wp - reinterpret_cast<char*>(ws)), stream);
+                         M <= 16 ? BLR_ALGO_STREAM : BLR_ALGO_TILED, ws, sub, stream);
   }
   StreamBlastArgs s = {};
   s.x = x; s.ldx = ldx; s.U = u_codes; s.V = v_codes; s.S = S; s.u_scales = u_scales; s.v_scales = v_scales;

@@ -214,9 +214,14 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     const int g = min(tid >> p.rch_log2, p.bo - 1);   // (replicas of a single output block all use S of block 0)
     const int r = min(w * (1 << p.rch_log2) + (tid & ((1 << p.rch_log2) - 1)), p.R - 1);
     const T* Sp = reinterpret_cast<const T*>(p.S);
+    if (Sp) {                                           // one uniform branch, then unconditional loads
 #pragma unroll
-    for (int u = 0; u < 16; ++u)
-      sv[u] = Sp ? TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]) : 1.0f;
+      for (int u = 0; u < 16; ++u)
+        sv[u] = TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < 16; ++u) sv[u] = 1.0f;
+    }
   }
 
   // Check-in: once the epoch has arrived this workgroup counts itself (no value comes back, so nothing
@@ -641,9 +646,14 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     const int g = min(tid >> p.rch_log2, p.bo - 1);   // (replicas of a single output block all use S of block 0)
     const int r = min((w % nrc) * (1 << p.rch_log2) + (tid & ((1 << p.rch_log2) - 1)), p.R - 1);
     const T* Sp = reinterpret_cast<const T*>(p.S);
+    if (Sp) {                                           // one uniform branch, then unconditional loads
 #pragma unroll
-    for (int u = 0; u < 16; ++u)
-      sv[u] = Sp ? TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]) : 1.0f;
+      for (int u = 0; u < 16; ++u)
+        sv[u] = TypeTraits<T>::to_f32(Sp[(int64_t)g * p.s_si + (int64_t)min(u, p.b - 1) * p.s_sj + (int64_t)r * p.s_sr]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < 16; ++u) sv[u] = 1.0f;
+    }
   }
 
   // ---- stage 1 -----------------------------------------------------------------------------------
