@@ -49,6 +49,7 @@ struct Decode2Params {
   const void* V; const void* U; const void* S;
   const f16* u_scales; const f16* v_scales;      // quantized weights only
   void* out; int64_t ldo;
+  int u_nk, rpw, kl_log2;                        // U (bo, q, r): rows of U per wave, log2 of the 16-byte loads per row and lane
   int perm_per; int64_t o_bs, o_ns;              // Monarch permutation period; output strides of (block, column)
   int zrep;                                      // bo == 1: z is published in zrep copies so that the slabs do not all poll one address range
   int M, b, bo, P, R, Q;                         // b blocks of the input (stage 1), bo blocks of the output (stage 2)
@@ -185,8 +186,15 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   const int n2 = n0_2 + cv2 * EPL;
   const bool col_ok2 = n2 < p.Q;
   const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)((int64_t)p.bo * p.R * p.Q * WB / 8));
-  const uint32_t uoff = (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs2) * p.Q + (col_ok2 ? n2 : 0)) * WB / 8);   // bytes, row rs2 of the slab
+  // U (bo, q, r) ("NK", two-byte weights only): a wave owns rpw consecutive rows of U_i, a lane 8 consecutive k
+  // of every 512; load u of a lane is row u >> kl_log2, piece u & (KL - 1).  No k-split, no partial sums.
+  const int nk_row0 = nc2 * 4 * p.rpw + (tid >> 6) * p.rpw;
+  const uint32_t uoff = p.u_nk ? (uint32_t)((((int64_t)i2 * p.Q + nk_row0) * p.R + (tid & 63) * 8) * 2)
+                               : (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs2) * p.Q + (col_ok2 ? n2 : 0)) * WB / 8);   // bytes, first load of this lane
   const uint32_t ustep = (uint32_t)((int64_t)rpp2 * p.Q * WB / 8);                                            // bytes between a lane's loads
+  auto u_soff = [&](int u) -> uint32_t {
+    return p.u_nk ? (uint32_t)(((u >> p.kl_log2) * p.R + (u & ((1 << p.kl_log2) - 1)) * 512) * 2) : (uint32_t)u * ustep;
+  };
 
   u32x4 pf[D2_PF];                                   // only slots below pfn are ever read after the prefetch
   auto issue_prefetch = [&]() {
@@ -202,7 +210,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
         else if (u >= 8 && p.pf_depth == 8) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
         else if (u >= 12 && p.pf_depth == 12) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
         else if (u >= 16 && p.pf_depth == 16) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
-        pf[u] = ldw16(ubuf, uoff, (uint32_t)u * ustep);
+        pf[u] = ldw16(ubuf, uoff, u_soff(u));
       }
     }
   };
@@ -447,6 +455,48 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   }
   __syncthreads();
   TR2(4);
+
+  if (p.u_nk) {
+    // ---- stage 2, U (bo, q, r): out[m, i Q + row] = sum_k z[m][k] U_i[row, k]; one wave per row, lanes along k ----
+    if constexpr (WB == 16) {
+      const int lane = tid & 63;
+      const int KL = 1 << p.kl_log2;
+      T* outp = reinterpret_cast<T*>(p.out);
+      float racc[MT];
+#pragma unroll
+      for (int m = 0; m < MT; ++m) racc[m] = 0.0f;
+#pragma unroll
+      for (int u = 0; u < D2_PF; ++u) {
+        if (u < p.pfn) {
+          float wv[8];
+          cvtw<T, 16>(pf[u], wv);
+          const int c = u & (KL - 1);
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            const f32x4 za = *reinterpret_cast<const f32x4*>(&a_s[m * KLD + c * 512 + lane * 8]);
+            const f32x4 zb = *reinterpret_cast<const f32x4*>(&a_s[m * KLD + c * 512 + lane * 8 + 4]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) racc[m] = fmaf(za[e], wv[e], racc[m]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) racc[m] = fmaf(zb[e], wv[4 + e], racc[m]);
+          }
+          if (c == KL - 1) {                               // the row is complete: add the 64 lanes, lane 0 stores
+            const int row = nk_row0 + (u >> p.kl_log2);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+              const float tot = wave_sum(racc[m]);
+              racc[m] = 0.0f;
+              if (lane == 0 && row < p.Q && row < (nc2 + 1) * 4 * p.rpw && m < M)
+                outp[(int64_t)m * p.ldo + (int64_t)i2 * p.o_bs + (int64_t)row * p.o_ns] = TypeTraits<T>::from_f32(tot);
+            }
+          }
+        }
+      }
+    }
+    TR2(7);
+    if (w == 0) finish_epoch(p, epoch, G);
+    return;
+  }
 
   // ---- stage 2: out[m, i Q + n] = sum_k z[m][k] U_i[k, n] ---------------------------------------
   float acc[MT][EPL];
@@ -973,7 +1023,8 @@ size_t decode2_region_bytes() { return (size_t)16 << 20; }
 bool decode2_applicable(const StreamBlastArgs& a) {
   static const int enabled = env_i("BLR_DECODE2", 1);
   if (!enabled || a.split) return false;
-  if (a.u_layout != BLR_U_RQ) return false;
+  static const int nk_on = env_i("BLR_D2_NK", 1);
+  if (a.u_layout != BLR_U_RQ && !(nk_on && a.u_layout == BLR_U_QR && a.wbits == 16 && a.M <= 4)) return false;
   if (a.wbits != 16 && (a.wbits != 8 && a.wbits != 4)) return false;
   if (a.wbits != 16 && (a.M > 4 || !a.u_scales || !a.v_scales)) return false;   // the matrix-core variant takes two-byte weights only
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
@@ -1058,6 +1109,20 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     if (((kc + rpp - 1) / rpp + unr1 - 1) / unr1 * unr1 * rpp > D2_AS / MT) return d2_bail(__LINE__);   // zero padding must fit too
     p.lpr1_log2 = ilog2(lpr); p.nch1 = nch; p.ks1 = ks; p.kc1 = kc; p.items1 = base * ks;
   }
+  if (a.u_layout == BLR_U_QR) {
+    // stage 2 on U (bo, q, r): a wave takes rpw rows, a lane 8 of every 512 k; everything a lane loads stays in registers
+    const int KL = (R + 511) / 512;
+    if (KL != 1 && KL != 2 && KL != 4 && KL != 8) return d2_bail(__LINE__);
+    if (KL * 512 * MT > D2_AS) return d2_bail(__LINE__);
+    const int pf_cap = d2_pf(MT, 16);
+    int rpw = (int)cdiv((int64_t)bo * Q, (int64_t)resident * 4);
+    if (rpw < 1) rpw = 1;
+    while ((int64_t)bo * cdiv(Q, 4 * rpw) > resident) ++rpw;
+    if (rpw * KL > pf_cap) return d2_bail(__LINE__);
+    p.u_nk = 1; p.rpw = rpw; p.kl_log2 = ilog2(KL);
+    p.lpr2_log2 = 4; p.nch2 = (int)cdiv(Q, 4 * rpw); p.ks2 = 1; p.kc2 = R; p.items2 = bo * p.nch2;
+    p.pfn = rpw * KL; p.kpad2 = KL * 512;
+  } else
   // stage 2: column chunks of 8 * lpr2 outputs; k split so that the slabs cover the resident grid
   {
     static const int e_lpr = env_i("BLR_D2_LPR2", 16), e_ks = env_i("BLR_D2_KS2", 0), e_ksmax = env_i("BLR_D2_KS2_MAX", 4);
