@@ -46,6 +46,11 @@ struct KcStage {
       p[i] = base + (int64_t)min(row0 + row, nrows - 1) * ld + kv;
     }
   }
+  // full tile, 16-byte friendly operand: no conditions, so the number of loads in flight is known statically
+  __device__ __forceinline__ void load_vec(Vals& r, int k0) const {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) r.v[i] = ldg16<V8>(p[i] + k0);
+  }
   __device__ __forceinline__ void load(Vals& r, int k0, int K, bool vec_ok, int tid) const {
     if (vec_ok && k0 + BK <= K) {
 #pragma unroll
@@ -98,6 +103,12 @@ struct KnStage {
       else gn = min(gn, ncols - 1);
       p[ps] = base + (int64_t)(kq * 4) * ld + gn;
     }
+  }
+  __device__ __forceinline__ void load_vec(Vals& r, int k0) const {
+#pragma unroll
+    for (int ps = 0; ps < NP; ++ps)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r.v[ps][i] = ldg16<V8>(p[ps] + (int64_t)(k0 + i) * ld);
   }
   __device__ __forceinline__ void load(Vals& r, int k0, int K, bool vec_ok, int tid) const {
     if (vec_ok && k0 + BK <= K) {
@@ -153,7 +164,8 @@ __device__ __forceinline__ int64_t epi_offset(const GemmArgs& g, int bt, int m, 
 }
 
 template <typename T, int BM, int BN, bool B_KN, int PD>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int a_vec, int b_vec, int c_vec) {
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int a_vec, int b_vec, int c_vec,
+                                                        int per_xcd, int group_m) {
   constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;    // 32x32 MFMA tiles per wave
   using V8 = typename TypeTraits<T>::vec8;
@@ -163,11 +175,21 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  // Tile order: consecutive workgroups walk down M for one N tile, so the weight tile they share
-  // stays hot in L2 / Infinity Cache while the activations stream past.
-  int tile = blockIdx.x;
-  int tm_i = tile % tiles_m, tn_i = tile / tiles_m;
-  const int bt = blockIdx.y;
+  // Tile order.  Workgroups are handed to the 8 XCDs round-robin by linear id and each XCD has its own
+  // L2, so the linear id is first turned into u = (id % 8) * per_xcd + id / 8: an XCD then works through a
+  // contiguous range of u.  u walks the tiles of a batch entry in strips of group_m row tiles, column by
+  // column, so the ~32 tiles an XCD has in flight form a roughly square patch of C and share their A and
+  // B tiles through that XCD's L2 instead of every XCD fetching every weight tile.
+  const int tiles = tiles_m * tiles_n;
+  int u = blockIdx.x;
+  if (per_xcd > 0) u = (u & 7) * per_xcd + (u >> 3);
+  if (u >= tiles * g.batch) return;
+  const int bt = u / tiles;
+  const int ut = u - bt * tiles;
+  const int strip = ut / (group_m * tiles_n);
+  const int rem = ut - strip * group_m * tiles_n;
+  const int gm_here = min(group_m, tiles_m - strip * group_m);
+  const int tm_i = strip * group_m + rem % gm_here, tn_i = rem / gm_here;
   const int m0 = tm_i * BM, n0 = tn_i * BN;
 
   const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)bt * g.sA;
@@ -185,64 +207,85 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
   KcStage<T, BM> sa;
   KcStage<T, BN> sb_kc;
   KnStage<T, BN> sb_kn;
-  // PD register sets of staged tiles: global loads run PD k-tiles ahead of the multiplication.
-  // One set measured fastest on MI355X (deeper prefetch only added register pressure).
+  // PD register sets of staged tiles: in the main loop the global loads run PD k-tiles ahead of the
+  // multiplication.  Every load of that loop is unconditional (tile indices past the end are clamped
+  // to the last full tile and fetched again for nothing), because a load under a condition makes the
+  // number of loads in flight unknown to the compiler, which then waits for all of them.
   typename KcStage<T, BM>::Vals ra[PD];
   typename KcStage<T, BN>::Vals rb_kc[B_KN ? 1 : PD];
   typename KnStage<T, BN>::Vals rb_kn[B_KN ? PD : 1];
 
   const int KT = (g.K + BK - 1) / BK;
+  const int KTm = (a_vec && b_vec) ? g.K / BK : 0;          // full tiles of 16-byte friendly operands
   sa.init(A, g.lda, m0, g.M, tid);
   if (B_KN) sb_kn.init(B, g.ldb, n0, g.N, tid, b_vec);
   else sb_kc.init(B, g.ldb, n0, g.N, tid);
-  auto load_tile = [&](int d, int t) {
-    sa.load(ra[d], t * BK, g.K, a_vec, tid);
-    if (B_KN) sb_kn.load(rb_kn[B_KN ? d : 0], t * BK, g.K, b_vec, tid);
-    else sb_kc.load(rb_kc[B_KN ? 0 : d], t * BK, g.K, b_vec, tid);
+  auto load_vec = [&](int d, int t) {
+    sa.load_vec(ra[d], t * BK);
+    if (B_KN) sb_kn.load_vec(rb_kn[B_KN ? d : 0], t * BK);
+    else sb_kc.load_vec(rb_kc[B_KN ? 0 : d], t * BK);
   };
   auto store_tile = [&](int d, Smem& dst) {
     sa.store(ra[d], dst.a, tid);
     if (B_KN) sb_kn.store(rb_kn[B_KN ? d : 0], dst.b, tid);
     else sb_kc.store(rb_kc[B_KN ? 0 : d], dst.b, tid);
   };
+  auto multiply = [&](Smem& cur) {
+    // fragments of step kk + 1 are fetched from LDS before the matrix instructions of step kk are issued
+    V8 af[2][TM], bf[2][TN];
+    auto frags = [&](int kk, int set) {
+      const int kof = kk * 16 + (lane >> 5) * 8;
 #pragma unroll
-  for (int d = 0; d < PD; ++d)
-    if (d < KT) load_tile(d, d);
-  store_tile(0, sm[0]);
-  __syncthreads();
-
-  for (int kt0 = 0; kt0 < KT; kt0 += PD) {
+      for (int i = 0; i < TM; ++i)
+        af[set][i] = *reinterpret_cast<const V8*>(&cur.a[wm * WM + i * 32 + (lane & 31)][kof]);
 #pragma unroll
-    for (int d = 0; d < PD; ++d) {
-      const int kt = kt0 + d;
-      if (kt < KT) {
-        Smem& cur = sm[kt & 1];
-        if (kt + PD < KT) load_tile(d, kt + PD);   // set d went to LDS one step ago: free again
-        // fragments of step kk + 1 are fetched from LDS before the matrix instructions of step kk are issued
-        V8 af[2][TM], bf[2][TN];
-        auto frags = [&](int kk, int set) {
-          const int kof = kk * 16 + (lane >> 5) * 8;
+      for (int j = 0; j < TN; ++j)
+        bf[set][j] = *reinterpret_cast<const V8*>(&cur.b[wn * WN + j * 32 + (lane & 31)][kof]);
+    };
+    frags(0, 0);
 #pragma unroll
-          for (int i = 0; i < TM; ++i)
-            af[set][i] = *reinterpret_cast<const V8*>(&cur.a[wm * WM + i * 32 + (lane & 31)][kof]);
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      if (kk + 1 < BK / 16) frags(kk + 1, (kk + 1) & 1);
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            bf[set][j] = *reinterpret_cast<const V8*>(&cur.b[wn * WN + j * 32 + (lane & 31)][kof]);
-        };
-        frags(0, 0);
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-          if (kk + 1 < BK / 16) frags(kk + 1, (kk + 1) & 1);
-#pragma unroll
-          for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = TypeTraits<T>::mfma32(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
-        }
-        if (kt + 1 < KT) store_tile((d + 1) % PD, sm[(kt + 1) & 1]);   // nobody reads that stage until the barrier
-        __syncthreads();
-      }
+        for (int j = 0; j < TN; ++j) acc[i][j] = TypeTraits<T>::mfma32(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
     }
+  };
+  // one step of the pipelined loop; d (which register set is free) is a constant after unrolling
+  auto step = [&](int kt, int d) {
+    load_vec(d, min(kt + PD, KTm - 1));                      // set d went to LDS one step ago
+    __builtin_amdgcn_sched_barrier(0);                       // keep the loads up here: the scheduler would sink them to their use
+    multiply(sm[kt & 1]);
+    store_tile((d + 1) % PD, sm[(kt + 1) & 1]);              // nobody reads that stage until the barrier
+    __syncthreads();
+  };
+  int kt = 0;
+  if (KTm > 0) {
+#pragma unroll
+    for (int d = 0; d < PD; ++d) load_vec(d, min(d, KTm - 1));
+    store_tile(0, sm[0]);
+    __syncthreads();
+    for (; kt + PD <= KTm; kt += PD) {
+#pragma unroll
+      for (int d = 0; d < PD; ++d) step(kt + d, d);
+    }
+#pragma unroll
+    for (int d = 0; d < PD - 1; ++d)
+      if (kt + d < KTm) step(kt + d, d);
+    kt = KTm;
   }
+  // what the pipelined loop does not take - a partial last tile, or every tile of operands that are
+  // not 16-byte friendly - goes one tile at a time through the guarded loads
+  for (; kt < KT; ++kt) {
+    sa.load(ra[0], kt * BK, g.K, a_vec, tid);
+    if (B_KN) sb_kn.load(rb_kn[0], kt * BK, g.K, b_vec, tid);
+    else sb_kc.load(rb_kc[0], kt * BK, g.K, b_vec, tid);
+    store_tile(0, sm[kt & 1]);
+    __syncthreads();
+    multiply(sm[kt & 1]);
+  }
+  __syncthreads();                                             // the epilogue reuses the LDS tiles
 
   // D fragment: element e of lane l is row (e/4)*8 + (l/32)*4 + e%4, column l%32.
   if (c_vec) {
@@ -339,8 +382,9 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) 
 template <typename T, int BM, int BN, bool B_KN>
 static void* mfma_kernel_ptr(int pd) {
   switch (pd) {
-    case 2: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 2>;
-    default: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 1>;
+    case 1: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 1>;
+    case 3: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 3>;
+    default: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 2>;
   }
 }
 
@@ -353,7 +397,7 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   int c_vec = g.epi == EPI_PLAIN && g.cn == 1 && aligned(g.C, 16) && g.ldc % 8 == 0 && g.sC % 8 == 0 && g.N % 8 == 0;
   size_t lds = 2 * sizeof(GemmSmem<T, BM, BN>);
   // k-tiles of global loads kept in flight (tuning aid: BLR_GEMM_PD = 1, 2 or 3)
-  static const int pd = [] { const char* e = getenv("BLR_GEMM_PD"); return e ? atoi(e) : 1; }();
+  static const int pd = [] { const char* e = getenv("BLR_GEMM_PD"); return e ? atoi(e) : 2; }();
   void* fn = g.b_kn ? mfma_kernel_ptr<T, BM, BN, true>(pd) : mfma_kernel_ptr<T, BM, BN, false>(pd);
   static std::mutex mu;
   static std::set<void*> raised;
@@ -365,9 +409,16 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
       raised.insert(fn);
     }
   }
-  dim3 grid(tiles_m * tiles_n, g.batch);
+  // tuning aids: BLR_GEMM_XCD=0 keeps the linear tile order, BLR_GEMM_GM sets the strip height in tiles
+  static const int xcd_on = [] { const char* e = getenv("BLR_GEMM_XCD"); return e ? atoi(e) : 1; }();
+  static const int gm_env = [] { const char* e = getenv("BLR_GEMM_GM"); return e ? atoi(e) : 4; }();
+  const int64_t total = (int64_t)tiles_m * tiles_n * g.batch;
+  if (total > (1ll << 30)) { set_error("gemm: too many tiles"); return BLR_ERR_UNSUPPORTED; }
+  int per_xcd = xcd_on ? (int)cdiv(total, 8) : 0;
+  int group_m = gm_env < 1 ? 1 : gm_env;
+  dim3 grid((unsigned)(per_xcd > 0 ? per_xcd * 8 : total));
   GemmArgs ga = g;
-  void* args[] = {&ga, &tiles_m, &tiles_n, &a_vec, &b_vec, &c_vec};
+  void* args[] = {&ga, &tiles_m, &tiles_n, &a_vec, &b_vec, &c_vec, &per_xcd, &group_m};
   hipError_t e = hipLaunchKernel(fn, grid, dim3(256), args, lds, st);
   if (e != hipSuccess) { set_error("gemm_mfma: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
