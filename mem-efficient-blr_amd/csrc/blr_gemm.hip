@@ -611,8 +611,9 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
   int r_chunks = (int)cdiv(R, 64);
   if (dtype != BLR_F32 && b <= 16 && R % 8 == 0 && aligned(Y, 16) && aligned(Z, 16)) {
     size_t lds = (size_t)b * b * 64 * 2;
-    int m_per_wg = 128;
-    while ((int64_t)r_chunks * cdiv(M, m_per_wg) < 512 && m_per_wg > 32) m_per_wg /= 2;
+    static const int mpw_env = [] { const char* e = getenv("BLR_MIX_MPW"); return e ? atoi(e) : 0; }();
+    int m_per_wg = 32;                             // one pass of the 32 row slots: more, smaller workgroups measured fastest
+    if (mpw_env > 0) m_per_wg = mpw_env;
     dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
     static const bool h2 = [] { const char* e = getenv("BLR_MIX_H2"); return e ? atoi(e) != 0 : true; }();
     if (dtype == BLR_F16 && h2)
