@@ -509,25 +509,59 @@ static void mix_dispatch(dim3 grid, size_t lds, hipStream_t st, const void* Y, c
     hipLaunchKernelGGL((blast_mix_kernel<T, 0>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
 }
 
+// S slab of a workgroup of the mix kernels: s_t[(j * b + i) * 64 + r] = S(i, j, r0 + r) for 64 ranks, zero past R.
+// 16-byte pieces along whichever of r or j is contiguous in memory; element-wise otherwise.
+template <typename T>
+__device__ __forceinline__ void mix_stage_s(const T* __restrict__ S, T* s_t, int b, int R, int r0,
+                                            int64_t s_si, int64_t s_sj, int64_t s_sr, int vec_ok) {
+  using V8 = typename TypeTraits<T>::vec8;
+  const int tid = threadIdx.x;
+  if (vec_ok && s_sr == 1) {                                   // (j, i, r) or (i, j, r): r contiguous
+    for (int idx = tid; idx < b * b * 8; idx += 256) {
+      const int r8 = (idx & 7) * 8, ji = idx >> 3;
+      const int j = ji / b, i = ji - j * b;
+      V8 v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (T)0.0f;
+      if (r0 + r8 < R) v = *reinterpret_cast<const V8*>(&S[(int64_t)i * s_si + (int64_t)j * s_sj + r0 + r8]);
+      *reinterpret_cast<V8*>(&s_t[ji * 64 + r8]) = v;
+    }
+  } else if (vec_ok && s_sj == 1 && (b & 7) == 0) {            // (r, i, j): j contiguous
+    const int jv = b >> 3;
+    for (int idx = tid; idx < 64 * b * jv; idx += 256) {
+      const int j8 = (idx % jv) * 8, t = idx / jv;
+      const int i = t % b, r = t / b;
+      V8 v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (T)0.0f;
+      if (r0 + r < R) v = *reinterpret_cast<const V8*>(&S[(int64_t)(r0 + r) * s_sr + (int64_t)i * s_si + j8]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s_t[((j8 + e) * b + i) * 64 + r] = v[e];
+    }
+  } else {
+    for (int idx = tid; idx < b * b * 64; idx += 256) {
+      const int r = idx & 63, ji = idx >> 6;
+      const int j = ji / b, i = ji - j * b;
+      T v = (T)0.0f;
+      if (r0 + r < R) v = S[(int64_t)i * s_si + (int64_t)j * s_sj + (int64_t)(r0 + r) * s_sr];
+      s_t[idx] = v;
+    }
+  }
+}
+
 // Vector variant for two-byte types, b <= 16, R % 8 == 0: thread = (8 consecutive r, one m); all
 // b vectors Y_j[m, r..r+7] are loaded (16 bytes each) before the b x b x 8 multiply-adds, S comes
 // from an LDS slab [j][i][64] staged once per workgroup and reused for 128 rows of m.
 template <typename T>
 __global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict__ Y, const T* __restrict__ S,
                                                             T* __restrict__ Z, int M, int b, int R,
-                                                            int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg) {
+                                                            int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg, int s_vec) {
   using V8 = typename TypeTraits<T>::vec8;
   extern __shared__ float s_lds[];
   T* s_t = reinterpret_cast<T*>(s_lds);      // [b][b][64]  (j, i, r)
   const int tid = threadIdx.x;
   const int r0 = blockIdx.x * 64;
-  for (int idx = tid; idx < b * b * 64; idx += 256) {
-    int r = idx & 63, ji = idx >> 6;
-    int j = ji / b, i = ji - j * b;
-    T v = (T)0.0f;
-    if (r0 + r < R) v = S[(int64_t)i * s_si + (int64_t)j * s_sj + (int64_t)(r0 + r) * s_sr];
-    s_t[idx] = v;
-  }
+  mix_stage_s<T>(S, s_t, b, R, r0, s_si, s_sj, s_sr, s_vec);
   __syncthreads();
   const int rl = tid & 7, ms = tid >> 3;     // 8 r-vectors x 32 m slots
   const int r = r0 + rl * 8;
@@ -537,8 +571,8 @@ __global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict_
   for (int m = m_begin + ms; m < m_end; m += 32) {
     V8 yv[16];
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
-      if (j < b) yv[j] = ldg16<V8>(&Y[((int64_t)j * M + m) * R + r]);
+    for (int j = 0; j < 16; ++j)                     // unconditional: planes past b re-read the last one and are not used
+      yv[j] = ldg16<V8>(&Y[((int64_t)min(j, b - 1) * M + m) * R + r]);
     for (int i = 0; i < b; ++i) {
       float acc[8];
 #pragma unroll
@@ -562,22 +596,17 @@ __global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict_
 // fp16 only: the same mix with packed half-precision multiply-adds (two per lane and instruction).
 // The b <= 16 products of one output are accumulated in fp16; Z is stored as fp16 anyway and the
 // reference rounds it to 16 bits as well, so this costs about one extra rounding of the result.
+template <bool FULL16>                           // FULL16: b == 16, so no load sits under a condition
 __global__ __launch_bounds__(256) void blast_mix_h2_kernel(const f16* __restrict__ Y, const f16* __restrict__ S,
                                                            f16* __restrict__ Z, int M, int b, int R,
-                                                           int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg) {
+                                                           int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg, int s_vec) {
   typedef _Float16 h2 __attribute__((ext_vector_type(2)));
   struct H8 { h2 v[4]; };
   extern __shared__ float s_lds[];
   f16* s_t = reinterpret_cast<f16*>(s_lds);      // [b][b][64]  (j, i, r)
   const int tid = threadIdx.x;
   const int r0 = blockIdx.x * 64;
-  for (int idx = tid; idx < b * b * 64; idx += 256) {
-    int r = idx & 63, ji = idx >> 6;
-    int j = ji / b, i = ji - j * b;
-    f16 v = (f16)0.0f;
-    if (r0 + r < R) v = S[(int64_t)i * s_si + (int64_t)j * s_sj + (int64_t)(r0 + r) * s_sr];
-    s_t[idx] = v;
-  }
+  mix_stage_s<f16>(S, s_t, b, R, r0, s_si, s_sj, s_sr, s_vec);
   __syncthreads();
   const int rl = tid & 7, ms = tid >> 3;     // 8 r-vectors x 32 m slots
   const int r = r0 + rl * 8;
@@ -587,15 +616,15 @@ __global__ __launch_bounds__(256) void blast_mix_h2_kernel(const f16* __restrict
   for (int m = m_begin + ms; m < m_end; m += 32) {
     H8 yv[16];
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
-      if (j < b) yv[j] = *reinterpret_cast<const H8*>(&Y[((int64_t)j * M + m) * R + r]);
+    for (int j = 0; j < 16; ++j)                     // unconditional: planes past b re-read the last one and are not used
+      yv[j] = *reinterpret_cast<const H8*>(&Y[((int64_t)(FULL16 ? j : min(j, b - 1)) * M + m) * R + r]);
     for (int i = 0; i < b; ++i) {
       H8 acc;
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc.v[e] = h2{(_Float16)0.0f, (_Float16)0.0f};
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        if (j < b) {
+        if (FULL16 || j < b) {
           const H8 sv = *reinterpret_cast<const H8*>(&s_t[(j * b + i) * 64 + rl * 8]);
 #pragma unroll
           for (int e = 0; e < 4; ++e) acc.v[e] = sv.v[e] * yv[j].v[e] + acc.v[e];
@@ -612,16 +641,20 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
   if (dtype != BLR_F32 && b <= 16 && R % 8 == 0 && aligned(Y, 16) && aligned(Z, 16)) {
     size_t lds = (size_t)b * b * 64 * 2;
     static const int mpw_env = [] { const char* e = getenv("BLR_MIX_MPW"); return e ? atoi(e) : 0; }();
+    // S may be fetched in 16-byte pieces if every piece starts on a 16-byte boundary
+    const int s_vec = aligned(S, 16) && ((s_sr == 1 && s_si % 8 == 0 && s_sj % 8 == 0) ||
+                                         (s_sj == 1 && s_si % 8 == 0 && s_sr % 8 == 0));
     int m_per_wg = 32;                             // one pass of the 32 row slots: more, smaller workgroups measured fastest
     if (mpw_env > 0) m_per_wg = mpw_env;
     dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
     static const bool h2 = [] { const char* e = getenv("BLR_MIX_H2"); return e ? atoi(e) != 0 : true; }();
     if (dtype == BLR_F16 && h2)
-      hipLaunchKernelGGL(blast_mix_h2_kernel, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+      if (b == 16) hipLaunchKernelGGL(blast_mix_h2_kernel<true>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
+      else hipLaunchKernelGGL(blast_mix_h2_kernel<false>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
     else if (dtype == BLR_F16)
-      hipLaunchKernelGGL(blast_mix_vec_kernel<f16>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+      hipLaunchKernelGGL(blast_mix_vec_kernel<f16>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
     else
-      hipLaunchKernelGGL(blast_mix_vec_kernel<bf16>, grid, dim3(256), lds, st, (const bf16*)Y, (const bf16*)S, (bf16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+      hipLaunchKernelGGL(blast_mix_vec_kernel<bf16>, grid, dim3(256), lds, st, (const bf16*)Y, (const bf16*)S, (bf16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
     BLR_CHECK_LAUNCH("blast_mix_vec");
     return BLR_OK;
   }
