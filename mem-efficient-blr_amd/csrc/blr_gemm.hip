@@ -434,7 +434,9 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   int64_t t128 = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
   // 256x256 needs 256 accumulator registers per lane and currently spills: only on request (BLR_GEMM_TILE=256).
   if (force == 256 && t256 > 0) return launch_mfma<T, 256, 256>(g, st);
-  if (force == 128256 || (force == 0 && g.M >= 256 && t128 >= cus)) return launch_mfma<T, 256, 128>(g, st);
+  // short reductions are dominated by filling and draining a tile: two smaller workgroups per CU overlap those
+  static const int small_k = [] { const char* e = getenv("BLR_GEMM_SMALL_K"); return e ? atoi(e) : 1024; }();
+  if (force == 128256 || (force == 0 && g.M >= 256 && t128 >= cus && g.K > small_k)) return launch_mfma<T, 256, 128>(g, st);
   return launch_mfma<T, 128, 128>(g, st);
 }
 
