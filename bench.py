@@ -35,7 +35,7 @@ B = 16
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE), scaled
 # by the same counters over a copy kernel of known size (1 FETCH_SIZE unit = 1.99978 KiB, 1 WRITE_SIZE unit = 1 KiB).
-TRAFFIC_BYTES = 70.96e6   # 70.33 MB fetched + 0.63 MB written (profiles/decode2_kernel_blast_llama7b_decode_m1.txt)
+TRAFFIC_BYTES = 71.06e6   # 70.43 MB fetched + 0.63 MB written (profiles/decode2_kernel_blast_llama7b_decode_m1.txt)
 
 
 def blast_bytes_flops(n, i, r, o, b=B, elt=2):
@@ -49,9 +49,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-table", action="store_true", help="skip the per-layer table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--pmc", choices=["dominant", "calib"], default=None,
-                    help="counter-collection helper: launch only the dominant kernel (dominant) or only copy/probe kernels "
-                         "of known size (calib), eagerly, and print nothing but a note")
+    ap.add_argument("--pmc", choices=["dominant", "calib", "prefill"], default=None,
+                    help="profiling helper: launch only the dominant decode kernel (dominant), only copy/probe kernels of "
+                         "known size (calib), or only the BLAST gate_up prefill kernels at M=2048 (prefill), eagerly, and "
+                         "print nothing but a note")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -187,6 +188,14 @@ def main():
             L.check(lib.blr_stream_probe(src.data_ptr(), nbytes, words.data_ptr(), torch.cuda.current_stream().cuda_stream), "probe")
         torch.cuda.synchronize()
         print(json.dumps({"pmc": "calib", "copy_bytes_read": nbytes, "copy_bytes_written": nbytes, "probe_bytes_read": nbytes}))
+        return
+    if args.pmc == "prefill":
+        pf = [mk_blast(2048, *LAYERS["gate_up"][:2], LAYERS["gate_up"][2], L.U_RQ, L.S_JIR) for _ in range(4)]
+        st = torch.cuda.current_stream().cuda_stream
+        for i in range(24):
+            pf[i % 4][0](st)
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc": "prefill", "launches": 24, "flops": blast_bytes_flops(2048, 4096, 1024, 22016)[1]}))
         return
     if args.pmc == "dominant":
         gu = [mk_blast(1, *LAYERS["gate_up"][:2], LAYERS["gate_up"][2], L.U_RQ, L.S_JIR) for _ in range(12)]
