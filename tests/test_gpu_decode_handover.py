@@ -1,0 +1,113 @@
+"""GPU tests of the two-stage decode kernels' hand-over protocol (tagged values, epoch in the workspace).
+
+Calls of different operators and shapes share one workspace per stream, as they do in a model; every
+call must see only values published by itself.  Results are compared with the oracle and, call after
+call, bit for bit with the first result of the same case (the reductions run in a fixed order).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import blr_oracle as O
+from gpu_util import assert_close, blast_inputs, dev, rounded, say
+
+pytestmark = pytest.mark.gpu
+
+
+def _blast_case(b, p, q, r, M, name, dtype, seed):
+    from triton_funcs import blast_kernels as K
+    x, U, Vt, S = blast_inputs(b, p, q, r, (1, M), seed=seed)
+    if "bmm" in name:
+        Uk, Vk, Sk = O.blast_to_bmm_layout(U, Vt, S)
+    else:
+        Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+    args = [dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype)]
+    ref = O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0]
+    return (lambda: getattr(K, name)(*args)), ref
+
+
+def _low_rank_case(in_f, out_f, r, M, dtype, seed):
+    from triton_funcs import low_rank_kernels as K
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((1, M, in_f)); a = rng.standard_normal((in_f, r)) / np.sqrt(r); bm = rng.standard_normal((r, out_f)) / np.sqrt(r)
+    args = [dev(x, dtype), dev(a, dtype), dev(bm, dtype)]
+    ref = (rounded(x, dtype) @ rounded(a, dtype)) @ rounded(bm, dtype)
+    return (lambda: K.triton_low_rank_fp16(*args)), ref.reshape(M, out_f)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_interleaved_calls_share_one_workspace(dtype):
+    cases = {
+        "blast_full_m1": _blast_case(16, 64, 72, 128, 1, "triton_blast_full_fp16", dtype, 1),
+        "blast_full_m3": _blast_case(16, 32, 40, 64, 3, "triton_blast_full_fp16", dtype, 2),
+        "blast_full_m16": _blast_case(16, 64, 72, 128, 16, "triton_blast_full_fp16", dtype, 3),
+        "blast_bmm_m2": _blast_case(16, 64, 72, 512, 2, "triton_blast_bmm_fp16", dtype, 4),
+        "blast_grouped_m7": _blast_case(4, 48, 24, 96, 7, "triton_blast_partial_grouped_fp16", dtype, 5),
+        "low_rank_m1": _low_rank_case(256, 200, 64, 1, dtype, 6),
+        "low_rank_m9": _low_rank_case(512, 328, 128, 9, dtype, 7),
+    }
+    first = {}
+    order = list(cases)
+    for rep in range(40):
+        for k in (order if rep % 2 == 0 else order[::-1]):
+            fn, ref = cases[k]
+            out = fn()
+            if k not in first:
+                say(f"[case] hand-over {k} {dtype}")
+                assert_close(out, ref.reshape(tuple(out.shape)), dtype, k)
+                first[k] = out.clone()
+            else:
+                assert torch.equal(out, first[k]), f"{k}: call {rep} differs from the first call"
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("M", list(range(1, 17)))
+def test_blast_every_m_up_to_16(M):
+    say(f"[case] blast full M={M}")
+    for name in ("triton_blast_full_fp16", "triton_blast_bmm_fp16"):
+        fn, ref = _blast_case(16, 64, 72, 128, M, name, torch.float16, 10 + M)
+        out = fn()
+        assert_close(out, ref.reshape(tuple(out.shape)), torch.float16, f"{name} M={M}")
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 16])
+def test_blast_q_every_decode_path(M, bits):
+    from triton_funcs import blast_sym_quant_kernels as Q
+    b, p, q, r = 16, 32, 64, 64
+    rng = np.random.default_rng(30 + M)
+    x = rng.standard_normal((1, M, b * p))
+    U = (rng.standard_normal((b, q, r)) / np.sqrt(r)).astype(np.float32)
+    V = (rng.standard_normal((b, p, r)) / np.sqrt(r)).astype(np.float32)
+    S = rng.standard_normal((r, b, b))
+    say(f"[case] blast_q bits={bits} M={M}")
+    Uq, Vq = Q.quantize_blast_factors(torch.from_numpy(U).cuda(), torch.from_numpy(V).cuda(), bits)
+    uc, us = O.quantize_sym(U, 2, bits); vc, vs = O.quantize_sym(V, 1, bits)
+    ref = O.blast_q_forward(rounded(x, torch.float16), uc, us, vc, vs, rounded(S, torch.float16))
+    out = Q.triton_blast_bmm_int8_fp16(dev(x, torch.float16), Uq, Vq, dev(S, torch.float16))
+    assert_close(out, ref, torch.float16, f"blast_q bits={bits} M={M}")
+
+
+def test_decode_call_replayed_from_a_graph():
+    """A captured decode call gives the eager result on every replay, with eager work in between."""
+    fn, ref = _blast_case(16, 64, 72, 128, 1, "triton_blast_full_fp16", torch.float16, 50)
+    other, _ = _blast_case(16, 32, 40, 64, 5, "triton_blast_full_fp16", torch.float16, 51)
+    eager = fn().clone()
+    assert_close(eager, ref.reshape(tuple(eager.shape)), torch.float16, "eager")
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()                                        # sizes this stream's workspace before the capture
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            captured = fn()
+    torch.cuda.synchronize()
+    for rep in range(6):
+        captured.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager), f"replay {rep} differs from the eager result"
+        other()                                     # eager calls between the replays
+        torch.cuda.synchronize()
