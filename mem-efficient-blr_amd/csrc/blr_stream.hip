@@ -463,13 +463,13 @@ __device__ __forceinline__ void phase_kn(const PhaseDesc& d, int M, float* smem,
 // registers (v_perm) into eight B fragments of v_mfma_f32_16x16x32 - fragment e holds column
 // 8*cv + e for the lane's 8 rows - and the activations, staged in LDS as [16][k], are the A
 // fragment.  A wave contracts its own 32 rows per batch; the four waves are added through LDS.
-constexpr int KNM_KC_MAX = 384;                  // 16 x (384 + 8) two-byte activations fit the staging area
+constexpr int KNM_KC_MAX = 2048;                 // 16 x (2048 + 8) two-byte activations: 66 KB of LDS, two workgroups per CU
 
 template <typename T>
 __device__ __forceinline__ void phase_kn_mfma(const PhaseDesc& d, int M, float* smem, int trb, float* zcur) {
   using V8 = typename TypeTraits<T>::vec8;
   T* a_s = reinterpret_cast<T*>(smem);              // [16][ka_ld]
-  float* red = smem + AS_FLOATS;                   // [4 waves][4 fragments][64 lanes][4]
+  float* red = smem;                               // [4 waves][4 fragments][64 lanes][4]; reuses the staging area once the products are done
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cv = lane & 15, kg = lane >> 4, rs = wave * 4 + kg;
   const int NC = 128;
@@ -491,6 +491,16 @@ __device__ __forceinline__ void phase_kn_mfma(const PhaseDesc& d, int M, float* 
         if (m < M && ka < kc) v = ld_dev4(d.amode == A_Z ? zcur : reinterpret_cast<const float*>(d.a), (uint32_t)((((int64_t)bt * M + m) * d.K + it.k0 + ka) * 4));
 #pragma unroll
         for (int e = 0; e < 4; ++e) a_s[m * ka_ld + ka + e] = TypeTraits<T>::from_f32(v[e]);
+      }
+    } else if (d.amode == A_X && ((d.lda | d.a_bs | it.k0 | kc) & 7) == 0 && (reinterpret_cast<uintptr_t>(d.a) & 15) == 0) {
+      // activations straight from x in 16-byte pieces (they already have the element type of the A fragment)
+      const int pieces = kcp >> 3;
+      const T* xp = reinterpret_cast<const T*>(d.a);
+      for (int idx = tid; idx < 16 * pieces; idx += 256) {
+        int m = idx / pieces, ka = (idx - m * pieces) * 8;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (m < M && ka < kc) v = *reinterpret_cast<const u32x4*>(&xp[(int64_t)m * d.lda + (int64_t)bt * d.a_bs + it.k0 + ka]);
+        *reinterpret_cast<u32x4*>(&a_s[m * ka_ld + ka]) = v;
       }
     } else {
       for (int idx = tid; idx < 16 * kcp; idx += 256) {
@@ -957,7 +967,11 @@ size_t lds_bytes_for(const StreamParams& p) {
   for (int i = 0; i < p.nph; ++i) {
     const PhaseDesc& d = p.ph[i];
     size_t b = 0;
-    if (d.kind == PH_KN) b = (size_t)(AS_FLOATS + 4 * RED_MG * NC_MAX) * sizeof(float);
+    if (d.kind == PH_KN && d.kn_mfma) {
+      const size_t kcp = (size_t)(d.kc + 127) / 128 * 128;
+      b = 16 * (kcp + 8) * 2;                                   // activations as [16][kcp + 8] two-byte values
+      if (b < 4 * 4 * 64 * 4 * sizeof(float)) b = 4 * 4 * 64 * 4 * sizeof(float);   // the reduction reuses the same area
+    } else if (d.kind == PH_KN) b = (size_t)(AS_FLOATS + 4 * RED_MG * NC_MAX) * sizeof(float);
     else if (d.kind == PH_NK) {
       int ks = nk_kstep(d.wbits);
       int Kp = (d.K + ks - 1) / ks * ks;
