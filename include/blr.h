@@ -82,6 +82,19 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
                   int dtype, int u_layout, int s_layout, int algo,
                   void* ws, size_t ws_bytes, void* stream);
 
+/* ---- BLAST with int8-valued intermediates ---------------------------------------------------
+ * The arithmetic of the reference's blast_bmm_int8 kernels (triton_funcs/blast_sym_quant_kernels.py:
+ * 92-112, 214-234, 340-360, launcher 558-580): Y = x_j V_j and Z = sum_j S Y are accumulated in fp32,
+ * rounded to nearest even and saturated to [-128, 127]; out = Z_i U_i is stored in dtype.  Weights stay
+ * in dtype (the reference kernels read them unquantized).  Same layouts and optional y_out / z_out as
+ * blr_blast_fwd; the intermediates hold the int8 values exactly, in dtype.  Three launches at any M. */
+size_t blr_blast_i8act_workspace_bytes(int M, int in_f, int out_f, int b, int r, int dtype);
+int blr_blast_i8act_fwd(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                        void* out, int64_t ldo, void* z_out, void* y_out,
+                        int M, int in_f, int out_f, int b, int r,
+                        int dtype, int u_layout, int s_layout,
+                        void* ws, size_t ws_bytes, void* stream);
+
 /* ---- weight-quantized BLAST ---------------------------------------------------------------
  * Same product with U and V stored as symmetric int8 (bits = 8) or packed int4 (bits = 4) codes
  * and fp16 per-output-channel scales.  Both factors are stored (k, n)-ordered, the order in which

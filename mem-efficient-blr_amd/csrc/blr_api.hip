@@ -194,6 +194,48 @@ static int check_blast_shape(const char* who, int M, int in_f, int out_f, int b,
   return BLR_OK;
 }
 
+// Three launches: Y = x_j V_j (batched GEMM), Z = mix(S, Y), out_i = Z_i U_i (batched GEMM).  sat8 rounds and
+// saturates Y and Z to the int8 range.  Y and Z (b, M, r) live in the workspace unless the caller wants them.
+static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                       void* out, int64_t ldo, void* z_out, void* y_out,
+                       int M, int in_f, int out_f, int b, int r,
+                       int dtype, int u_layout, int s_layout, int sat8,
+                       void* ws, size_t ws_bytes, hipStream_t st) {
+  const int P = in_f / b, Q = out_f / b;
+  const size_t es = elt_size(dtype);
+  const size_t ybytes = align_up((size_t)b * M * r * es, 256);
+  size_t need = (y_out ? 0 : ybytes) + (z_out ? 0 : ybytes);
+  if (need && (!ws || ws_bytes < need)) { set_error("blast: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
+  char* wp = reinterpret_cast<char*>(ws);
+  void* Y = y_out ? y_out : (void*)wp; if (!y_out) wp += ybytes;
+  void* Z = z_out ? z_out : (void*)wp;
+
+  GemmArgs g1 = {};
+  g1.A = x; g1.lda = ldx; g1.sA = P;
+  g1.B = V; g1.ldb = r; g1.sB = (int64_t)P * r; g1.b_kn = 1;
+  g1.C = Y; g1.ldc = r; g1.sC = (int64_t)M * r; g1.cn = 1;
+  g1.M = M; g1.N = r; g1.K = P; g1.batch = b;
+  g1.sat8 = sat8;
+  int rc = gemm_launch(g1, dtype, st);
+  if (rc) return rc;
+
+  int64_t si, sj, sr;
+  if (s_layout == BLR_S_JIR) { sj = (int64_t)b * r; si = r; sr = 1; }
+  else if (s_layout == BLR_S_RIJ) { sr = (int64_t)b * b; si = b; sj = 1; }
+  else { si = (int64_t)b * r; sj = r; sr = 1; }
+  rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st, sat8);
+  if (rc) return rc;
+
+  GemmArgs g2 = {};
+  g2.A = Z; g2.lda = r; g2.sA = (int64_t)M * r;
+  g2.B = U;
+  if (u_layout == BLR_U_RQ) { g2.b_kn = 1; g2.ldb = Q; g2.sB = (int64_t)r * Q; }
+  else { g2.b_kn = 0; g2.ldb = r; g2.sB = (int64_t)Q * r; }
+  g2.C = out; g2.ldc = ldo; g2.sC = Q; g2.cn = 1;
+  g2.M = M; g2.N = Q; g2.K = r; g2.batch = b;
+  return gemm_launch(g2, dtype, st);
+}
+
 int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
                   void* out, int64_t ldo, void* z_out, void* y_out,
                   int M, int in_f, int out_f, int b, int r,
@@ -217,37 +259,31 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
     return stream_blast_launch(s, st);
   }
   if (a != BLR_ALGO_TILED) { set_error("blast: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
-  const size_t es = elt_size(dtype);
-  const size_t ybytes = align_up((size_t)b * M * r * es, 256);
-  size_t need = (y_out ? 0 : ybytes) + (z_out ? 0 : ybytes);
-  if (need && (!ws || ws_bytes < need)) { set_error("blast: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
-  char* wp = reinterpret_cast<char*>(ws);
-  void* Y = y_out ? y_out : (void*)wp; if (!y_out) wp += ybytes;
-  void* Z = z_out ? z_out : (void*)wp;
+  return blast_tiled(x, ldx, U, V, S, out, ldo, z_out, y_out, M, in_f, out_f, b, r, dtype, u_layout, s_layout, 0, ws, ws_bytes, st);
+}
 
-  GemmArgs g1 = {};
-  g1.A = x; g1.lda = ldx; g1.sA = P;
-  g1.B = V; g1.ldb = r; g1.sB = (int64_t)P * r; g1.b_kn = 1;
-  g1.C = Y; g1.ldc = r; g1.sC = (int64_t)M * r; g1.cn = 1;
-  g1.M = M; g1.N = r; g1.K = P; g1.batch = b;
-  rc = gemm_launch(g1, dtype, st);
+// ---- BLAST with int8-valued intermediates ----------------------------------------------------------
+// Reference triton_funcs/blast_sym_quant_kernels.py:92-112 (Y), :214-234 (Z), :340-360 (out): the two
+// intermediates are rounded to nearest even and saturated to [-128, 127] after fp32 accumulation.  The
+// values are kept in the activation dtype (every integer of that range is exact in f16, bf16 and f32).
+size_t blr_blast_i8act_workspace_bytes(int M, int in_f, int out_f, int b, int r, int dtype) {
+  (void)in_f; (void)out_f;
+  if (M <= 0 || b <= 0 || r <= 0) return 0;
+  return 2 * align_up((size_t)b * M * r * elt_size(dtype), 256);
+}
+
+int blr_blast_i8act_fwd(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                        void* out, int64_t ldo, void* z_out, void* y_out,
+                        int M, int in_f, int out_f, int b, int r,
+                        int dtype, int u_layout, int s_layout,
+                        void* ws, size_t ws_bytes, void* stream) {
+  if (!x || !U || !V || !S || !out) { set_error("blast_i8act: null pointer"); return BLR_ERR_BAD_ARG; }
+  if (!dtype_ok(dtype) || u_layout < 0 || u_layout > 1 || s_layout < 0 || s_layout > 2) { set_error("blast_i8act: bad enum"); return BLR_ERR_BAD_ARG; }
+  int rc = check_blast_shape("blast_i8act", M, in_f, out_f, b, r);
   if (rc) return rc;
-
-  int64_t si, sj, sr;
-  if (s_layout == BLR_S_JIR) { sj = (int64_t)b * r; si = r; sr = 1; }
-  else if (s_layout == BLR_S_RIJ) { sr = (int64_t)b * b; si = b; sj = 1; }
-  else { si = (int64_t)b * r; sj = r; sr = 1; }
-  rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st);
-  if (rc) return rc;
-
-  GemmArgs g2 = {};
-  g2.A = Z; g2.lda = r; g2.sA = (int64_t)M * r;
-  g2.B = U;
-  if (u_layout == BLR_U_RQ) { g2.b_kn = 1; g2.ldb = Q; g2.sB = (int64_t)r * Q; }
-  else { g2.b_kn = 0; g2.ldb = r; g2.sB = (int64_t)Q * r; }
-  g2.C = out; g2.ldc = ldo; g2.sC = Q; g2.cn = 1;
-  g2.M = M; g2.N = Q; g2.K = r; g2.batch = b;
-  return gemm_launch(g2, dtype, st);
+  if (ldx < in_f || ldo < out_f) { set_error("blast_i8act: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  return blast_tiled(x, ldx, U, V, S, out, ldo, z_out, y_out, M, in_f, out_f, b, r, dtype, u_layout, s_layout, 1,
+                     ws, ws_bytes, (hipStream_t)stream);
 }
 
 // ---- quantized BLAST -----------------------------------------------------------------------------

@@ -52,6 +52,9 @@ template <> struct TypeTraits<float> {
   static __device__ __forceinline__ float from_f32(float v) { return v; }
 };
 
+// Round to nearest even, then clamp to the int8 range (reference blast_sym_quant_kernels.py:105-108: nearbyint, clamp).
+__device__ __forceinline__ float sat8_rne(float v) { return fminf(fmaxf(rintf(v), -128.0f), 127.0f); }
+
 // 16-byte global load / store of 8 two-byte elements (pointer must be 16-byte aligned).
 template <typename V> __device__ __forceinline__ V ldg16(const void* p) {
   return *reinterpret_cast<const V*>(p);
@@ -91,14 +94,16 @@ struct GemmArgs {
   int epi;          // EPI_*
   int per;          // EPI_MONARCH_SCATTER: column c of batch kk -> C[(c/per)*sL + m*ldc + kk*per + c%per]
   int64_t sL;
+  int sat8;         // 1: the fp32 result is rounded to nearest even and clamped to [-128, 127] before it is stored
 };
 // dtype: blr_dtype.  Returns blr_status.
 int gemm_launch(const GemmArgs& a, int dtype, hipStream_t st);
 
 // ---- BLAST rank-space mix, tiled path (blr_gemm.hip) ------------------------------------
 // Z[i, m, r] = sum_j S(i, j, r) * Y[j, m, r];  Y, Z (b, M, R) contiguous of dtype.
+// sat8: accumulate in fp32, then round to nearest even and clamp to [-128, 127] before the store.
 int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
-                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st);
+                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st, int sat8 = 0);
 
 // ---- streaming (decode) engine (blr_stream.hip) -------------------------------------------
 struct StreamBlastArgs {

@@ -300,7 +300,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           int row = wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-          cs[row * CLD + col] = TypeTraits<T>::from_f32(acc[i][j][e]);
+          cs[row * CLD + col] = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][e]) : acc[i][j][e]);
         }
       }
     __syncthreads();
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         int row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row < g.M && col < g.N) C[epi_offset(g, bt, row, col)] = TypeTraits<T>::from_f32(acc[i][j][e]);
+        if (row < g.M && col < g.N) C[epi_offset(g, bt, row, col)] = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][e]) : acc[i][j][e]);
       }
     }
 }
@@ -375,7 +375,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) 
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       int row = m0 + ty * 4 + i, col = n0 + tx * 4 + j;
-      if (row < g.M && col < g.N) C[epi_offset(g, bt, row, col)] = acc[i][j];
+      if (row < g.M && col < g.N) C[epi_offset(g, bt, row, col)] = g.sat8 ? sat8_rne(acc[i][j]) : acc[i][j];
     }
 }
 
@@ -462,7 +462,7 @@ int gemm_launch(const GemmArgs& g, int dtype, hipStream_t st) {
 template <typename T, int MAXB>
 __global__ __launch_bounds__(256) void blast_mix_kernel(const T* __restrict__ Y, const T* __restrict__ S,
                                                         T* __restrict__ Z, int M, int b, int R,
-                                                        int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg) {
+                                                        int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg, int sat8) {
   extern __shared__ float s_lds[];           // [b][b][64]  (j, i, r)
   const int tid = threadIdx.x;
   const int r0 = blockIdx.x * 64;
@@ -489,14 +489,14 @@ __global__ __launch_bounds__(256) void blast_mix_kernel(const T* __restrict__ Y,
 #pragma unroll
         for (int j = 0; j < MAXB; ++j)
           if (j < b) acc = fmaf(s_lds[(j * b + i) * 64 + rr], yv[j], acc);
-        Z[((int64_t)i * M + m) * R + r] = TypeTraits<T>::from_f32(acc);
+        Z[((int64_t)i * M + m) * R + r] = TypeTraits<T>::from_f32(sat8 ? sat8_rne(acc) : acc);
       }
     } else {
       for (int i = 0; i < b; ++i) {
         float acc = 0.0f;
         for (int j = 0; j < b; ++j)
           acc = fmaf(s_lds[(j * b + i) * 64 + rr], TypeTraits<T>::to_f32(Y[((int64_t)j * M + m) * R + r]), acc);
-        Z[((int64_t)i * M + m) * R + r] = TypeTraits<T>::from_f32(acc);
+        Z[((int64_t)i * M + m) * R + r] = TypeTraits<T>::from_f32(sat8 ? sat8_rne(acc) : acc);
       }
     }
   }
@@ -504,11 +504,11 @@ __global__ __launch_bounds__(256) void blast_mix_kernel(const T* __restrict__ Y,
 
 template <typename T>
 static void mix_dispatch(dim3 grid, size_t lds, hipStream_t st, const void* Y, const void* S, void* Z, int M, int b, int R,
-                         int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg) {
+                         int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg, int sat8) {
   if (b <= 16)
-    hipLaunchKernelGGL((blast_mix_kernel<T, 16>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+    hipLaunchKernelGGL((blast_mix_kernel<T, 16>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, sat8);
   else
-    hipLaunchKernelGGL((blast_mix_kernel<T, 0>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+    hipLaunchKernelGGL((blast_mix_kernel<T, 0>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, sat8);
 }
 
 // S slab of a workgroup of the mix kernels: s_t[(j * b + i) * 64 + r] = S(i, j, r0 + r) for 64 ranks, zero past R.
@@ -557,7 +557,7 @@ __device__ __forceinline__ void mix_stage_s(const T* __restrict__ S, T* s_t, int
 template <typename T>
 __global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict__ Y, const T* __restrict__ S,
                                                             T* __restrict__ Z, int M, int b, int R,
-                                                            int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg, int s_vec) {
+                                                            int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg, int s_vec, int sat8) {
   using V8 = typename TypeTraits<T>::vec8;
   extern __shared__ float s_lds[];
   T* s_t = reinterpret_cast<T*>(s_lds);      // [b][b][64]  (j, i, r)
@@ -589,7 +589,7 @@ __global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict_
       }
       V8 o;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = TypeTraits<T>::from_f32(acc[e]);
+      for (int e = 0; e < 8; ++e) o[e] = TypeTraits<T>::from_f32(sat8 ? sat8_rne(acc[e]) : acc[e]);
       *reinterpret_cast<V8*>(&Z[((int64_t)i * M + m) * R + r]) = o;
     }
   }
@@ -638,7 +638,7 @@ __global__ __launch_bounds__(256) void blast_mix_h2_kernel(const f16* __restrict
 }
 
 int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
-                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st) {
+                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st, int sat8) {
   int r_chunks = (int)cdiv(R, 64);
   if (dtype != BLR_F32 && b <= 16 && R % 8 == 0 && aligned(Y, 16) && aligned(Z, 16)) {
     size_t lds = (size_t)b * b * 64 * 2;
@@ -650,13 +650,13 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
     if (mpw_env > 0) m_per_wg = mpw_env;
     dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
     static const bool h2 = [] { const char* e = getenv("BLR_MIX_H2"); return e ? atoi(e) != 0 : true; }();
-    if (dtype == BLR_F16 && h2)
+    if (dtype == BLR_F16 && h2 && !sat8)
       if (b == 16) hipLaunchKernelGGL(blast_mix_h2_kernel<true>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
       else hipLaunchKernelGGL(blast_mix_h2_kernel<false>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
     else if (dtype == BLR_F16)
-      hipLaunchKernelGGL(blast_mix_vec_kernel<f16>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
+      hipLaunchKernelGGL(blast_mix_vec_kernel<f16>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec, sat8);
     else
-      hipLaunchKernelGGL(blast_mix_vec_kernel<bf16>, grid, dim3(256), lds, st, (const bf16*)Y, (const bf16*)S, (bf16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
+      hipLaunchKernelGGL(blast_mix_vec_kernel<bf16>, grid, dim3(256), lds, st, (const bf16*)Y, (const bf16*)S, (bf16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec, sat8);
     BLR_CHECK_LAUNCH("blast_mix_vec");
     return BLR_OK;
   }
@@ -665,9 +665,9 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
   int m_per_wg = 64;
   while ((int64_t)r_chunks * cdiv(M, m_per_wg) < 1024 && m_per_wg > 4) m_per_wg /= 2;
   dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
-  if (dtype == BLR_F16) mix_dispatch<f16>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
-  else if (dtype == BLR_BF16) mix_dispatch<bf16>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
-  else mix_dispatch<float>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg);
+  if (dtype == BLR_F16) mix_dispatch<f16>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, sat8);
+  else if (dtype == BLR_BF16) mix_dispatch<bf16>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, sat8);
+  else mix_dispatch<float>(grid, lds, st, Y, S, Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, sat8);
   BLR_CHECK_LAUNCH("blast_mix");
   return BLR_OK;
 }

@@ -32,6 +32,8 @@ _SIGNATURES = {
     "blr_device_cus": (_i, []),
     "blr_blast_workspace_bytes": (_sz, [_i] * 7),
     "blr_blast_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp] + [_i] * 9 + [_vp, _sz, _vp]),
+    "blr_blast_i8act_workspace_bytes": (_sz, [_i] * 6),
+    "blr_blast_i8act_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp] + [_i] * 8 + [_vp, _sz, _vp]),
     "blr_blast_q_workspace_bytes": (_sz, [_i] * 6),
     "blr_blast_q_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64] + [_i] * 8 + [_vp, _sz, _vp]),
     "blr_quantize_sym": (_i, [_vp, _i, _i64, _i64, _i64, _i, _vp, _vp, _vp]),

@@ -2,10 +2,14 @@
 
 ``triton_blast_bmm_int8_fp16(x, U, V, S, config)`` keeps the reference's signature and bmm
 operand layouts (U (b, q, r), V (b, p, r), S (r, b2, b1); reference
-triton_funcs/blast_sym_quant_kernels.py:558-580).  U and V are passed as ``QuantFactor``s -
-int8 or packed-int4 codes plus fp16 per-output-channel scales, made once by
-``quantize_blast_factors`` - and are dequantised in registers inside the streaming kernel:
-the scale of V is folded into S, the scale of U is applied to the output row.
+triton_funcs/blast_sym_quant_kernels.py:558-580).  It has two modes, chosen by what U and V are:
+
+* plain tensors of x's dtype - the reference's own arithmetic: the weights are read as they are
+  and the two intermediates are rounded to nearest even and saturated to the int8 range after
+  fp32 accumulation (reference :92-112 and :214-234);
+* ``QuantFactor``s - int8 or packed-int4 codes plus fp16 per-output-channel scales, made once by
+  ``quantize_blast_factors`` - weight-only quantization, dequantised in registers inside the
+  streaming kernel: the scale of V is applied to Y, the scale of U to the output row.
 
 The reference has no weight quantizer; the scheme is this library's own: symmetric, per output
 channel, scale = fp16(max|w| / Qmax) (1 for an all-zero channel), code = clamp(rne(w / scale),
@@ -73,9 +77,37 @@ def quantize_blast_factors(U, V, bits=8):
     return QuantFactor(uc, us, bits, tuple(U.shape)), QuantFactor(vc, vs, bits, tuple(V.shape))
 
 
+def _blast_bmm_i8act(x, U, V, S):
+    """Reference arithmetic of blast_bmm_int8 (blast_sym_quant_kernels.py:558-580): int8-valued Y and Z."""
+    L.require_gpu(x, U, V, S)
+    b1, p, r = V.shape
+    b2, q, r_u = U.shape
+    assert b1 == b2                                   # reference blast_sym_quant_kernels.py:568-569
+    assert b1 != 1 and b2 != 1
+    assert r_u == r
+    assert tuple(S.shape) == (r, b2, b1)
+    assert U.dtype == x.dtype and V.dtype == x.dtype and S.dtype == x.dtype
+    assert x.shape[-1] == b1 * p
+    U, V, S = U.contiguous(), V.contiguous(), S.contiguous()
+    dt = L.dtype_code(x.dtype)
+    x2 = L.rows(x)
+    M, in_f, out_f = x2.shape[0], b1 * p, b2 * q
+    out = torch.empty((M, out_f), device=x.device, dtype=x.dtype)
+    lib = L.lib()
+    ws = L.workspace(x.device, lib.blr_blast_i8act_workspace_bytes(M, in_f, out_f, b1, r, dt), L.ALGO_TILED)
+    rc = lib.blr_blast_i8act_fwd(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
+                                 out.data_ptr(), out.stride(0), None, None, M, in_f, out_f, b1, r, dt,
+                                 L.U_QR, L.S_RIJ, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
+    L.check(rc, "triton_blast_bmm_int8_fp16")
+    _last_config["q"] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": b1, "rank": r, "bits": 0}
+    return out.reshape(*x.shape[:-1], out_f)
+
+
 def triton_blast_bmm_int8_fp16(x, U, V, S, config=(None, None, None)):
+    if isinstance(U, torch.Tensor) and isinstance(V, torch.Tensor):
+        return _blast_bmm_i8act(x, U, V, S)
     if not (isinstance(U, QuantFactor) and isinstance(V, QuantFactor)):
-        raise L.BlrError("triton_blast_bmm_int8_fp16 takes QuantFactor U and V (see quantize_blast_factors)")
+        raise L.BlrError("triton_blast_bmm_int8_fp16 takes U and V both as tensors or both as QuantFactor")
     L.require_gpu(x, S, U.codes, V.codes)
     assert U.bits == V.bits
     b1, p, r = V.shape

@@ -102,9 +102,9 @@ def test_blast_q_llama7b(layer, bits, M):
 def test_blast_q_rejects_bad_input():
     from triton_funcs import blast_sym_quant_kernels as Q, _lib as L
     x = torch.zeros(1, 1, 16, device="cuda", dtype=torch.float16)
-    with pytest.raises(L.BlrError):
-        Q.triton_blast_bmm_int8_fp16(x, torch.zeros(2, 8, 8, device="cuda"), torch.zeros(2, 8, 8, device="cuda"), torch.zeros(8, 2, 2, device="cuda"))
     U = torch.randn(2, 8, 24, device="cuda"); V = torch.randn(2, 8, 24, device="cuda")
     Uq, Vq = Q.quantize_blast_factors(U, V, 8)
+    with pytest.raises(L.BlrError):      # one plain tensor, one QuantFactor
+        Q.triton_blast_bmm_int8_fp16(x, U.half(), Vq, torch.zeros(24, 2, 2, device="cuda", dtype=torch.float16))
     with pytest.raises(L.BlrError):      # r = 24 is not a multiple of 32
         Q.triton_blast_bmm_int8_fp16(x, Uq, Vq, torch.zeros(24, 2, 2, device="cuda", dtype=torch.float16))
