@@ -326,6 +326,248 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
     }
 }
 
+// ---- large problems: 256 x 256 tiles, operand tiles copied global -> LDS without passing through registers -------
+// One workgroup of 4 waves (2 x 2, wave tile 128 x 128: 256 accumulator registers) per tile.  The k loop advances in
+// stages of 32: a stage of A (256 rows x 64 bytes) and a stage of B live in two rings in LDS (4 and 5 stages), filled by
+// global_load_lds_dwordx4 - each wave instruction moves 1 KiB and lane l's 16 bytes land at the wave's LDS address
+// + 16 l, so the layout in LDS is chosen by which global address every lane fetches:
+//   K-contiguous operand: chunk c (16 bytes) of row r sits at chunk position c ^ ((r >> 1) & 3), which makes the
+//     128-bit fragment reads of 8 consecutive rows hit 8 different 16-byte bank groups;
+//   (k, n) operand: 32 rows of 256 n as they are in memory, chunk c of row k at position c ^ ((k & 3) << 1); the
+//     fragments (8 consecutive k for one n) come out of ds_read_b64_tr_b16, which hands lane j of a 16-lane group
+//     the j-th 16-bit column of the 4 rows whose addresses lanes 4e + j/4 supply.
+// The loads are written as assembly so that the compiler does not count them: it would otherwise wait for all of them
+// before every LDS read that follows.  The kernel waits itself (s_waitcnt vmcnt) before a stage is read.
+constexpr int RING_BM = 256, RING_BN = 256, RING_NA = 4, RING_NB = 5;
+constexpr size_t ring_lds_bytes() {
+  size_t st = (size_t)(RING_NA * RING_BM + RING_NB * RING_BN) * 64, ep = (size_t)RING_BM * (RING_BN + 8) * 2;
+  return st > ep ? st : ep;
+}
+constexpr int ring_vmcnt(int n) { return (n & 0xf) | ((n >> 4) << 14) | (7 << 4) | (0xf << 8); }   // s_waitcnt immediate: vmcnt = n only
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+// 16 bytes per lane from base + off into LDS at lds + 16 * lane (base and lds are wave-uniform; lds goes through M0)
+__device__ __forceinline__ void ring_load_lds(const void* base, uint32_t off, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(off), "s"(base) : "memory");
+}
+__device__ __forceinline__ uint32_t ring_lds_addr(const void* p) {
+  return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((void __attribute__((address_space(3)))*)(p)));
+}
+
+template <typename T, bool B_KN>
+__global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
+  constexpr int BM = RING_BM, BN = RING_BN, NA = RING_NA, NB = RING_NB;
+  constexpr int ASTG = BM * 64, BSTG = BN * 64, BRING = NA * ASTG;   // stage sizes, start of the B ring
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  constexpr int LA = BM / 64, LB = BN / 64;          // 1 KiB direct loads per wave and k tile
+  constexpr int LT = LA + LB;
+  constexpr int RB = BN * 2, CPR = BN / 8, RPI = 1024 / RB;
+  constexpr int NMF = TM * TN;
+  constexpr int SLOTS_PRE = NMF + NMF / 2;              // slots before the barrier of a step
+  using V8 = typename TypeTraits<T>::vec8;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles = tiles_m * tiles_n;
+  int u = blockIdx.x;
+  if (per_xcd > 0) u = (u & 7) * per_xcd + (u >> 3);
+  if (u >= tiles * g.batch) return;
+  const int bt = u / tiles;
+  const int ut = u - bt * tiles;
+  const int strip = ut / (group_m * tiles_n);
+  const int rem = ut - strip * group_m * tiles_n;
+  const int gm_here = min(group_m, tiles_m - strip * group_m);
+  const int tm_i = strip * group_m + rem % gm_here, tn_i = rem / gm_here;
+  const int m0 = tm_i * BM, n0 = tn_i * BN;
+
+  const char* Ab = reinterpret_cast<const char*>(g.A) + (int64_t)bt * g.sA * 2;
+  const char* Bb = reinterpret_cast<const char*>(g.B) + (int64_t)bt * g.sB * 2;
+  T* C = reinterpret_cast<T*>(g.C);
+
+  const int KT = (g.K + 31) >> 5;
+  const int ktail = g.K & 31;                         // 0 or 16
+
+  // K-contiguous operand tile: rows of 32 k (64 bytes); chunk c of row r is stored at chunk c ^ ((r >> 1) & 3).
+  // (k, n) operand tile: 32 rows of BN n; chunk c of row k is stored at chunk c ^ ((k & 3) << 1): the four rows a
+  // 16-lane group of a transposing read touches then sit in four different 32-byte bank groups.
+  uint32_t a_off[LA], b_off[LB];
+  const int row16 = lane >> 2;
+  const int kc_chunk = (lane & 3) ^ ((row16 >> 1) & 3);
+#pragma unroll
+  for (int i = 0; i < LA; ++i)
+    a_off[i] = (uint32_t)(min(m0 + (i * 4 + wave) * 16 + row16, g.M - 1) * g.lda * 2 + kc_chunk * 16);
+#pragma unroll
+  for (int i = 0; i < LB; ++i) {
+    if (B_KN) {
+      const int krow = (i * 4 + wave) * RPI + lane / CPR;
+      const int chunk = (lane % CPR) ^ ((krow & 3) << 1);
+      b_off[i] = (uint32_t)(krow * g.ldb * 2 + min(n0 + chunk * 8, g.N - 8) * 2);
+    } else {
+      b_off[i] = (uint32_t)(min(n0 + (i * 4 + wave) * 16 + row16, g.N - 1) * g.ldb * 2 + kc_chunk * 16);
+    }
+  }
+  // what to subtract from those offsets in a partial last tile (16 valid k): chunks 2, 3 of a K-contiguous row and rows
+  // 16 .. 31 of a (k, n) tile are replaced by valid ones (what lands there is never multiplied)
+  const uint32_t tail_kc = (uint32_t)((kc_chunk - min(kc_chunk, 1)) * 16);
+  uint32_t tail_kn[LB];
+#pragma unroll
+  for (int i = 0; i < LB; ++i) {
+    const int krow = (i * 4 + wave) * RPI + lane / CPR;
+    tail_kn[i] = B_KN ? (uint32_t)((krow - min(krow, 15)) * g.ldb * 2) : tail_kc;
+  }
+  const uint32_t lds0 = ring_lds_addr(smem + wave * 1024);
+  // load number li of the A tile ta (into A stage sa) or of the B tile tb (into B stage sb)
+  auto issue_a = [&](int li, int ta, int sa, bool partial) {
+    ring_load_lds(Ab + (int64_t)ta * 64, a_off[li] - (partial ? tail_kc : 0u), lds0 + sa * ASTG + li * 4096);
+  };
+  auto issue_b = [&](int li, int tb, int sb, bool partial) {
+    const char* Bp = B_KN ? Bb + (int64_t)tb * 32 * g.ldb * 2 : Bb + (int64_t)tb * 64;
+    ring_load_lds(Bp, b_off[li] - (partial ? tail_kn[li] : 0u), lds0 + BRING + sb * BSTG + li * 4096);
+  };
+
+  // fragment addresses
+  const int half = lane >> 5;
+  uint32_t rowA[TM], rowB[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) rowA[i] = (uint32_t)((wm * WM + i * 32 + (lane & 31)) * 64);
+  const int g4 = lane >> 4, i16 = lane & 15;
+  if (B_KN) {
+    const int chunk0 = wn * WN / 8 + (g4 & 1) * 2 + ((i16 & 3) >> 1);
+    const int swz = (i16 >> 2) << 1;
+    const uint32_t kn_base = (uint32_t)(((g4 >> 1) * 8 + (i16 >> 2)) * RB + (i16 & 1) * 8);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) rowB[j] = kn_base + (uint32_t)(((chunk0 + 4 * j) ^ swz) << 4);
+  } else {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) rowB[j] = (uint32_t)((wn * WN + j * 32 + (lane & 31)) * 64);
+  }
+  uint32_t xo[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) xo[kk] = (uint32_t)((((kk * 2 + half) ^ ((lane >> 1) & 3)) << 4));
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  V8 af[2][TM], bf[2][TN];
+  auto frags = [&](int sa, int sb, int kk, int set) {
+    const unsigned char* sta = smem + sa * ASTG;
+    const unsigned char* st = smem + BRING + sb * BSTG;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[set][i] = *reinterpret_cast<const V8*>(sta + rowA[i] + xo[kk]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      if (B_KN) {
+        union { V8 v; s16x4 h[2]; } w;
+        w.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(st + rowB[j] + (kk * 16) * RB));
+        w.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(st + rowB[j] + (kk * 16 + 4) * RB));
+        bf[set][j] = w.v;
+      } else {
+        bf[set][j] = *reinterpret_cast<const V8*>(st + rowB[j] + xo[kk]);
+      }
+    }
+  };
+  auto mfma_one = [&](int set, int idx) {
+    const int i = idx / TN, j = idx % TN;
+    acc[i][j] = TypeTraits<T>::mfma32(af[set][i], bf[set][j], acc[i][j]);
+  };
+
+  // One k tile per step.  During step t the loads of A tile t + NA - 1 and of B tile t + NB - 1 go out (A first), into the
+  // stages that tile t - 1 occupied.  Loads complete in the order they were issued, so "tile t + 1 has landed" is a bound
+  // on the loads still in flight: everything issued after A(t+1) may be - that is B(t+NB-2) of the same step and the A and
+  // B loads of the NA - 2 steps after it, this step included.  On entry set 0 holds the kk = 0 fragments of tile t.  The
+  // loop body is one straight block for every tile: the last step also waits for, and fetches fragments of, a tile that
+  // does not exist (whatever the stage holds; never multiplied), and a partial last tile multiplies its missing half with
+  // zeros.
+  constexpr int INFLIGHT = LB + (NA - 2) * LT;
+  static_assert(NB >= NA, "B must not be needed before A under the in-order bound");
+#pragma unroll
+  for (int s = 0; s < NB - 1; ++s) {
+    const int tc = min(s, KT - 1);
+    const bool partial = ktail && tc == KT - 1;
+    if (s < NA - 1) {
+#pragma unroll
+      for (int li = 0; li < LA; ++li) issue_a(li, tc, s, partial);
+    }
+#pragma unroll
+    for (int li = 0; li < LB; ++li) issue_b(li, tc, s, partial);
+  }
+  // in flight after A(0), B(0): A(1..NA-2), B(1..NB-2)
+  __builtin_amdgcn_s_waitcnt(ring_vmcnt((NA - 2) * LA + (NB - 2) * LB));
+  __builtin_amdgcn_s_barrier();
+  frags(0, 0, 0, 0);
+  int ca = 0, cb = 0;                                // stages of tile t in the two rings
+  for (int t = 0; t < KT; ++t) {
+    const int ta = min(t + NA - 1, KT - 1), tb = min(t + NB - 1, KT - 1);
+    const bool pa = ktail && ta == KT - 1, pb = ktail && tb == KT - 1;
+    const bool zero_hi = ktail && t == KT - 1;
+    const int sla = (ca + NA - 1) & (NA - 1);        // NA is a power of two
+    const int slb = cb == 0 ? NB - 1 : cb - 1;
+    frags(ca, cb, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // the step's loads go out between its first SLOTS_PRE matrix instructions, all of them before the barrier
+    auto slot = [&](int sidx) {
+      if (sidx < SLOTS_PRE && (sidx * LT) / SLOTS_PRE != ((sidx + 1) * LT) / SLOTS_PRE) {
+        const int li = (sidx * LT) / SLOTS_PRE;
+        __builtin_amdgcn_sched_barrier(0);
+        if (li < LA) issue_a(li, ta, sla, pa);
+        else issue_b(li - LA, tb, slb, pb);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+#pragma unroll
+    for (int m = 0; m < NMF; ++m) { mfma_one(0, m); slot(m); }
+    __builtin_amdgcn_sched_barrier(0);
+    if (zero_hi) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) af[1][i][e] = (T)0.0f;
+    }
+#pragma unroll
+    for (int m = 0; m < NMF / 2; ++m) { mfma_one(1, m); slot(NMF + m); }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(ring_vmcnt(INFLIGHT));  // tile t + 1 has landed (this wave's part)
+    __builtin_amdgcn_s_barrier();                    // everybody's part has, and nobody reads the stages of tile t any more
+    ca = (ca + 1) & (NA - 1);
+    cb = cb + 1 == NB ? 0 : cb + 1;
+    frags(ca, cb, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = NMF / 2; m < NMF; ++m) mfma_one(1, m);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
+  __syncthreads();                                                   // the epilogue reuses the tile memory
+
+  constexpr int CLD = BN + 8;
+  T* cs = reinterpret_cast<T*>(smem);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        cs[row * CLD + col] = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][e]) : acc[i][j][e]);
+      }
+    }
+  __syncthreads();
+  constexpr int VPR = BN / 8;
+  for (int v = tid; v < BM * VPR; v += 256) {
+    const int row = v / VPR, cvec = (v - row * VPR) * 8;
+    const int gr = m0 + row, gc = n0 + cvec;
+    if (gr < g.M && gc < g.N)
+      *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
+  }
+}
+
+
 // ---- fp32 verification GEMM: 64x64 tile, 16x16 threads, 4x4 outputs per thread ---------------
 template <bool B_KN>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) {
@@ -424,6 +666,46 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   return BLR_OK;
 }
 
+// The 256 x 256 ring kernel takes plain row-major output and 16-byte friendly operands whose per-lane byte offsets fit 32 bits.
+static bool ring_ok(const GemmArgs& g) {
+  if (g.epi != EPI_PLAIN || g.cn != 1 || g.N < 8 || g.N % 8 || g.K % 16) return false;
+  if (!aligned(g.A, 16) || !aligned(g.B, 16) || !aligned(g.C, 16)) return false;
+  if (g.lda % 8 || g.sA % 8 || g.ldb % 8 || g.sB % 8 || g.ldc % 8 || g.sC % 8) return false;
+  const int64_t lim = (int64_t)1 << 32;
+  if ((int64_t)(g.M - 1) * g.lda * 2 + 64 >= lim) return false;
+  if (g.b_kn ? 31 * g.ldb * 2 + (int64_t)g.N * 2 >= lim : (int64_t)(g.N - 1) * g.ldb * 2 + 64 >= lim) return false;
+  return true;
+}
+
+template <typename T>
+static int launch_ring(const GemmArgs& g, hipStream_t st) {
+  int tiles_m = (int)cdiv(g.M, RING_BM), tiles_n = (int)cdiv(g.N, RING_BN);
+  const size_t lds = ring_lds_bytes();
+  void* fn = g.b_kn ? (void*)gemm_ring_kernel<T, true> : (void*)gemm_ring_kernel<T, false>;
+  static std::mutex mu;
+  static std::set<void*> raised;
+  {
+    std::lock_guard<std::mutex> lk(mu);
+    if (!raised.count(fn)) {
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) { set_error("gemm: cannot raise LDS limit: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+      raised.insert(fn);
+    }
+  }
+  static const int xcd_on = [] { const char* e = getenv("BLR_GEMM_XCD"); return e ? atoi(e) : 1; }();
+  static const int gm_env = [] { const char* e = getenv("BLR_GEMM_GM"); return e ? atoi(e) : 4; }();
+  const int64_t total = (int64_t)tiles_m * tiles_n * g.batch;
+  if (total > (1ll << 30)) { set_error("gemm: too many tiles"); return BLR_ERR_UNSUPPORTED; }
+  int per_xcd = xcd_on ? (int)cdiv(total, 8) : 0;
+  int group_m = gm_env < 1 ? 1 : gm_env;
+  dim3 grid((unsigned)(per_xcd > 0 ? per_xcd * 8 : total));
+  GemmArgs ga = g;
+  void* args[] = {&ga, &tiles_m, &tiles_n, &per_xcd, &group_m};
+  hipError_t e = hipLaunchKernel(fn, grid, dim3(256), args, lds, st);
+  if (e != hipSuccess) { set_error("gemm_ring: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  return BLR_OK;
+}
+
 template <typename T>
 static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   // Bigger tiles do more MFMA work per LDS byte (the 2x2 wave grid reads 0.5 fragments per MFMA at
@@ -432,7 +714,13 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   const int cus = device_cus() > 0 ? device_cus() : 256;
   int64_t t256 = cdiv(g.M, 256) * cdiv(g.N, 256) * g.batch;
   int64_t t128 = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
-  // 256x256 needs 256 accumulator registers per lane and currently spills: only on request (BLR_GEMM_TILE=256).
+  // Problems that fill the chip with 256 x 256 tiles go to the ring kernel (BLR_GEMM_RING: 0 never, 1 by this rule,
+  // 2 whenever the operands allow it - read at every call so that tests can switch it).
+  const char* ring_e = getenv("BLR_GEMM_RING");
+  const int ring = ring_e ? atoi(ring_e) : 1;
+  if (ring > 0 && force == 0 && ring_ok(g) && (ring > 1 || (g.M >= 192 && g.K >= 64 && t256 * 10 >= (int64_t)cus * 9)))
+    return launch_ring<T>(g, st);
+  // the register-staged kernel at 256x256 needs more registers than there are and spills: only on request (BLR_GEMM_TILE=256)
   if (force == 256 && t256 > 0) return launch_mfma<T, 256, 256>(g, st);
   // short reductions are dominated by filling and draining a tile: two smaller workgroups per CU overlap those
   static const int small_k = [] { const char* e = getenv("BLR_GEMM_SMALL_K"); return e ? atoi(e) : 1024; }();
