@@ -326,21 +326,22 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
     }
 }
 
-// ---- large problems: 256 x 256 tiles, operand tiles copied global -> LDS without passing through registers -------
-// One workgroup of 4 waves (2 x 2, wave tile 128 x 128: 256 accumulator registers) per tile.  The k loop advances in
-// stages of 32: a stage of A (256 rows x 64 bytes) and a stage of B live in two rings in LDS (4 and 5 stages), filled by
+// ---- large problems: operand tiles copied global -> LDS without passing through registers --------------------------
+// One workgroup of 4 waves (2 x 2) per BM x BN tile (256 x 256: wave tile 128 x 128, 256 accumulator registers).  The k loop advances in
+// stages of 32: a stage of A (BM rows x 64 bytes) and a stage of B live in two rings in LDS (4 and 5 stages), filled by
 // global_load_lds_dwordx4 - each wave instruction moves 1 KiB and lane l's 16 bytes land at the wave's LDS address
 // + 16 l, so the layout in LDS is chosen by which global address every lane fetches:
 //   K-contiguous operand: chunk c (16 bytes) of row r sits at chunk position c ^ ((r >> 1) & 3), which makes the
 //     128-bit fragment reads of 8 consecutive rows hit 8 different 16-byte bank groups;
-//   (k, n) operand: 32 rows of 256 n as they are in memory, chunk c of row k at position c ^ ((k & 3) << 1); the
+//   (k, n) operand: 32 rows of BN n as they are in memory, chunk c of row k at position c ^ ((k & 3) << 1); the
 //     fragments (8 consecutive k for one n) come out of ds_read_b64_tr_b16, which hands lane j of a 16-lane group
 //     the j-th 16-bit column of the 4 rows whose addresses lanes 4e + j/4 supply.
 // The loads are written as assembly so that the compiler does not count them: it would otherwise wait for all of them
 // before every LDS read that follows.  The kernel waits itself (s_waitcnt vmcnt) before a stage is read.
-constexpr int RING_BM = 256, RING_BN = 256, RING_NA = 4, RING_NB = 5;
+constexpr int RING_NA = 4, RING_NB = 5;
+template <int BM, int BN>
 constexpr size_t ring_lds_bytes() {
-  size_t st = (size_t)(RING_NA * RING_BM + RING_NB * RING_BN) * 64, ep = (size_t)RING_BM * (RING_BN + 8) * 2;
+  size_t st = (size_t)(RING_NA * BM + RING_NB * BN) * 64, ep = (size_t)BM * (BN + 8) * 2;
   return st > ep ? st : ep;
 }
 constexpr int ring_vmcnt(int n) { return (n & 0xf) | ((n >> 4) << 14) | (7 << 4) | (0xf << 8); }   // s_waitcnt immediate: vmcnt = n only
@@ -353,9 +354,9 @@ __device__ __forceinline__ uint32_t ring_lds_addr(const void* p) {
   return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((void __attribute__((address_space(3)))*)(p)));
 }
 
-template <typename T, bool B_KN>
+template <typename T, bool B_KN, int BM, int BN>
 __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
-  constexpr int BM = RING_BM, BN = RING_BN, NA = RING_NA, NB = RING_NB;
+  constexpr int NA = RING_NA, NB = RING_NB;
   constexpr int ASTG = BM * 64, BSTG = BN * 64, BRING = NA * ASTG;   // stage sizes, start of the B ring
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int LA = BM / 64, LB = BN / 64;          // 1 KiB direct loads per wave and k tile
@@ -666,7 +667,7 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   return BLR_OK;
 }
 
-// The 256 x 256 ring kernel takes plain row-major output and 16-byte friendly operands whose per-lane byte offsets fit 32 bits.
+// The ring kernels take plain row-major output and 16-byte friendly operands whose per-lane byte offsets fit 32 bits.
 static bool ring_ok(const GemmArgs& g) {
   if (g.epi != EPI_PLAIN || g.cn != 1 || g.N < 8 || g.N % 8 || g.K % 16) return false;
   if (!aligned(g.A, 16) || !aligned(g.B, 16) || !aligned(g.C, 16)) return false;
@@ -677,11 +678,11 @@ static bool ring_ok(const GemmArgs& g) {
   return true;
 }
 
-template <typename T>
+template <typename T, int BM, int BN>
 static int launch_ring(const GemmArgs& g, hipStream_t st) {
-  int tiles_m = (int)cdiv(g.M, RING_BM), tiles_n = (int)cdiv(g.N, RING_BN);
-  const size_t lds = ring_lds_bytes();
-  void* fn = g.b_kn ? (void*)gemm_ring_kernel<T, true> : (void*)gemm_ring_kernel<T, false>;
+  int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
+  const size_t lds = ring_lds_bytes<BM, BN>();
+  void* fn = g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN> : (void*)gemm_ring_kernel<T, false, BM, BN>;
   static std::mutex mu;
   static std::set<void*> raised;
   {
@@ -714,12 +715,29 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   const int cus = device_cus() > 0 ? device_cus() : 256;
   int64_t t256 = cdiv(g.M, 256) * cdiv(g.N, 256) * g.batch;
   int64_t t128 = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
-  // Problems that fill the chip with 256 x 256 tiles go to the ring kernel (BLR_GEMM_RING: 0 never, 1 by this rule,
-  // 2 whenever the operands allow it - read at every call so that tests can switch it).
+  // Problems with enough work go to the ring kernels, with the largest of their tiles that still gives every compute unit
+  // one (BLR_GEMM_RING: 0 never, 1 by this rule, 2 whenever the operands allow it; BLR_GEMM_RING_TILE = 256256, 256128
+  // or 128128 picks the tile - both read at every call so that tests can switch them).
   const char* ring_e = getenv("BLR_GEMM_RING");
   const int ring = ring_e ? atoi(ring_e) : 1;
-  if (ring > 0 && force == 0 && ring_ok(g) && (ring > 1 || (g.M >= 192 && g.K >= 64 && t256 * 10 >= (int64_t)cus * 9)))
-    return launch_ring<T>(g, st);
+  if (ring > 0 && force == 0 && ring_ok(g)) {
+    const char* rt_e = getenv("BLR_GEMM_RING_TILE");
+    int rt = rt_e ? atoi(rt_e) : 0;
+    const int64_t fill = ((int64_t)cus * 9 + 9) / 10;
+    const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
+    if (rt == 0) {
+      // short reductions are mostly tile start-up and write-out: two small workgroups per compute unit overlap those
+      if (g.K <= 512 && r128 >= fill) rt = 128128;
+      else if (t256 >= fill) rt = 256256;
+      else if (t128 >= fill) rt = 256128;
+      else if (r128 >= fill || ring > 1) rt = 128128;
+    }
+    if (rt && (ring > 1 || (g.M >= 96 && g.K >= 64))) {
+      if (rt == 256256) return launch_ring<T, 256, 256>(g, st);
+      if (rt == 256128) return launch_ring<T, 256, 128>(g, st);
+      return launch_ring<T, 128, 128>(g, st);
+    }
+  }
   // the register-staged kernel at 256x256 needs more registers than there are and spills: only on request (BLR_GEMM_TILE=256)
   if (force == 256 && t256 > 0) return launch_mfma<T, 256, 256>(g, st);
   // short reductions are dominated by filling and draining a tile: two smaller workgroups per CU overlap those

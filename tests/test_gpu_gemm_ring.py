@@ -1,7 +1,7 @@
-"""GPU parity of the 256 x 256 tile GEMM kernel (operand tiles copied global -> LDS directly) against the oracle.
+"""GPU parity of the GEMM kernels whose operand tiles are copied global -> LDS directly, against the oracle.
 
-The kernel is normally chosen only for problems that fill the chip; BLR_GEMM_RING=2 selects it whenever the operands
-allow it, so small, ragged and tail shapes (M, N not multiples of 256; K with a 16-wide last slice; K shorter than
+They are normally chosen only for problems that fill the chip; BLR_GEMM_RING=2 selects them whenever the operands
+allow it and BLR_GEMM_RING_TILE picks the tile shape (256x256, 256x128, 128x128), so small, ragged and tail shapes (M, N not multiples of 256; K with a 16-wide last slice; K shorter than
 the prefetch depth) run through it here.  Every case is also run with the kernel switched off and the two results
 must agree to rounding.
 """
@@ -17,15 +17,18 @@ from gpu_util import assert_close, back, blast_inputs, dev, rounded, say
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture
-def ring_forced():
-    old = os.environ.get("BLR_GEMM_RING")
+@pytest.fixture(params=["256256", "256128", "128128"])
+def ring_forced(request):
+    """Selects the kernel for every legal problem, with one of its three tile shapes."""
+    old = {k: os.environ.get(k) for k in ("BLR_GEMM_RING", "BLR_GEMM_RING_TILE")}
     os.environ["BLR_GEMM_RING"] = "2"
-    yield
-    if old is None:
-        del os.environ["BLR_GEMM_RING"]
-    else:
-        os.environ["BLR_GEMM_RING"] = old
+    os.environ["BLR_GEMM_RING_TILE"] = request.param
+    yield request.param
+    for k, v in old.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
 
 
 def _without_ring(fn):
@@ -50,7 +53,7 @@ def test_dense_through_ring_kernel(shape, dtype, ring_forced):
     M, in_f, out_f = shape
     rng = np.random.default_rng(M + in_f)
     x = rng.standard_normal((M, in_f)); w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)
-    say(f"[case] ring dense {shape} {dtype}")
+    say(f"[case] ring dense {shape} {dtype} tile {ring_forced}")
     xd, wd = dev(x, dtype), dev(w, dtype)
     out = K.triton_dense_fp16(xd, wd, TILED)
     assert_close(out, rounded(x, dtype) @ rounded(w, dtype), dtype, f"dense {shape}")
@@ -66,7 +69,7 @@ def test_blast_through_ring_kernel(b, p, q, r, M, name, dtype, ring_forced):
     from triton_funcs import blast_kernels as K
     x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=b + M)
     Uk, Vk, Sk = (O.blast_to_bmm_layout if "bmm" in name else O.blast_to_partial_layout)(U, Vt, S)
-    say(f"[case] ring {name} b={b} p={p} q={q} r={r} M={M} {dtype}")
+    say(f"[case] ring {name} b={b} p={p} q={q} r={r} M={M} {dtype} tile {ring_forced}")
     args = [dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype)]
     out = getattr(K, name)(*args, TILED)
     ref = O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0]
