@@ -904,7 +904,7 @@ __global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict_
 // fp16 only: the same mix with packed half-precision multiply-adds (two per lane and instruction).
 // The b <= 16 products of one output are accumulated in fp16; Z is stored as fp16 anyway and the
 // reference rounds it to 16 bits as well, so this costs about one extra rounding of the result.
-template <bool FULL16>                           // FULL16: b == 16, so no load sits under a condition
+template <bool FULL16, int MB>                   // FULL16: b == 16, so no load sits under a condition; MB rows of m per thread
 __global__ __launch_bounds__(256) void blast_mix_h2_kernel(const f16* __restrict__ Y, const f16* __restrict__ S,
                                                            f16* __restrict__ Z, int M, int b, int R,
                                                            int64_t s_si, int64_t s_sj, int64_t s_sr, int m_per_wg, int s_vec) {
@@ -921,24 +921,35 @@ __global__ __launch_bounds__(256) void blast_mix_h2_kernel(const f16* __restrict
   if (r >= R) return;
   const int m_begin = blockIdx.y * m_per_wg;
   const int m_end = min(M, m_begin + m_per_wg);
-  for (int m = m_begin + ms; m < m_end; m += 32) {
-    H8 yv[16];
+  // Each S vector read from LDS serves MB rows: the kernel is otherwise bound by LDS reads (16 bytes per 8 multiply-adds).
+  for (int m = m_begin + ms; m < m_end; m += 32 * MB) {
+    H8 yv[MB][16];
 #pragma unroll
-    for (int j = 0; j < 16; ++j)                     // unconditional: planes past b re-read the last one and are not used
-      yv[j] = *reinterpret_cast<const H8*>(&Y[((int64_t)(FULL16 ? j : min(j, b - 1)) * M + m) * R + r]);
+    for (int u = 0; u < MB; ++u) {
+      const int mu = min(m + 32 * u, M - 1);         // rows past the end are fetched again and not stored
+#pragma unroll
+      for (int j = 0; j < 16; ++j)                   // unconditional: planes past b re-read the last one and are not used
+        yv[u][j] = *reinterpret_cast<const H8*>(&Y[((int64_t)(FULL16 ? j : min(j, b - 1)) * M + mu) * R + r]);
+    }
     for (int i = 0; i < b; ++i) {
-      H8 acc;
+      H8 acc[MB];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc.v[e] = h2{(_Float16)0.0f, (_Float16)0.0f};
+      for (int u = 0; u < MB; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[u].v[e] = h2{(_Float16)0.0f, (_Float16)0.0f};
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         if (FULL16 || j < b) {
           const H8 sv = *reinterpret_cast<const H8*>(&s_t[(j * b + i) * 64 + rl * 8]);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc.v[e] = sv.v[e] * yv[j].v[e] + acc.v[e];
+          for (int u = 0; u < MB; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[u].v[e] = sv.v[e] * yv[u][j].v[e] + acc[u].v[e];
         }
       }
-      *reinterpret_cast<H8*>(&Z[((int64_t)i * M + m) * R + r]) = acc;
+#pragma unroll
+      for (int u = 0; u < MB; ++u)
+        if (m + 32 * u < m_end) *reinterpret_cast<H8*>(&Z[((int64_t)i * M + m + 32 * u) * R + r]) = acc[u];
     }
   }
 }
@@ -952,13 +963,19 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
     // S may be fetched in 16-byte pieces if every piece starts on a 16-byte boundary
     const int s_vec = aligned(S, 16) && ((s_sr == 1 && s_si % 8 == 0 && s_sj % 8 == 0) ||
                                          (s_sj == 1 && s_si % 8 == 0 && s_sr % 8 == 0));
-    int m_per_wg = 32;                             // one pass of the 32 row slots: more, smaller workgroups measured fastest
+    static const bool h2 = [] { const char* e = getenv("BLR_MIX_H2"); return e ? atoi(e) != 0 : true; }();
+    static const int mb_env = [] { const char* e = getenv("BLR_MIX_MB"); return e ? atoi(e) : 2; }();
+    const bool use_h2 = dtype == BLR_F16 && h2 && !sat8;
+    const int mb = use_h2 && mb_env == 2 && M >= 64 ? 2 : 1;
+    int m_per_wg = 32 * mb;                        // one pass of the 32 row slots: more, smaller workgroups measured fastest
     if (mpw_env > 0) m_per_wg = mpw_env;
     dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
-    static const bool h2 = [] { const char* e = getenv("BLR_MIX_H2"); return e ? atoi(e) != 0 : true; }();
-    if (dtype == BLR_F16 && h2 && !sat8)
-      if (b == 16) hipLaunchKernelGGL(blast_mix_h2_kernel<true>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
-      else hipLaunchKernelGGL(blast_mix_h2_kernel<false>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
+    if (use_h2 && mb == 2)
+      if (b == 16) hipLaunchKernelGGL((blast_mix_h2_kernel<true, 2>), grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
+      else hipLaunchKernelGGL((blast_mix_h2_kernel<false, 2>), grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
+    else if (use_h2)
+      if (b == 16) hipLaunchKernelGGL((blast_mix_h2_kernel<true, 1>), grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
+      else hipLaunchKernelGGL((blast_mix_h2_kernel<false, 1>), grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);
     else if (dtype == BLR_F16)
       hipLaunchKernelGGL(blast_mix_vec_kernel<f16>, grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec, sat8);
     else
