@@ -632,6 +632,15 @@ __device__ __forceinline__ void dm_batch(const u32x4 (&cur)[8], const T* a_s, in
   }
 }
 
+// The same batch when the weights are stored (n, k): load e is row n = column e of the lane's 8 at the lane's 8 consecutive k.
+template <typename T>
+__device__ __forceinline__ void dm_batch_nk(const u32x4 (&cur)[8], const T* a_s, int ald, int cv, int rs, int kbase, f32x4 (&acc)[8]) {
+  using V8 = typename TypeTraits<T>::vec8;
+  const V8 af = *reinterpret_cast<const V8*>(&a_s[cv * ald + kbase + rs * 8]);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = TypeTraits<T>::mfma16(af, __builtin_bit_cast(V8, cur[e]), acc[e]);
+}
+
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
   typedef T T2 __attribute__((ext_vector_type(2)));
@@ -671,8 +680,14 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   const int n2 = n0_2 + cv * 8;
   const bool col_ok2 = n2 < p.Q;
   const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.bo * p.R * p.Q * 2u);
-  const uint32_t uoff = (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs * 8) * p.Q + (col_ok2 ? n2 : 0)) * 2);
+  // U (bo, r, q): load u of a batch is row k + u of the lane's 8 columns.  U (bo, q, r): load u is row q = column u of
+  // the lane's 8, at the lane's 8 consecutive k - already a B fragment, so no transpose follows.
+  const uint32_t uoff = p.u_nk ? (uint32_t)((((int64_t)i2 * p.Q + (col_ok2 ? n2 : 0)) * p.R + k0_2 + rs * 8) * 2)
+                               : (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs * 8) * p.Q + (col_ok2 ? n2 : 0)) * 2);
   const uint32_t urow = (uint32_t)p.Q * 2u;
+  auto u_soff = [&](int batch, int u) -> uint32_t {
+    return p.u_nk ? (uint32_t)((u * p.R + batch * DM_ROWS) * 2) : (uint32_t)(batch * DM_ROWS + u) * urow;
+  };
   u32x4 pf[DM_PF];
   auto issue_prefetch = [&]() {
 #pragma unroll
@@ -681,7 +696,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
         if (u >= 4 && p.pf_depth == 4) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
         else if (u >= 8 && p.pf_depth == 8) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
         else if (u >= 16 && p.pf_depth == 16) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
-        pf[u] = ldw16(ubuf, uoff, (uint32_t)((u >> 3) * DM_ROWS + (u & 7)) * urow);
+        pf[u] = ldw16(ubuf, uoff, u_soff(u >> 3, u & 7));
       }
     }
   };
@@ -947,14 +962,16 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
       u32x4 cur[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) cur[u] = pf[bq * 8 + u];
-      dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+      if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+      else dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
     }
   }
   for (int bq = p.pfn / 8; bq * DM_ROWS < kcur2; ++bq) {          // deeper slabs: stream the rest
     u32x4 cur[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) cur[u] = ldw16(ubuf, uoff, (uint32_t)(bq * DM_ROWS + u) * urow);
-    dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+    for (int u = 0; u < 8; ++u) cur[u] = ldw16(ubuf, uoff, u_soff(bq, u));
+    if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+    else dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
   }
   TR2(5);
   T* outp = reinterpret_cast<T*>(p.out);
@@ -1059,7 +1076,7 @@ bool decode2_applicable(const StreamBlastArgs& a) {
   static const int enabled = env_i("BLR_DECODE2", 1);
   if (!enabled || a.split) return false;
   static const int nk_on = env_i("BLR_D2_NK", 1);
-  if (a.u_layout != BLR_U_RQ && !(nk_on && a.u_layout == BLR_U_QR && a.wbits == 16 && a.M <= 4)) return false;
+  if (a.u_layout != BLR_U_RQ && !(nk_on && a.u_layout == BLR_U_QR && a.wbits == 16)) return false;
   if (a.wbits != 16 && (a.wbits != 8 && a.wbits != 4)) return false;
   if (a.wbits != 16 && (a.M > 4 || !a.u_scales || !a.v_scales)) return false;   // the matrix-core variant takes two-byte weights only
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
@@ -1285,6 +1302,7 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     if (pfn > DM_PF) pfn = DM_PF;
     p.lpr2_log2 = 4; p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn;
     p.kpad2 = (kc + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
+    p.u_nk = a.u_layout == BLR_U_QR;
   }
   {
     p.zrep = bo == 1 ? 16 : 1;
