@@ -386,7 +386,7 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
   T* C = reinterpret_cast<T*>(g.C);
 
   const int KT = (g.K + 31) >> 5;
-  const int ktail = g.K & 31;                         // 0 or 16
+  const int ktail = g.K & 31;                         // valid k of the last tile when it is partial: 8, 16 or 24
 
   // K-contiguous operand tile: rows of 32 k (64 bytes); chunk c of row r is stored at chunk c ^ ((r >> 1) & 3).
   // (k, n) operand tile: 32 rows of BN n; chunk c of row k is stored at chunk c ^ ((k & 3) << 1): the four rows a
@@ -407,14 +407,15 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
       b_off[i] = (uint32_t)(min(n0 + (i * 4 + wave) * 16 + row16, g.N - 1) * g.ldb * 2 + kc_chunk * 16);
     }
   }
-  // what to subtract from those offsets in a partial last tile (16 valid k): chunks 2, 3 of a K-contiguous row and rows
-  // 16 .. 31 of a (k, n) tile are replaced by valid ones (what lands there is never multiplied)
-  const uint32_t tail_kc = (uint32_t)((kc_chunk - min(kc_chunk, 1)) * 16);
+  // what to subtract from those offsets in a partial last tile (ktail valid k): the chunks of a K-contiguous row and the
+  // rows of a (k, n) tile past ktail are replaced by valid ones (what lands there is multiplied by zeros)
+  const int cmax = max((ktail >> 3) - 1, 0), rmax = max(ktail - 1, 0);
+  const uint32_t tail_kc = (uint32_t)((kc_chunk - min(kc_chunk, cmax)) * 16);
   uint32_t tail_kn[LB];
 #pragma unroll
   for (int i = 0; i < LB; ++i) {
     const int krow = (i * 4 + wave) * RPI + lane / CPR;
-    tail_kn[i] = B_KN ? (uint32_t)((krow - min(krow, 15)) * g.ldb * 2) : tail_kc;
+    tail_kn[i] = B_KN ? (uint32_t)((krow - min(krow, rmax)) * g.ldb * 2) : tail_kc;
   }
   const uint32_t lds0 = ring_lds_addr(smem + wave * 1024);
   // load number li of the A tile ta (into A stage sa) or of the B tile tb (into B stage sb)
@@ -482,7 +483,7 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
   // on the loads still in flight: everything issued after A(t+1) may be - that is B(t+NB-2) of the same step and the A and
   // B loads of the NA - 2 steps after it, this step included.  On entry set 0 holds the kk = 0 fragments of tile t.  The
   // loop body is one straight block for every tile: the last step also waits for, and fetches fragments of, a tile that
-  // does not exist (whatever the stage holds; never multiplied), and a partial last tile multiplies its missing half with
+  // does not exist (whatever the stage holds; never multiplied), and a partial last tile multiplies what it lacks with
   // zeros.
   constexpr int INFLIGHT = LB + (NA - 2) * LT;
   static_assert(NB >= NA, "B must not be needed before A under the in-order bound");
@@ -505,7 +506,7 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
   for (int t = 0; t < KT; ++t) {
     const int ta = min(t + NA - 1, KT - 1), tb = min(t + NB - 1, KT - 1);
     const bool pa = ktail && ta == KT - 1, pb = ktail && tb == KT - 1;
-    const bool zero_hi = ktail && t == KT - 1;
+    const bool last_partial = ktail && t == KT - 1;
     const int sla = (ca + NA - 1) & (NA - 1);        // NA is a power of two
     const int slb = cb == 0 ? NB - 1 : cb - 1;
     frags(ca, cb, 1, 1);
@@ -520,10 +521,17 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
         __builtin_amdgcn_sched_barrier(0);
       }
     };
+    // partial last tile: a lane's A fragment of slice kk covers k = (2 kk + half) * 8 .. + 7; those past ktail become zero
+    if (last_partial && half * 8 >= ktail) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) af[0][i][e] = (T)0.0f;
+    }
 #pragma unroll
     for (int m = 0; m < NMF; ++m) { mfma_one(0, m); slot(m); }
     __builtin_amdgcn_sched_barrier(0);
-    if (zero_hi) {
+    if (last_partial && (2 + half) * 8 >= ktail) {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -669,7 +677,7 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
 
 // The ring kernels take plain row-major output and 16-byte friendly operands whose per-lane byte offsets fit 32 bits.
 static bool ring_ok(const GemmArgs& g) {
-  if (g.epi != EPI_PLAIN || g.cn != 1 || g.N < 8 || g.N % 8 || g.K % 16) return false;
+  if (g.epi != EPI_PLAIN || g.cn != 1 || g.N < 8 || g.N % 8 || g.K % 8) return false;
   if (!aligned(g.A, 16) || !aligned(g.B, 16) || !aligned(g.C, 16)) return false;
   if (g.lda % 8 || g.sA % 8 || g.ldb % 8 || g.sB % 8 || g.ldc % 8 || g.sC % 8) return false;
   const int64_t lim = (int64_t)1 << 32;

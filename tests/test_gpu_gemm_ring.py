@@ -42,8 +42,9 @@ def _without_ring(fn):
 
 TILED = {"algo": 2}
 
-# (M, in, out): multiples and non-multiples of 256; K = in with K % 32 in {0, 16}; K below / above the prefetch depth
-DENSE_SHAPES = [(17, 64, 64), (300, 176, 1000), (256, 32, 256), (257, 16, 264), (513, 4096, 520), (700, 688, 1376), (2048, 256, 512)]
+# (M, in, out): multiples and non-multiples of 256; K = in with K % 32 in {0, 8, 16, 24}; K below / above the prefetch depth
+DENSE_SHAPES = [(17, 64, 64), (300, 176, 1000), (256, 32, 256), (257, 16, 264), (513, 4096, 520), (700, 688, 1376), (2048, 256, 512),
+                (100, 8, 72), (130, 24, 136), (300, 72, 576), (260, 216, 264), (64, 40, 64)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
