@@ -194,8 +194,12 @@ def main():
         st = torch.cuda.current_stream().cuda_stream
         for i in range(24):
             pf[i % 4][0](st)
+        dn = [mk_dense(2048, *LAYERS["gate_up"][:2]) for _ in range(2)]
+        for i in range(8):
+            dn[i % 2][0](st)
         torch.cuda.synchronize()
-        print(json.dumps({"pmc": "prefill", "launches": 24, "flops": blast_bytes_flops(2048, 4096, 1024, 22016)[1]}))
+        print(json.dumps({"pmc": "prefill", "launches": 24, "flops": blast_bytes_flops(2048, 4096, 1024, 22016)[1],
+                          "dense_launches": 8, "dense_flops": 2.0 * 2048 * 4096 * 22016}))
         return
     if args.pmc == "dominant":
         gu = [mk_blast(1, *LAYERS["gate_up"][:2], LAYERS["gate_up"][2], L.U_RQ, L.S_JIR) for _ in range(12)]
