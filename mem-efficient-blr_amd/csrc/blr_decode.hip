@@ -1187,7 +1187,10 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     const int nch = (vecs + lpr - 1) / lpr;
     const int base = bo * nch;
     if (base > resident) return d2_bail(__LINE__);
-    int ks = e_ks > 0 ? e_ks : resident / base;
+    // BLAST proper (b output blocks): no k split of stage 2 - handing partial outputs of up to 16 rows between workgroups
+    // costs more than the shorter slabs save (measured at every M from 5 to 16); low rank and Monarch keep the split
+    const bool no_split = bo == b && bo > 1 && a.perm_per == 0;
+    int ks = e_ks > 0 ? e_ks : (no_split ? 1 : resident / base);
     if (ks > e_ksmax) ks = e_ksmax;
     if (ks > resident / base) ks = resident / base;
     if (ks < 1) ks = 1;
@@ -1288,7 +1291,10 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     static const int e_ks = env_i("BLR_DM_KS2", 0), e_ksmax = env_i("BLR_DM_KS2_MAX", 4);
     const int nch = (Q + 127) / 128, base = bo * nch;
     if (base > resident) return d2_bail(__LINE__);
-    int ks = e_ks > 0 ? e_ks : resident / base;
+    // BLAST proper (b output blocks): no k split of stage 2 - handing partial outputs of up to 16 rows between workgroups
+    // costs more than the shorter slabs save (measured at every M from 5 to 16); low rank and Monarch keep the split
+    const bool no_split = bo == b && bo > 1 && a.perm_per == 0;
+    int ks = e_ks > 0 ? e_ks : (no_split ? 1 : resident / base);
     if (ks > e_ksmax) ks = e_ksmax;
     if (ks > 4) ks = 4;
     if (ks > resident / base) ks = resident / base;
