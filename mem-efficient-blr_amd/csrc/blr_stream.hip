@@ -343,7 +343,14 @@ __device__ __forceinline__ void phase_kn(const PhaseDesc& d, int M, float* smem,
     int kk = rs;
     Raw8<WB> raw[UNR];
     bool have_raw = false;
-    if (VEC && it.col_ok && kk + (UNR - 1) * rpp < kc) {
+    // Whole chunk inside the matrix and room for one batch of zero activations behind the slice: every batch is full and
+    // every load unconditional (rows past the slice are fetched from its last row and multiplied by zeros) - a load under
+    // a condition makes the compiler wait for all loads in flight at every use.
+    const bool fast = VEC && n0 + NC <= d.N && kc + UNR * rpp <= KC_LD;
+    if (fast) {
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) raw[u] = load_raw8<WB>(d.W, it.wbase + (int64_t)min(kk + u * rpp, kc - 1) * d.ldw);
+    } else if (VEC && it.col_ok && kk + (UNR - 1) * rpp < kc) {
 #pragma unroll
       for (int u = 0; u < UNR; ++u) raw[u] = load_raw8<WB>(d.W, it.wbase + (int64_t)(kk + u * rpp) * d.ldw);
       have_raw = true;
@@ -363,6 +370,12 @@ __device__ __forceinline__ void phase_kn(const PhaseDesc& d, int M, float* smem,
         a_s[m * KC_LD + ka] = (m < M) ? act_load<T>(d, M, bt, m, it.k0 + ka, zcur) : 0.0f;
       }
     }
+    if (fast) {
+      for (int idx = tid; idx < MT * UNR * rpp; idx += 256) {
+        const int m = idx / (UNR * rpp), ka = idx - m * (UNR * rpp);
+        a_s[m * KC_LD + kc + ka] = 0.0f;
+      }
+    }
     __syncthreads();
     TR(trb + 1);
 
@@ -371,7 +384,23 @@ __device__ __forceinline__ void phase_kn(const PhaseDesc& d, int M, float* smem,
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[m][e] = 0.0f;
-    if (it.col_ok) {
+    if (fast) {
+      for (int kcur = kk; kcur < kc; kcur += UNR * rpp) {
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+          float w[8];
+          raw_to_f32<T>(raw[u], w);
+          raw[u] = load_raw8<WB>(d.W, it.wbase + (int64_t)min(kcur + (UNR + u) * rpp, kc - 1) * d.ldw);   // refill the slot right away
+          const int k = kcur + u * rpp;
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            const float a = a_s[m * KC_LD + k];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[m][e] = fmaf(a, w[e], acc[m][e]);
+          }
+        }
+      }
+    } else if (it.col_ok) {
       if (VEC) {
         while (have_raw) {
           const int kcur = kk;
