@@ -63,6 +63,9 @@ typedef enum { BLR_W2_SR = 0, BLR_W2_RS = 1 } blr_w2_layout;
  * out[n, ll*S + s] of the right_ideal names (reference triton_funcs/monarch_kernels.py:1004). */
 typedef enum { BLR_OUT_INTERLEAVED = 0, BLR_OUT_BLOCKED = 1 } blr_monarch_out;
 
+/* Activation of the fused output stage (the *_fwd_ep entry points). */
+typedef enum { BLR_ACT_NONE = 0, BLR_ACT_GELU_TANH = 1, BLR_ACT_SILU = 2 } blr_act;
+
 const char* blr_last_error(void);
 int blr_version(void);
 /* Number of compute units of the current device (0 if no device). */
@@ -156,6 +159,29 @@ int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t 
  * low_rank_kernels.py:419-450): an empirical bandwidth ceiling for the decode kernels.        */
 int blr_probe_dst_words(void);
 int blr_stream_probe(const void* src, size_t bytes, void* dst, void* stream);
+
+/* ---- fused output stage ---------------------------------------------------------------------
+ * out = act(op(x) + bias): what the callers do right after the operator - the bias add of the wrapper
+ * modules (reference models/wrappers.py:176-177) and the activation that follows the first MLP linear
+ * (GELU-tanh in DiT, reference DiT/models.py:111-112; SiLU in Llama).  bias: out_f values of dtype or NULL;
+ * act: blr_act.  The other arguments are those of the entry point without the suffix.  On the tiled path
+ * (M > 16) bias and activation are applied while the last GEMM writes its tile out (to the result rounded
+ * to dtype, as the callers' separate kernels would), so the M x out_f round trip of those kernels
+ * disappears; on the streaming path (M <= 16) a small elementwise launch follows the operator.   */
+int blr_blast_fwd_ep(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                     void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
+                     int dtype, int u_layout, int s_layout, int algo,
+                     void* ws, size_t ws_bytes, void* stream, const void* bias, int act);
+int blr_monarch_fwd_ep(const void* x, int64_t ldx, const void* w1, const void* w2,
+                       void* out, int64_t ldo, int M, int in_f, int out_f, int b, int rank,
+                       int dtype, int w2_layout, int out_order, int algo,
+                       void* ws, size_t ws_bytes, void* stream, const void* bias, int act);
+int blr_low_rank_fwd_ep(const void* x, int64_t ldx, const void* A, const void* B,
+                        void* out, int64_t ldo, int M, int in_f, int out_f, int r, int dtype, int algo,
+                        void* ws, size_t ws_bytes, void* stream, const void* bias, int act);
+int blr_dense_fwd_ep(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
+                     int M, int in_f, int out_f, int dtype, int algo,
+                     void* ws, size_t ws_bytes, void* stream, const void* bias, int act);
 
 #ifdef __cplusplus
 }

@@ -157,6 +157,50 @@ static int quantize_t(const void* w, int64_t outer, int64_t reduce, int64_t inne
   return BLR_OK;
 }
 
+// ---- fused output stage ------------------------------------------------------------------------------
+// The *_fwd_ep entry points arm this per-thread record and call the plain entry point; the tiled path attaches it
+// to its last GEMM (attach_epilogue), any other path leaves it and the entry point finishes with bias_act_kernel.
+struct PendingEpilogue { const void* bias; int act; bool armed; bool used; };
+static thread_local PendingEpilogue tl_ep = {nullptr, 0, false, false};
+
+static void attach_epilogue(GemmArgs& g) {
+  if (!tl_ep.armed) return;
+  g.bias = tl_ep.bias; g.act = tl_ep.act;
+  tl_ep.used = true;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bias_act_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ bias, int act, int M, int N) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * N) return;
+  const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
+  float v = TypeTraits<T>::to_f32(out[(int64_t)m * ldo + n]);
+  if (bias) v += TypeTraits<T>::to_f32(bias[n]);
+  out[(int64_t)m * ldo + n] = TypeTraits<T>::from_f32(apply_act(v, act));
+}
+
+static int bias_act_launch(void* out, int64_t ldo, const void* bias, int act, int M, int N, int dtype, hipStream_t st) {
+  if (!bias && !act) return BLR_OK;
+  const unsigned grid = (unsigned)cdiv((int64_t)M * N, 256);
+  if (dtype == BLR_F16) hipLaunchKernelGGL(bias_act_kernel<f16>, dim3(grid), dim3(256), 0, st, (f16*)out, ldo, (const f16*)bias, act, M, N);
+  else if (dtype == BLR_BF16) hipLaunchKernelGGL(bias_act_kernel<bf16>, dim3(grid), dim3(256), 0, st, (bf16*)out, ldo, (const bf16*)bias, act, M, N);
+  else hipLaunchKernelGGL(bias_act_kernel<float>, dim3(grid), dim3(256), 0, st, (float*)out, ldo, (const float*)bias, act, M, N);
+  BLR_CHECK_LAUNCH("bias_act");
+  return BLR_OK;
+}
+
+// Runs `call` (a plain entry point) with the epilogue armed and finishes whatever the call did not fuse.
+template <typename F>
+static int with_epilogue(const void* bias, int act, void* out, int64_t ldo, int M, int out_f, int dtype, void* stream, F&& call) {
+  if (act < BLR_ACT_NONE || act > BLR_ACT_SILU) { set_error("epilogue: unknown activation %d", act); return BLR_ERR_BAD_ARG; }
+  tl_ep = {bias, act, (bias != nullptr) || act != BLR_ACT_NONE, false};
+  const int rc = call();
+  const bool used = tl_ep.used, armed = tl_ep.armed;
+  tl_ep = {nullptr, 0, false, false};
+  if (rc != BLR_OK || !armed || used) return rc;
+  return bias_act_launch(out, ldo, bias, act, M, out_f, dtype, (hipStream_t)stream);
+}
+
 }  // namespace blr
 
 using namespace blr;
@@ -233,6 +277,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   else { g2.b_kn = 0; g2.ldb = r; g2.sB = (int64_t)Q * r; }
   g2.C = out; g2.ldc = ldo; g2.sC = Q; g2.cn = 1;
   g2.M = M; g2.N = Q; g2.K = r; g2.batch = b;
+  if (!sat8) attach_epilogue(g2);
   return gemm_launch(g2, dtype, st);
 }
 
@@ -409,6 +454,7 @@ int blr_monarch_fwd(const void* x, int64_t ldx, const void* w1, const void* w2,
   if (out_order == BLR_OUT_INTERLEAVED) { g2.sC = 1; g2.cn = b; }
   else { g2.sC = S; g2.cn = 1; }
   g2.M = M; g2.N = S; g2.K = rank; g2.batch = b;
+  attach_epilogue(g2);
   return gemm_launch(g2, dtype, st);
 }
 
@@ -454,6 +500,7 @@ int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
   GemmArgs g2 = {};
   g2.A = Z; g2.lda = r; g2.B = B; g2.ldb = out_f; g2.b_kn = 1;
   g2.C = out; g2.ldc = ldo; g2.cn = 1; g2.M = M; g2.N = out_f; g2.K = r; g2.batch = 1;
+  attach_epilogue(g2);
   return gemm_launch(g2, dtype, st);
 }
 
@@ -486,7 +533,43 @@ int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t 
   GemmArgs g = {};
   g.A = x; g.lda = ldx; g.B = W; g.ldb = out_f; g.b_kn = 1;
   g.C = out; g.ldc = ldo; g.cn = 1; g.M = M; g.N = out_f; g.K = in_f; g.batch = 1;
+  attach_epilogue(g);
   return gemm_launch(g, dtype, st);
+}
+
+// ---- fused output stage: out = act(op(x) + bias) ------------------------------------------------------
+int blr_blast_fwd_ep(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                     void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
+                     int dtype, int u_layout, int s_layout, int algo,
+                     void* ws, size_t ws_bytes, void* stream, const void* bias, int act) {
+  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
+    return blr_blast_fwd(x, ldx, U, V, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, u_layout, s_layout, algo, ws, ws_bytes, stream);
+  });
+}
+
+int blr_monarch_fwd_ep(const void* x, int64_t ldx, const void* w1, const void* w2,
+                       void* out, int64_t ldo, int M, int in_f, int out_f, int b, int rank,
+                       int dtype, int w2_layout, int out_order, int algo,
+                       void* ws, size_t ws_bytes, void* stream, const void* bias, int act) {
+  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
+    return blr_monarch_fwd(x, ldx, w1, w2, out, ldo, nullptr, M, in_f, out_f, b, rank, dtype, w2_layout, out_order, algo, ws, ws_bytes, stream);
+  });
+}
+
+int blr_low_rank_fwd_ep(const void* x, int64_t ldx, const void* A, const void* B,
+                        void* out, int64_t ldo, int M, int in_f, int out_f, int r, int dtype, int algo,
+                        void* ws, size_t ws_bytes, void* stream, const void* bias, int act) {
+  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
+    return blr_low_rank_fwd(x, ldx, A, B, out, ldo, nullptr, M, in_f, out_f, r, dtype, algo, ws, ws_bytes, stream);
+  });
+}
+
+int blr_dense_fwd_ep(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
+                     int M, int in_f, int out_f, int dtype, int algo,
+                     void* ws, size_t ws_bytes, void* stream, const void* bias, int act) {
+  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
+    return blr_dense_fwd(x, ldx, W, out, ldo, M, in_f, out_f, dtype, algo, ws, ws_bytes, stream);
+  });
 }
 
 }  // extern "C"

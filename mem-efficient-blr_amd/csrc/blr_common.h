@@ -55,6 +55,15 @@ template <> struct TypeTraits<float> {
 // Round to nearest even, then clamp to the int8 range (reference blast_sym_quant_kernels.py:105-108: nearbyint, clamp).
 __device__ __forceinline__ float sat8_rne(float v) { return fminf(fmaxf(rintf(v), -128.0f), 127.0f); }
 
+// Activation of the fused output stage (blr_act): GELU with the tanh approximation (what the reference's DiT uses,
+// DiT/models.py:111: approx_gelu = nn.GELU(approximate="tanh")) or SiLU (Llama's gate).
+__device__ __forceinline__ float apply_act(float v, int act) {
+  // 0.5 v (1 + tanh u) = v / (1 + exp(-2u)), u = sqrt(2/pi) (v + 0.044715 v^3): one exponential and one reciprocal
+  if (act == BLR_ACT_GELU_TANH) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-1.5957691216057308f * (v + 0.044715f * v * v * v)));
+  if (act == BLR_ACT_SILU) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+  return v;
+}
+
 // 16-byte global load / store of 8 two-byte elements (pointer must be 16-byte aligned).
 template <typename V> __device__ __forceinline__ V ldg16(const void* p) {
   return *reinterpret_cast<const V*>(p);
@@ -95,6 +104,8 @@ struct GemmArgs {
   int per;          // EPI_MONARCH_SCATTER: column c of batch kk -> C[(c/per)*sL + m*ldc + kk*per + c%per]
   int64_t sL;
   int sat8;         // 1: the fp32 result is rounded to nearest even and clamped to [-128, 127] before it is stored
+  const void* bias; // optional: values of dtype added to the rounded result, indexed by the element's offset inside its row of C
+  int act;          // blr_act applied after the bias
 };
 // dtype: blr_dtype.  Returns blr_status.
 int gemm_launch(const GemmArgs& a, int dtype, hipStream_t st);

@@ -163,7 +163,30 @@ __device__ __forceinline__ int64_t epi_offset(const GemmArgs& g, int bt, int m, 
   return (int64_t)bt * g.sC + (int64_t)m * g.ldc + (int64_t)n * g.cn;
 }
 
-template <typename T, int BM, int BN, bool B_KN, int PD>
+// Fused output stage (kernels instantiated with EP): bias (indexed by the element's offset inside its row of C) and
+// activation are applied to the rounded result on its way out, like the separate kernels of the callers would.  The
+// plain instantiations do not contain this code: it costs registers that the main loops need.
+template <typename T>
+__device__ __forceinline__ T ep_value(const GemmArgs& g, T r, int64_t in_row) {
+  float v = TypeTraits<T>::to_f32(r);
+  if (g.bias) v += TypeTraits<T>::to_f32(reinterpret_cast<const T*>(g.bias)[in_row]);
+  return TypeTraits<T>::from_f32(apply_act(v, g.act));
+}
+
+// eight consecutive outputs; their offset inside the row is a multiple of 8, so the bias comes as one 16-byte load
+template <typename T>
+__device__ __forceinline__ typename TypeTraits<T>::vec8 ep_vector(const GemmArgs& g, typename TypeTraits<T>::vec8 r, int64_t in_row) {
+  using V8 = typename TypeTraits<T>::vec8;
+  V8 bv;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) bv[e] = (T)0.0f;
+  if (g.bias) bv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(g.bias) + in_row);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = TypeTraits<T>::from_f32(apply_act(TypeTraits<T>::to_f32(r[e]) + TypeTraits<T>::to_f32(bv[e]), g.act));
+  return r;
+}
+
+template <typename T, int BM, int BN, bool B_KN, int PD, bool EP = false>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int a_vec, int b_vec, int c_vec,
                                                         int per_xcd, int group_m) {
   constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
@@ -308,8 +331,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
     for (int v = tid; v < BM * VPR; v += 256) {
       int row = v / VPR, cvec = (v - row * VPR) * 8;
       int gr = m0 + row, gc = n0 + cvec;
-      if (gr < g.M && gc < g.N)
-        *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
+      if (gr < g.M && gc < g.N) {
+        V8 v = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
+        if (EP) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc);
+        *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = v;
+      }
     }
     return;
   }
@@ -321,7 +347,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         int row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row < g.M && col < g.N) C[epi_offset(g, bt, row, col)] = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][e]) : acc[i][j][e]);
+        if (row < g.M && col < g.N) {
+          const int64_t off = epi_offset(g, bt, row, col);
+          T v = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][e]) : acc[i][j][e]);
+          if (EP) v = ep_value<T>(g, v, off - (int64_t)row * g.ldc);
+          C[off] = v;
+        }
       }
     }
 }
@@ -354,7 +385,7 @@ __device__ __forceinline__ uint32_t ring_lds_addr(const void* p) {
   return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((void __attribute__((address_space(3)))*)(p)));
 }
 
-template <typename T, bool B_KN, int BM, int BN>
+template <typename T, bool B_KN, int BM, int BN, bool EP = false>
 __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
   constexpr int NA = RING_NA, NB = RING_NB;
   constexpr int ASTG = BM * 64, BSTG = BN * 64, BRING = NA * ASTG;   // stage sizes, start of the B ring
@@ -571,8 +602,11 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
   for (int v = tid; v < BM * VPR; v += 256) {
     const int row = v / VPR, cvec = (v - row * VPR) * 8;
     const int gr = m0 + row, gc = n0 + cvec;
-    if (gr < g.M && gc < g.N)
-      *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
+    if (gr < g.M && gc < g.N) {
+      V8 v = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
+      if (EP) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc);
+      *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = v;
+    }
   }
 }
 
@@ -626,12 +660,18 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) 
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       int row = m0 + ty * 4 + i, col = n0 + tx * 4 + j;
-      if (row < g.M && col < g.N) C[epi_offset(g, bt, row, col)] = g.sat8 ? sat8_rne(acc[i][j]) : acc[i][j];
+      if (row < g.M && col < g.N) {
+        const int64_t off = epi_offset(g, bt, row, col);
+        float v = g.sat8 ? sat8_rne(acc[i][j]) : acc[i][j];
+        if (g.bias || g.act) v = ep_value<float>(g, v, off - (int64_t)row * g.ldc);
+        C[off] = v;
+      }
     }
 }
 
 template <typename T, int BM, int BN, bool B_KN>
-static void* mfma_kernel_ptr(int pd) {
+static void* mfma_kernel_ptr(int pd, bool ep) {
+  if (ep) return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 2, true>;
   switch (pd) {
     case 1: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 1>;
     case 3: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 3>;
@@ -645,11 +685,13 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   // 16-byte vector accesses need every row start and every k (or n) offset to be 16-byte aligned.
   int a_vec = aligned(g.A, 16) && g.lda % 8 == 0 && g.sA % 8 == 0;
   int b_vec = aligned(g.B, 16) && g.ldb % 8 == 0 && g.sB % 8 == 0;
-  int c_vec = g.epi == EPI_PLAIN && g.cn == 1 && aligned(g.C, 16) && g.ldc % 8 == 0 && g.sC % 8 == 0 && g.N % 8 == 0;
+  int c_vec = g.epi == EPI_PLAIN && g.cn == 1 && aligned(g.C, 16) && g.ldc % 8 == 0 && g.sC % 8 == 0 && g.N % 8 == 0 &&
+              (!g.bias || aligned(g.bias, 16));
   size_t lds = 2 * sizeof(GemmSmem<T, BM, BN>);
   // k-tiles of global loads kept in flight (tuning aid: BLR_GEMM_PD = 1, 2 or 3)
   static const int pd = [] { const char* e = getenv("BLR_GEMM_PD"); return e ? atoi(e) : 2; }();
-  void* fn = g.b_kn ? mfma_kernel_ptr<T, BM, BN, true>(pd) : mfma_kernel_ptr<T, BM, BN, false>(pd);
+  const bool ep = g.bias != nullptr || g.act != 0;
+  void* fn = g.b_kn ? mfma_kernel_ptr<T, BM, BN, true>(pd, ep) : mfma_kernel_ptr<T, BM, BN, false>(pd, ep);
   static std::mutex mu;
   static std::set<void*> raised;
   {
@@ -678,7 +720,7 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
 // The ring kernels take plain row-major output and 16-byte friendly operands whose per-lane byte offsets fit 32 bits.
 static bool ring_ok(const GemmArgs& g) {
   if (g.epi != EPI_PLAIN || g.cn != 1 || g.N < 8 || g.N % 8 || g.K % 8) return false;
-  if (!aligned(g.A, 16) || !aligned(g.B, 16) || !aligned(g.C, 16)) return false;
+  if (!aligned(g.A, 16) || !aligned(g.B, 16) || !aligned(g.C, 16) || (g.bias && !aligned(g.bias, 16))) return false;
   if (g.lda % 8 || g.sA % 8 || g.ldb % 8 || g.sB % 8 || g.ldc % 8 || g.sC % 8) return false;
   const int64_t lim = (int64_t)1 << 32;
   if ((int64_t)(g.M - 1) * g.lda * 2 + 64 >= lim) return false;
@@ -690,7 +732,9 @@ template <typename T, int BM, int BN>
 static int launch_ring(const GemmArgs& g, hipStream_t st) {
   int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
   const size_t lds = ring_lds_bytes<BM, BN>();
-  void* fn = g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN> : (void*)gemm_ring_kernel<T, false, BM, BN>;
+  const bool ep = g.bias != nullptr || g.act != 0;
+  void* fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true> : (void*)gemm_ring_kernel<T, false, BM, BN, true>)
+                : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN> : (void*)gemm_ring_kernel<T, false, BM, BN>);
   static std::mutex mu;
   static std::set<void*> raised;
   {

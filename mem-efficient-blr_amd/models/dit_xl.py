@@ -56,7 +56,10 @@ class Mlp(nn.Module):
         self.fc2 = nn.Linear(hidden, dim)
 
     def forward(self, x):
-        return self.fc2(self.act(self.fc1(x)))
+        h = self.fc1(x)
+        if getattr(self.fc1, "fused_act", None) is None:     # a structured fc1 applies the GELU in its kernel's output stage
+            h = self.act(h)
+        return self.fc2(h)
 
 
 class DiTBlock(nn.Module):
@@ -133,6 +136,9 @@ class CustomDiT(nn.Module):
         self.replaced = 0
         if layer_configs is not None and method is not None:
             self.replaced = replace_linear_with_custom(self.model.blocks, layer_configs, method)
+            for blk in self.model.blocks:                    # hand the MLP's activation to a structured fc1
+                if hasattr(blk.mlp.fc1, "fused_act"):
+                    blk.mlp.fc1.fused_act = "gelu_tanh"
 
     def forward(self, x, t, y):
         return self.model(x, t, y)

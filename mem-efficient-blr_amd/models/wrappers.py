@@ -7,7 +7,9 @@ exactly as in the reference:
   "torch"  in name -> baseline layouts, function returns a tuple whose first item is the output;
   BLAST   "bmm" in name  -> U (b, q, r), S (r, b, b), else U (b, r, q), S (b, b, r); V (b, p, r)
   Monarch "left" in name -> w2 (b, r, s), else (b, s, r); w1 (b, p, r)
-The bias is added as `out += bias.to(x.dtype)` (reference wrappers.py:176-177).
+The bias is added as `out += bias.to(x.dtype)` (reference wrappers.py:176-177); with a library kernel
+("triton" names other than the quantized one) the bias - and an activation the owner of the module asks
+for by setting `fused_act` ("gelu_tanh" or "silu") - is handed to the kernel's output stage instead.
 Factors are drawn with std 1/sqrt(fan-in of the factor) instead of the reference's std 1, so that
 fp16 activations stay in range at the ranks the networks use.
 """
@@ -37,15 +39,31 @@ class _StructuredLinear(nn.Module):
             self.bias = nn.Parameter(torch.randn(out_features, device=device, dtype=dtype))
         else:
             self.register_parameter("bias", None)
+        self.fused_act = None          # set by the owner (e.g. an MLP) to have its activation applied by the kernel
+        self.fuses = self.kind == "triton" and not is_compiled and "int8" not in self.func_name and "int4" not in self.func_name
 
     def _param(self, shape, fan_in):
         return nn.Parameter(torch.randn(shape, device=self.device, dtype=torch.float32).mul_(1.0 / math.sqrt(fan_in)).to(self.dtype))
 
-    def _finish(self, out):
+    def _call(self, *args):
+        """The forward function; library kernels take bias and activation into their output stage."""
+        if not self.fuses or (self.bias is None and self.fused_act is None):
+            return self.func(*args), False
+        from triton_funcs import _lib as L
+        with L.fused_epilogue(self.bias, self.fused_act):
+            return self.func(*args), True
+
+    def _finish(self, out, fused=False):
         if self.kind == "torch" and isinstance(out, tuple):
             out = out[0]
+        if fused:
+            return out
         if self.bias is not None:
             out += self.bias.to(out.dtype)
+        if self.fused_act == "gelu_tanh":
+            out = torch.nn.functional.gelu(out, approximate="tanh")
+        elif self.fused_act == "silu":
+            out = torch.nn.functional.silu(out)
         return out
 
 
@@ -66,7 +84,7 @@ class BlastLinear(_StructuredLinear):
             self.S = self._param((b, b, rank), 1)
 
     def forward(self, x):
-        return self._finish(self.func(x, self.U, self.V, self.S))
+        return self._finish(*self._call(x, self.U, self.V, self.S))
 
     def extra_repr(self):
         return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
@@ -103,7 +121,7 @@ class MonarchLinear(_StructuredLinear):
             self.w2_bfly = self._param((b, s, rank), rank)
 
     def forward(self, x):
-        return self._finish(self.func(x, self.w1_bfly, self.w2_bfly))
+        return self._finish(*self._call(x, self.w1_bfly, self.w2_bfly))
 
     def extra_repr(self):
         return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
@@ -122,10 +140,10 @@ class LowRankLinear(_StructuredLinear):
             self.U = self._param((out_features, rank), rank)
 
     def forward(self, x):
-        out = self.func(x, self.V, self.U)
+        out, fused = self._call(x, self.V, self.U)
         if self.kind == "triton":                      # the kernel returns (N, out_f): restore the leading dims
             out = out.reshape(*x.shape[:-1], self.out_features)
-        return self._finish(out)
+        return self._finish(out, fused)
 
     def extra_repr(self):
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, rank={self.rank}, func={self.func_name}"
@@ -138,10 +156,10 @@ class DenseLinear(_StructuredLinear):
         self.W = self._param(shape, in_features)
 
     def forward(self, x):
-        out = self.func(x, self.W)
+        out, fused = self._call(x, self.W)
         if self.kind == "triton":
             out = out.reshape(*x.shape[:-1], self.out_features)
-        return self._finish(out)
+        return self._finish(out, fused)
 
     def extra_repr(self):
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, func={self.func_name}"

@@ -22,6 +22,8 @@ S_JIR, S_RIJ, S_IJR = 0, 1, 2
 ALGO_AUTO, ALGO_STREAM, ALGO_TILED, ALGO_FUSED, ALGO_STREAM_SPLIT = 0, 1, 2, 3, 4
 W2_SR, W2_RS = 0, 1
 OUT_INTERLEAVED, OUT_BLOCKED = 0, 1
+ACT_NONE, ACT_GELU_TANH, ACT_SILU = 0, 1, 2
+ACTS = {None: ACT_NONE, "none": ACT_NONE, "gelu_tanh": ACT_GELU_TANH, "silu": ACT_SILU}
 
 _c = ctypes
 _vp, _i, _i64, _sz = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_size_t
@@ -43,6 +45,10 @@ _SIGNATURES = {
     "blr_low_rank_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _i64, _vp] + [_i] * 6 + [_vp, _sz, _vp]),
     "blr_dense_workspace_bytes": (_sz, [_i] * 5),
     "blr_dense_fwd": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp]),
+    "blr_blast_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64] + [_i] * 9 + [_vp, _sz, _vp, _vp, _i]),
+    "blr_monarch_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 9 + [_vp, _sz, _vp, _vp, _i]),
+    "blr_low_rank_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 6 + [_vp, _sz, _vp, _vp, _i]),
+    "blr_dense_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp, _vp, _i]),
     "blr_probe_dst_words": (_i, []),
     "blr_stream_probe": (_i, [_vp, _sz, _vp, _vp]),
 }
@@ -127,3 +133,39 @@ def require_gpu(*tensors):
     for t in tensors:
         if not t.is_cuda:
             raise BlrError("libblr kernels need tensors on the GPU (there is no CPU path)")
+
+
+# ---- fused output stage ------------------------------------------------------------------------------
+# The operator functions keep the reference's signatures, so bias and activation reach them through a
+# per-thread context: inside ``with fused_epilogue(bias, act):`` the next structured-linear call returns
+# act(op(x) + bias), computed by the *_fwd_ep entry points (fused into the last GEMM at M > 16).
+_ep_state = threading.local()
+
+
+class fused_epilogue:
+    def __init__(self, bias=None, act=None):
+        if act not in ACTS:
+            raise BlrError(f"unknown activation {act!r}")
+        self.bias, self.act = bias, ACTS[act]
+
+    def __enter__(self):
+        self.prev = getattr(_ep_state, "ep", None)
+        _ep_state.ep = (self.bias, self.act) if (self.bias is not None or self.act) else None
+        return self
+
+    def __exit__(self, *exc):
+        _ep_state.ep = self.prev
+        return False
+
+
+def pending_epilogue(out_f, dtype, device):
+    """(bias pointer or None, activation code, keep-alive) of the active context, or None."""
+    ep = getattr(_ep_state, "ep", None)
+    if ep is None:
+        return None
+    bias, act = ep
+    if bias is not None:
+        if bias.numel() != out_f:
+            raise BlrError(f"bias has {bias.numel()} values, the operator {out_f} outputs")
+        bias = bias.detach().to(device=device, dtype=dtype).contiguous()
+    return (bias.data_ptr() if bias is not None else None), act, bias

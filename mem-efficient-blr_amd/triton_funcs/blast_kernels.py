@@ -71,11 +71,17 @@ def _blast(name, x, U, V, S, u_layout, s_layout, algo, want_intermediates):
     lib = L.lib()
     need = lib.blr_blast_workspace_bytes(M, in_f, out_f, b1, r, dt, algo)
     ws = L.workspace(x.device, need, algo, M, dt)
-    rc = lib.blr_blast_fwd(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
-                           out.data_ptr(), out.stride(0),
-                           z.data_ptr() if z is not None else None, y.data_ptr() if y is not None else None,
-                           M, in_f, out_f, b1, r, dt, u_layout, s_layout, algo,
-                           ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
+    ep = None if want_intermediates else L.pending_epilogue(out_f, x.dtype, x.device)
+    if ep is not None:
+        rc = lib.blr_blast_fwd_ep(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
+                                  out.data_ptr(), out.stride(0), M, in_f, out_f, b1, r, dt, u_layout, s_layout, algo,
+                                  ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1])
+    else:
+        rc = lib.blr_blast_fwd(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
+                               out.data_ptr(), out.stride(0),
+                               z.data_ptr() if z is not None else None, y.data_ptr() if y is not None else None,
+                               M, in_f, out_f, b1, r, dt, u_layout, s_layout, algo,
+                               ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
     L.check(rc, name)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": b1, "rank": r,
                           "algo": algo, "dtype": str(x.dtype)}

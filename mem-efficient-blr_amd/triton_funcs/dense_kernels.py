@@ -27,8 +27,13 @@ def _dense(name, x, w, algo):
     out = torch.empty((M, out_f), device=x.device, dtype=x.dtype)
     lib = L.lib()
     ws = L.workspace(x.device, lib.blr_dense_workspace_bytes(M, in_f, out_f, dt, algo), algo, M, dt)
-    rc = lib.blr_dense_fwd(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
-                           M, in_f, out_f, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
+    ep = L.pending_epilogue(out_f, x.dtype, x.device)
+    if ep is not None:
+        rc = lib.blr_dense_fwd_ep(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
+                                  M, in_f, out_f, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1])
+    else:
+        rc = lib.blr_dense_fwd(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
+                               M, in_f, out_f, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
     L.check(rc, name)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "algo": algo}
     return out

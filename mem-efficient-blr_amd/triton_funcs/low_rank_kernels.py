@@ -29,9 +29,14 @@ def _low_rank(name, x, a, b, algo, want_z):
     z = torch.empty((M, r), device=x.device, dtype=x.dtype) if want_z else None
     lib = L.lib()
     ws = L.workspace(x.device, lib.blr_low_rank_workspace_bytes(M, in_f, out_f, r, dt, algo), algo, M, dt)
-    rc = lib.blr_low_rank_fwd(x2.data_ptr(), x2.stride(0), a.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
-                              z.data_ptr() if z is not None else None,
-                              M, in_f, out_f, r, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
+    ep = None if want_z else L.pending_epilogue(out_f, x.dtype, x.device)
+    if ep is not None:
+        rc = lib.blr_low_rank_fwd_ep(x2.data_ptr(), x2.stride(0), a.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
+                                     M, in_f, out_f, r, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1])
+    else:
+        rc = lib.blr_low_rank_fwd(x2.data_ptr(), x2.stride(0), a.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
+                                  z.data_ptr() if z is not None else None,
+                                  M, in_f, out_f, r, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
     L.check(rc, name)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "rank": r, "algo": algo}
     return out, z

@@ -55,10 +55,16 @@ def _monarch(name, x, w1, w2, w2_layout, out_order, algo, want_out1):
         algo = L.ALGO_TILED
     lib = L.lib()
     ws = L.workspace(x.device, lib.blr_monarch_workspace_bytes(M, in_f, out_f, k, q, dt, algo), algo, M, dt)
-    rc = lib.blr_monarch_fwd(x2.data_ptr(), x2.stride(0), w1.data_ptr(), w2.data_ptr(), out.data_ptr(), out.stride(0),
-                             out1.data_ptr() if out1 is not None else None,
-                             M, in_f, out_f, k, q, dt, w2_layout, out_order, algo,
-                             ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
+    ep = None if want_out1 else L.pending_epilogue(out_f, x.dtype, x.device)
+    if ep is not None:
+        rc = lib.blr_monarch_fwd_ep(x2.data_ptr(), x2.stride(0), w1.data_ptr(), w2.data_ptr(), out.data_ptr(), out.stride(0),
+                                    M, in_f, out_f, k, q, dt, w2_layout, out_order, algo,
+                                    ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1])
+    else:
+        rc = lib.blr_monarch_fwd(x2.data_ptr(), x2.stride(0), w1.data_ptr(), w2.data_ptr(), out.data_ptr(), out.stride(0),
+                                 out1.data_ptr() if out1 is not None else None,
+                                 M, in_f, out_f, k, q, dt, w2_layout, out_order, algo,
+                                 ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
     L.check(rc, name)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": k, "rank": q, "algo": algo}
     return out.reshape(*x.shape[:-1], out_f), out1

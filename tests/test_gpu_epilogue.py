@@ -1,0 +1,102 @@
+"""GPU parity of the fused output stage, out = act(op(x) + bias), against the oracle plus numpy bias / activation.
+
+Covers the tiled path (bias and activation applied to the last GEMM's fp32 accumulators: register-staged and
+direct-to-LDS kernels, plain and interleaved outputs) and the streaming path (M <= 16, elementwise launch after the
+operator), through the C ABI and through the wrapper modules.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import blr_oracle as O
+from gpu_util import assert_close, blast_inputs, dev, rounded, say
+
+pytestmark = pytest.mark.gpu
+
+
+def _act(v, act):
+    if act == "gelu_tanh":
+        return 0.5 * v * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (v + 0.044715 * v ** 3)))
+    if act == "silu":
+        return v / (1.0 + np.exp(-v))
+    return v
+
+
+@pytest.mark.parametrize("ring", ["0", "2"])
+@pytest.mark.parametrize("act", [None, "gelu_tanh", "silu"])
+@pytest.mark.parametrize("M", [3, 16, 40, 300])
+def test_blast_bias_activation(M, act, ring):
+    from triton_funcs import blast_kernels as K, _lib as L
+    os.environ["BLR_GEMM_RING"] = ring
+    try:
+        b, p, q, r = 4, 32, 40, 64
+        dtype = torch.float16
+        x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=M)
+        bias = np.random.default_rng(M).standard_normal(b * q)
+        Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+        say(f"[case] epilogue blast M={M} act={act} ring={ring}")
+        with L.fused_epilogue(dev(bias, dtype), act):
+            out = K.triton_blast_full_fp16(dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype))
+        ref = O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0]
+        assert_close(out, _act(ref + rounded(bias, dtype), act), dtype, "blast + bias + act")
+        plain = K.triton_blast_full_fp16(dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype))   # context closed: no epilogue
+        assert_close(plain, ref, dtype, "plain call after the context")
+    finally:
+        os.environ.pop("BLR_GEMM_RING", None)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M", [5, 130])
+def test_dense_low_rank_monarch_bias_activation(M, dtype):
+    from triton_funcs import dense_kernels as D, low_rank_kernels as LR, _lib as L
+    from test_gpu_monarch_lowrank_dense import _ref_monarch, _run_monarch, monarch_inputs
+    rng = np.random.default_rng(M)
+    in_f, r, out_f = 128, 48, 200
+    x = rng.standard_normal((M, in_f)); w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)
+    a = rng.standard_normal((in_f, r)) / np.sqrt(in_f); bm = rng.standard_normal((r, out_f)) / np.sqrt(r)
+    bias = rng.standard_normal(out_f)
+    say(f"[case] epilogue dense / low rank / monarch M={M} {dtype}")
+    f16 = dtype != torch.float32
+    with L.fused_epilogue(dev(bias, dtype), "silu"):
+        out = (D.triton_dense_fp16 if f16 else D.triton_dense_fp32)(dev(x, dtype), dev(w, dtype))
+    assert_close(out, _act(rounded(x, dtype) @ rounded(w, dtype) + rounded(bias, dtype), "silu"), dtype, "dense")
+    with L.fused_epilogue(dev(bias, dtype), "gelu_tanh"):
+        out = LR.triton_low_rank_fp16(dev(x, dtype), dev(a, dtype), dev(bm, dtype)) if f16 else None
+    if f16:
+        assert_close(out, _act((rounded(x, dtype) @ rounded(a, dtype)) @ rounded(bm, dtype) + rounded(bias, dtype), "gelu_tanh"), dtype, "low rank", scale=2.0)
+        # Monarch with interleaved output: the bias index is the final feature index
+        xm, w1_t, w2_t = monarch_inputs(4, 16, 32, 24, (M,), seed=3)
+        mb = rng.standard_normal(4 * 24)
+        with L.fused_epilogue(dev(mb, dtype), None):
+            out = _run_monarch("triton_monarch_right_fp16", xm, w1_t, w2_t, dtype)
+        assert_close(out, _ref_monarch(xm, w1_t, w2_t, dtype)[0] + rounded(mb, dtype), dtype, "monarch + bias", scale=2.0)
+
+
+def test_wrapper_modules_fuse_bias_and_activation():
+    """BlastLinear with a bias (and an activation requested by its owner) equals the unfused computation."""
+    from models import wrappers as W
+    torch.manual_seed(0)
+    lin = W.BlastLinear(256, 320, 4, 64, "triton_funcs.blast_kernels.triton_blast_full_fp16", torch.device("cuda"), torch.float16, bias=True)
+    x = torch.randn(2, 150, 256, device="cuda", dtype=torch.float16)
+    with torch.no_grad():
+        fused = lin(x)
+        lin.fuses = False
+        plain = lin(x)
+        assert_close(fused, plain.double().cpu().numpy(), torch.float16, "bias fused vs added")
+        lin.fuses, lin.fused_act = True, "gelu_tanh"
+        fused = lin(x)
+        lin.fuses = False
+        plain = lin(x)
+        assert_close(fused, plain.double().cpu().numpy(), torch.float16, "bias + gelu fused vs separate")
+
+
+def test_bad_activation_is_rejected():
+    from triton_funcs import _lib as L
+    lib = L.lib()
+    t = torch.zeros(64, device="cuda", dtype=torch.float16)
+    rc = lib.blr_dense_fwd_ep(t.data_ptr(), 8, t.data_ptr(), t.data_ptr(), 8, 1, 8, 8, 0, 0, None, 0, None, None, 7)
+    assert rc == -1 and b"activation" in lib.blr_last_error()
+    with pytest.raises(L.BlrError):
+        L.fused_epilogue(None, "relu")
