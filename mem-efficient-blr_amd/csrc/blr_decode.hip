@@ -1163,14 +1163,16 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   }
   if (a.u_layout == BLR_U_QR) {
     // stage 2 on U (bo, q, r): a wave takes rpw rows, a lane 8 of every 512 k; everything a lane loads stays in registers
+    // shapes this geometry does not hold (rows of a wave times k pieces beyond the registers of a lane) go to the
+    // matrix-core variant, which takes this layout at any M
     const int KL = (R + 511) / 512;
-    if (KL != 1 && KL != 2 && KL != 4 && KL != 8) return d2_bail(__LINE__);
-    if (KL * 512 * MT > D2_AS) return d2_bail(__LINE__);
+    if (KL != 1 && KL != 2 && KL != 4 && KL != 8) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
+    if (KL * 512 * MT > D2_AS) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
     const int pf_cap = d2_pf(MT, 16);
     int rpw = (int)cdiv((int64_t)bo * Q, (int64_t)resident * 4);
     if (rpw < 1) rpw = 1;
     while ((int64_t)bo * cdiv(Q, 4 * rpw) > resident) ++rpw;
-    if (rpw * KL > pf_cap) return d2_bail(__LINE__);
+    if (rpw * KL > pf_cap) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
     p.u_nk = 1; p.rpw = rpw; p.kl_log2 = ilog2(KL);
     p.lpr2_log2 = 4; p.nch2 = (int)cdiv(Q, 4 * rpw); p.ks2 = 1; p.kc2 = R; p.items2 = bo * p.nch2;
     p.pfn = rpw * KL; p.kpad2 = KL * 512;
@@ -1187,10 +1189,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     const int nch = (vecs + lpr - 1) / lpr;
     const int base = bo * nch;
     if (base > resident) return d2_bail(__LINE__);
-    // BLAST proper (b output blocks): no k split of stage 2 - handing partial outputs of up to 16 rows between workgroups
-    // costs more than the shorter slabs save (measured at every M from 5 to 16); low rank and Monarch keep the split
-    const bool no_split = bo == b && bo > 1 && a.perm_per == 0;
-    int ks = e_ks > 0 ? e_ks : (no_split ? 1 : resident / base);
+    int ks = e_ks > 0 ? e_ks : resident / base;
     if (ks > e_ksmax) ks = e_ksmax;
     if (ks > resident / base) ks = resident / base;
     if (ks < 1) ks = 1;
