@@ -1098,7 +1098,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
   static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
-  if (M >= mfma_min_m) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
+  if (M >= mfma_min_m && a.wbits == 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);   // codes stay with the vector variant
   if (M > 4) return d2_bail(__LINE__);
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int WBITS = a.wbits, EPL = 128 / WBITS;  // weights per 16-byte load
@@ -1261,6 +1261,7 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
   const int cus = device_cus() > 0 ? device_cus() : 256;
   const int resident = (occ < 2 ? occ : 2) * cus;
   if (R % 4) return d2_bail(__LINE__);
+  if (a.wbits != 16) return d2_bail(__LINE__);       // this kernel reads two-byte weights; its buffer bounds assume them
 
   Decode2Params p = {};
   p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
