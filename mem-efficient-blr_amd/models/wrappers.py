@@ -92,15 +92,66 @@ class BlastLinear(_StructuredLinear):
 
 
 class QuantBlastLinear(BlastLinear):
-    """BLAST with int8 / packed-int4 factors (method "blast_sym_quant"): quantized once at construction."""
+    """BLAST with int8 / packed-int4 factors (method "blast_sym_quant").
+
+    The factors are quantized once and kept in the order the kernels stream them: buffers ``u_codes`` (b, r, q[/2]),
+    ``u_scales`` (b, q), ``v_codes`` (b, p, r[/2]), ``v_scales`` (b, r); int4 packs two codes per byte along the last
+    axis, even index in the low nibble.  These buffers are what ``state_dict()`` holds (plus S, the bias and an extra
+    state naming bits and layout), so a packed checkpoint loads without touching the floating factors again.
+    ``load_state_dict`` also takes a checkpoint of the floating module (keys ``U`` (b, q, r) and ``V`` (b, p, r), the
+    bmm layouts) and repacks it on the way in."""
+    PACK_FORMAT = "blr-packed-blast/1: U codes (b,r,q[/2]) + scales (b,q); V codes (b,p,r[/2]) + scales (b,r); int4 low nibble = even index"
 
     def __init__(self, in_features, out_features, b, rank, func_path, device, dtype, bias=True, is_compiled=False, bits=8):
         super().__init__(in_features, out_features, b, rank, func_path, device, dtype, bias, is_compiled)
-        from triton_funcs.blast_sym_quant_kernels import quantize_blast_factors
         assert "bmm" in self.func_name, "the quantized kernel takes the bmm layouts"
+        assert bits in (8, 4)
         self.bits = bits
-        self.Uq, self.Vq = quantize_blast_factors(self.U.detach().float(), self.V.detach().float(), bits)
+        U, V = self.U.detach().float(), self.V.detach().float()
         del self.U, self.V
+        self._pack(U, V)
+
+    def _pack(self, U, V):
+        from triton_funcs.blast_sym_quant_kernels import quantize_blast_factors
+        Uq, Vq = quantize_blast_factors(U, V, self.bits)
+        for name, t in (("u_codes", Uq.codes), ("u_scales", Uq.scales), ("v_codes", Vq.codes), ("v_scales", Vq.scales)):
+            if name in self._buffers:
+                self._buffers[name] = t
+            else:
+                self.register_buffer(name, t)
+        self._u_shape, self._v_shape = tuple(Uq.shape), tuple(Vq.shape)
+
+    @property
+    def Uq(self):
+        from triton_funcs.blast_sym_quant_kernels import QuantFactor
+        return QuantFactor(self.u_codes, self.u_scales, self.bits, self._u_shape)
+
+    @property
+    def Vq(self):
+        from triton_funcs.blast_sym_quant_kernels import QuantFactor
+        return QuantFactor(self.v_codes, self.v_scales, self.bits, self._v_shape)
+
+    def get_extra_state(self):
+        return {"format": self.PACK_FORMAT, "bits": self.bits, "u_shape": list(self._u_shape), "v_shape": list(self._v_shape)}
+
+    def set_extra_state(self, state):
+        if state.get("format") != self.PACK_FORMAT:
+            raise RuntimeError(f"unknown packed format {state.get('format')!r}")
+        if int(state["bits"]) != self.bits:
+            raise RuntimeError(f"checkpoint holds {state['bits']}-bit factors, the module {self.bits}-bit")
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+        ku, kv = prefix + "U", prefix + "V"
+        if ku in state_dict and kv in state_dict:                  # floating checkpoint: repack
+            U, V = state_dict.pop(ku), state_dict.pop(kv)
+            if tuple(U.shape) != self._u_shape or tuple(V.shape) != self._v_shape:
+                error_msgs.append(f"{prefix}: floating factors {tuple(U.shape)}, {tuple(V.shape)} do not fit {self._u_shape}, {self._v_shape}")
+            else:
+                self._pack(U.to(self.u_codes.device).float(), V.to(self.u_codes.device).float())
+                for name in ("u_codes", "u_scales", "v_codes", "v_scales"):
+                    state_dict[prefix + name] = self._buffers[name]
+                state_dict.setdefault(prefix + "_extra_state", self.get_extra_state())
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
 
     def forward(self, x):
         return self._finish(self.func(x, self.Uq, self.Vq, self.S))

@@ -108,3 +108,39 @@ def test_blast_q_rejects_bad_input():
         Q.triton_blast_bmm_int8_fp16(x, U.half(), Vq, torch.zeros(24, 2, 2, device="cuda", dtype=torch.float16))
     with pytest.raises(L.BlrError):      # r = 24 is not a multiple of 32
         Q.triton_blast_bmm_int8_fp16(x, Uq, Vq, torch.zeros(24, 2, 2, device="cuda", dtype=torch.float16))
+
+
+def test_packed_factors_round_trip_through_a_checkpoint(tmp_path):
+    """state_dict of the quantized module = the packed buffers; saved with safetensors and loaded into a fresh module
+    they give bit-identical outputs; a checkpoint of the floating module is repacked on load."""
+    import safetensors.torch as st
+    from models import wrappers as W
+    dev_, dt = torch.device("cuda"), torch.float16
+    path = "triton_funcs.blast_sym_quant_kernels.triton_blast_bmm_int8_fp16"
+    for bits in (8, 4):
+        torch.manual_seed(bits)
+        a = W.QuantBlastLinear(256, 512, 4, 64, path, dev_, dt, bias=True, bits=bits)
+        x = torch.randn(3, 256, device="cuda", dtype=dt)
+        with torch.no_grad():
+            ya = a(x)
+        sd = a.state_dict()
+        assert {"u_codes", "u_scales", "v_codes", "v_scales", "S", "bias", "_extra_state"} <= set(sd)
+        assert sd["u_codes"].shape == (4, 64, 128 * bits // 8) and sd["v_codes"].shape == (4, 64, 64 * bits // 8)
+        tensors = {k: v.contiguous() for k, v in sd.items() if isinstance(v, torch.Tensor)}
+        st.save_file(tensors, str(tmp_path / f"q{bits}.safetensors"), metadata={"format": sd["_extra_state"]["format"], "bits": str(bits)})
+        loaded = st.load_file(str(tmp_path / f"q{bits}.safetensors"), device="cuda")
+        loaded["_extra_state"] = sd["_extra_state"]
+        b = W.QuantBlastLinear(256, 512, 4, 64, path, dev_, dt, bias=True, bits=bits)
+        b.load_state_dict(loaded)
+        with torch.no_grad():
+            yb = b(x)
+        assert torch.equal(ya, yb)
+        # a floating checkpoint (bmm layouts) is repacked on load and matches quantizing the same factors directly
+        f = W.BlastLinear(256, 512, 4, 64, "triton_funcs.blast_kernels.triton_blast_bmm_fp16", dev_, dt, bias=True)
+        c = W.QuantBlastLinear(256, 512, 4, 64, path, dev_, dt, bias=True, bits=bits)
+        c.load_state_dict(f.state_dict())
+        Uq, Vq = __import__("triton_funcs.blast_sym_quant_kernels", fromlist=["x"]).quantize_blast_factors(f.U.detach().float(), f.V.detach().float(), bits)
+        assert torch.equal(c.u_codes, Uq.codes) and torch.equal(c.v_scales, Vq.scales) and torch.equal(c.S, f.S)
+        wrong = W.QuantBlastLinear(256, 512, 4, 64, path, dev_, dt, bias=True, bits=12 - bits)
+        with pytest.raises(RuntimeError):
+            wrong.load_state_dict(loaded)
