@@ -369,10 +369,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
 //     the j-th 16-bit column of the 4 rows whose addresses lanes 4e + j/4 supply.
 // The loads are written as assembly so that the compiler does not count them: it would otherwise wait for all of them
 // before every LDS read that follows.  The kernel waits itself (s_waitcnt vmcnt) before a stage is read.
-constexpr int RING_NA = 4, RING_NB = 5;
-template <int BM, int BN>
+// Ring depths.  SHALLOW (256x128 only) keeps three stages of each operand instead of four and five, so that two
+// workgroups share a compute unit (72 KB each) and one's tile start-up and write-out run under the other's main loop:
+// better when a compute unit gets several tiles with short reductions, worse when it gets one long one.
+template <bool SHALLOW> constexpr int ring_na() { return SHALLOW ? 3 : 4; }
+template <bool SHALLOW> constexpr int ring_nb() { return SHALLOW ? 3 : 5; }
+template <int BM, int BN, bool SHALLOW>
 constexpr size_t ring_lds_bytes() {
-  size_t st = (size_t)(RING_NA * BM + RING_NB * BN) * 64, ep = (size_t)BM * (BN + 8) * 2;
+  size_t st = (size_t)(ring_na<SHALLOW>() * BM + ring_nb<SHALLOW>() * BN) * 64, ep = (size_t)BM * (BN + 8) * 2;
   return st > ep ? st : ep;
 }
 constexpr int ring_vmcnt(int n) { return (n & 0xf) | ((n >> 4) << 14) | (7 << 4) | (0xf << 8); }   // s_waitcnt immediate: vmcnt = n only
@@ -385,9 +389,9 @@ __device__ __forceinline__ uint32_t ring_lds_addr(const void* p) {
   return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((void __attribute__((address_space(3)))*)(p)));
 }
 
-template <typename T, bool B_KN, int BM, int BN, bool EP = false>
-__global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
-  constexpr int NA = RING_NA, NB = RING_NB;
+template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false>
+__global__ __launch_bounds__(256, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
+  constexpr int NA = ring_na<SHALLOW>(), NB = ring_nb<SHALLOW>();
   constexpr int ASTG = BM * 64, BSTG = BN * 64, BRING = NA * ASTG;   // stage sizes, start of the B ring
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int LA = BM / 64, LB = BN / 64;          // 1 KiB direct loads per wave and k tile
@@ -516,7 +520,9 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
   // loop body is one straight block for every tile: the last step also waits for, and fetches fragments of, a tile that
   // does not exist (whatever the stage holds; never multiplied), and a partial last tile multiplies what it lacks with
   // zeros.
-  constexpr int INFLIGHT = LB + (NA - 2) * LT;
+  // With rings of equal depth B(t+1) goes out in the same step as A(t+1), after it: then only the loads of the NB - 2
+  // later steps may be in flight.
+  constexpr int INFLIGHT = NB > NA ? LB + (NA - 2) * LT : (NB - 2) * LT;
   static_assert(NB >= NA, "B must not be needed before A under the in-order bound");
 #pragma unroll
   for (int s = 0; s < NB - 1; ++s) {
@@ -538,7 +544,7 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
     const int ta = min(t + NA - 1, KT - 1), tb = min(t + NB - 1, KT - 1);
     const bool pa = ktail && ta == KT - 1, pb = ktail && tb == KT - 1;
     const bool last_partial = ktail && t == KT - 1;
-    const int sla = (ca + NA - 1) & (NA - 1);        // NA is a power of two
+    const int sla = ca == 0 ? NA - 1 : ca - 1;
     const int slb = cb == 0 ? NB - 1 : cb - 1;
     frags(ca, cb, 1, 1);
     __builtin_amdgcn_sched_barrier(0);
@@ -573,7 +579,7 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmArgs g, int tiles_m,
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(ring_vmcnt(INFLIGHT));  // tile t + 1 has landed (this wave's part)
     __builtin_amdgcn_s_barrier();                    // everybody's part has, and nobody reads the stages of tile t any more
-    ca = (ca + 1) & (NA - 1);
+    ca = ca + 1 == NA ? 0 : ca + 1;
     cb = cb + 1 == NB ? 0 : cb + 1;
     frags(ca, cb, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
@@ -728,13 +734,13 @@ static bool ring_ok(const GemmArgs& g) {
   return true;
 }
 
-template <typename T, int BM, int BN>
+template <typename T, int BM, int BN, bool SHALLOW = false>
 static int launch_ring(const GemmArgs& g, hipStream_t st) {
   int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
-  const size_t lds = ring_lds_bytes<BM, BN>();
+  const size_t lds = ring_lds_bytes<BM, BN, SHALLOW>();
   const bool ep = g.bias != nullptr || g.act != 0;
-  void* fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true> : (void*)gemm_ring_kernel<T, false, BM, BN, true>)
-                : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN> : (void*)gemm_ring_kernel<T, false, BM, BN>);
+  void* fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true, SHALLOW> : (void*)gemm_ring_kernel<T, false, BM, BN, true, SHALLOW>)
+                : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW>);
   static std::mutex mu;
   static std::set<void*> raised;
   {
@@ -769,7 +775,8 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   int64_t t128 = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
   // Problems with enough work go to the ring kernels, with the largest of their tiles that still gives every compute unit
   // one (BLR_GEMM_RING: 0 never, 1 by this rule, 2 whenever the operands allow it; BLR_GEMM_RING_TILE = 256256, 256128
-  // or 128128 picks the tile - both read at every call so that tests can switch them).
+  // or 128128 picks the tile, BLR_GEMM_RING_PER_CU = 1 or 2 the deep or the shallow 256x128 variant - all read at every
+  // call so that tests can switch them).
   const char* ring_e = getenv("BLR_GEMM_RING");
   const int ring = ring_e ? atoi(ring_e) : 1;
   if (ring > 0 && force == 0 && ring_ok(g)) {
@@ -777,17 +784,21 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     int rt = rt_e ? atoi(rt_e) : 0;
     const int64_t fill = ((int64_t)cus * 9 + 9) / 10;
     const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
+    const char* pc_e = getenv("BLR_GEMM_RING_PER_CU");
+    int per_cu = pc_e ? atoi(pc_e) : 0;
     if (rt == 0) {
-      // short reductions are mostly tile start-up and write-out: two small workgroups per compute unit overlap those
-      if (g.K <= 512 && r128 >= fill) rt = 128128;
+      // short reductions are mostly tile start-up and write-out: two workgroups per compute unit overlap those
+      if (g.K <= 2048 && t128 >= 2 * (int64_t)cus) { rt = 256128; if (!per_cu) per_cu = 2; }
+      else if (g.K <= 512 && r128 >= fill) rt = 128128;
       else if (t256 >= fill) rt = 256256;
       else if (t128 >= fill) rt = 256128;
       else if (r128 >= fill || ring > 1) rt = 128128;
     }
     if (rt && (ring > 1 || (g.M >= 96 && g.K >= 64))) {
       if (rt == 256256) return launch_ring<T, 256, 256>(g, st);
-      if (rt == 256128) return launch_ring<T, 256, 128>(g, st);
-      return launch_ring<T, 128, 128>(g, st);
+      if (rt == 256128) return per_cu == 2 ? launch_ring<T, 256, 128, true>(g, st) : launch_ring<T, 256, 128>(g, st);
+      if (!per_cu) per_cu = r128 >= 2 * (int64_t)cus ? 2 : 1;     // three shallow workgroups per compute unit, or two deep ones
+      return per_cu == 2 ? launch_ring<T, 128, 128, true>(g, st) : launch_ring<T, 128, 128>(g, st);
     }
   }
   // the register-staged kernel at 256x256 needs more registers than there are and spills: only on request (BLR_GEMM_TILE=256)
