@@ -358,7 +358,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
 }
 
 // ---- large problems: operand tiles copied global -> LDS without passing through registers --------------------------
-// One workgroup of 4 waves (2 x 2) per BM x BN tile (256 x 256: wave tile 128 x 128, 256 accumulator registers).  The k loop advances in
+// One workgroup per BM x BN tile: 4 waves as 2 x 2 (256 x 256: wave tile 128 x 128, 256 accumulator registers), or 8
+// waves, two per SIMD, as 2 x 4 (256 x 256: wave tile 128 x 64) - the pair on a SIMD fills each other's waits at the
+// barrier and for LDS, which is worth ~4 % on long reductions although a wave then reads 0.75 instead of 0.5 fragments
+// per matrix instruction.  The k loop advances in
 // stages of 32: a stage of A (BM rows x 64 bytes) and a stage of B live in two rings in LDS (4 and 5 stages), filled by
 // global_load_lds_dwordx4 - each wave instruction moves 1 KiB and lane l's 16 bytes land at the wave's LDS address
 // + 16 l, so the layout in LDS is chosen by which global address every lane fetches:
@@ -369,8 +372,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
 //     the j-th 16-bit column of the 4 rows whose addresses lanes 4e + j/4 supply.
 // The loads are written as assembly so that the compiler does not count them: it would otherwise wait for all of them
 // before every LDS read that follows.  The kernel waits itself (s_waitcnt vmcnt) before a stage is read.
-// Ring depths.  SHALLOW (256x128 only) keeps three stages of each operand instead of four and five, so that two
-// workgroups share a compute unit (72 KB each) and one's tile start-up and write-out run under the other's main loop:
+// Ring depths.  SHALLOW (256x128, 128x128) keeps three stages of each operand instead of four and five, so that two
+// (three) workgroups share a compute unit (72 KB / 48 KB each) and one's tile start-up and write-out run under the other's main loop:
 // better when a compute unit gets several tiles with short reductions, worse when it gets one long one.
 template <bool SHALLOW> constexpr int ring_na() { return SHALLOW ? 3 : 4; }
 template <bool SHALLOW> constexpr int ring_nb() { return SHALLOW ? 3 : 5; }
@@ -389,12 +392,13 @@ __device__ __forceinline__ uint32_t ring_lds_addr(const void* p) {
   return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((void __attribute__((address_space(3)))*)(p)));
 }
 
-template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false>
-__global__ __launch_bounds__(256, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
+template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false, int NWV = 4>
+__global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
   constexpr int NA = ring_na<SHALLOW>(), NB = ring_nb<SHALLOW>();
   constexpr int ASTG = BM * 64, BSTG = BN * 64, BRING = NA * ASTG;   // stage sizes, start of the B ring
-  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
-  constexpr int LA = BM / 64, LB = BN / 64;          // 1 KiB direct loads per wave and k tile
+  constexpr int WGN = (NWV == 8 && BN == 256) ? 4 : 2, WGM = NWV / WGN;   // waves: 2 x 2, or 2 x 4 / 4 x 2 (two per SIMD)
+  constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+  constexpr int LA = BM / (16 * NWV), LB = BN / (16 * NWV);   // 1 KiB direct loads per wave and k tile
   constexpr int LT = LA + LB;
   constexpr int RB = BN * 2, CPR = BN / 8, RPI = 1024 / RB;
   constexpr int NMF = TM * TN;
@@ -403,7 +407,7 @@ __global__ __launch_bounds__(256, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmA
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int tiles = tiles_m * tiles_n;
   int u = blockIdx.x;
   if (per_xcd > 0) u = (u & 7) * per_xcd + (u >> 3);
@@ -431,15 +435,15 @@ __global__ __launch_bounds__(256, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmA
   const int kc_chunk = (lane & 3) ^ ((row16 >> 1) & 3);
 #pragma unroll
   for (int i = 0; i < LA; ++i)
-    a_off[i] = (uint32_t)(min(m0 + (i * 4 + wave) * 16 + row16, g.M - 1) * g.lda * 2 + kc_chunk * 16);
+    a_off[i] = (uint32_t)(min(m0 + (i * NWV + wave) * 16 + row16, g.M - 1) * g.lda * 2 + kc_chunk * 16);
 #pragma unroll
   for (int i = 0; i < LB; ++i) {
     if (B_KN) {
-      const int krow = (i * 4 + wave) * RPI + lane / CPR;
+      const int krow = (i * NWV + wave) * RPI + lane / CPR;
       const int chunk = (lane % CPR) ^ ((krow & 3) << 1);
       b_off[i] = (uint32_t)(krow * g.ldb * 2 + min(n0 + chunk * 8, g.N - 8) * 2);
     } else {
-      b_off[i] = (uint32_t)(min(n0 + (i * 4 + wave) * 16 + row16, g.N - 1) * g.ldb * 2 + kc_chunk * 16);
+      b_off[i] = (uint32_t)(min(n0 + (i * NWV + wave) * 16 + row16, g.N - 1) * g.ldb * 2 + kc_chunk * 16);
     }
   }
   // what to subtract from those offsets in a partial last tile (ktail valid k): the chunks of a K-contiguous row and the
@@ -449,17 +453,17 @@ __global__ __launch_bounds__(256, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmA
   uint32_t tail_kn[LB];
 #pragma unroll
   for (int i = 0; i < LB; ++i) {
-    const int krow = (i * 4 + wave) * RPI + lane / CPR;
+    const int krow = (i * NWV + wave) * RPI + lane / CPR;
     tail_kn[i] = B_KN ? (uint32_t)((krow - min(krow, rmax)) * g.ldb * 2) : tail_kc;
   }
   const uint32_t lds0 = ring_lds_addr(smem + wave * 1024);
   // load number li of the A tile ta (into A stage sa) or of the B tile tb (into B stage sb)
   auto issue_a = [&](int li, int ta, int sa, bool partial) {
-    ring_load_lds(Ab + (int64_t)ta * 64, a_off[li] - (partial ? tail_kc : 0u), lds0 + sa * ASTG + li * 4096);
+    ring_load_lds(Ab + (int64_t)ta * 64, a_off[li] - (partial ? tail_kc : 0u), lds0 + sa * ASTG + li * (NWV * 1024));
   };
   auto issue_b = [&](int li, int tb, int sb, bool partial) {
     const char* Bp = B_KN ? Bb + (int64_t)tb * 32 * g.ldb * 2 : Bb + (int64_t)tb * 64;
-    ring_load_lds(Bp, b_off[li] - (partial ? tail_kn[li] : 0u), lds0 + BRING + sb * BSTG + li * 4096);
+    ring_load_lds(Bp, b_off[li] - (partial ? tail_kn[li] : 0u), lds0 + BRING + sb * BSTG + li * (NWV * 1024));
   };
 
   // fragment addresses
@@ -605,7 +609,7 @@ __global__ __launch_bounds__(256, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmA
     }
   __syncthreads();
   constexpr int VPR = BN / 8;
-  for (int v = tid; v < BM * VPR; v += 256) {
+  for (int v = tid; v < BM * VPR; v += NWV * 64) {
     const int row = v / VPR, cvec = (v - row * VPR) * 8;
     const int gr = m0 + row, gc = n0 + cvec;
     if (gr < g.M && gc < g.N) {
@@ -734,13 +738,13 @@ static bool ring_ok(const GemmArgs& g) {
   return true;
 }
 
-template <typename T, int BM, int BN, bool SHALLOW = false>
+template <typename T, int BM, int BN, bool SHALLOW = false, int NWV = 4>
 static int launch_ring(const GemmArgs& g, hipStream_t st) {
   int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
   const size_t lds = ring_lds_bytes<BM, BN, SHALLOW>();
   const bool ep = g.bias != nullptr || g.act != 0;
-  void* fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true, SHALLOW> : (void*)gemm_ring_kernel<T, false, BM, BN, true, SHALLOW>)
-                : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW>);
+  void* fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true, SHALLOW, NWV> : (void*)gemm_ring_kernel<T, false, BM, BN, true, SHALLOW, NWV>)
+                : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW, NWV> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW, NWV>);
   static std::mutex mu;
   static std::set<void*> raised;
   {
@@ -760,7 +764,7 @@ static int launch_ring(const GemmArgs& g, hipStream_t st) {
   dim3 grid((unsigned)(per_xcd > 0 ? per_xcd * 8 : total));
   GemmArgs ga = g;
   void* args[] = {&ga, &tiles_m, &tiles_n, &per_xcd, &group_m};
-  hipError_t e = hipLaunchKernel(fn, grid, dim3(256), args, lds, st);
+  hipError_t e = hipLaunchKernel(fn, grid, dim3(NWV * 64), args, lds, st);
   if (e != hipSuccess) { set_error("gemm_ring: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
 }
@@ -775,8 +779,9 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   int64_t t128 = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
   // Problems with enough work go to the ring kernels, with the largest of their tiles that still gives every compute unit
   // one (BLR_GEMM_RING: 0 never, 1 by this rule, 2 whenever the operands allow it; BLR_GEMM_RING_TILE = 256256, 256128
-  // or 128128 picks the tile, BLR_GEMM_RING_PER_CU = 1 or 2 the deep or the shallow 256x128 variant - all read at every
-  // call so that tests can switch them).
+  // or 128128 picks the tile, BLR_GEMM_RING_PER_CU = 1 or 2 the deep or the shallow variant of the two smaller tiles,
+  // BLR_GEMM_RING_WAVES = 4 or 8 the workgroup size of the two larger ones - all read at every call so that tests can
+  // switch them).
   const char* ring_e = getenv("BLR_GEMM_RING");
   const int ring = ring_e ? atoi(ring_e) : 1;
   if (ring > 0 && force == 0 && ring_ok(g)) {
@@ -795,8 +800,16 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       else if (r128 >= fill || ring > 1) rt = 128128;
     }
     if (rt && (ring > 1 || (g.M >= 96 && g.K >= 64))) {
-      if (rt == 256256) return launch_ring<T, 256, 256>(g, st);
-      if (rt == 256128) return per_cu == 2 ? launch_ring<T, 256, 128, true>(g, st) : launch_ring<T, 256, 128>(g, st);
+      if (rt == 256256) {
+        const char* w_e = getenv("BLR_GEMM_RING_WAVES");
+        // eight waves (2 x 4, wave tile 128 x 64, two per SIMD) hide each other's barrier and LDS waits: the default
+        return (w_e && atoi(w_e) == 4) ? launch_ring<T, 256, 256>(g, st) : launch_ring<T, 256, 256, false, 8>(g, st);
+      }
+      if (rt == 256128) {
+        const char* w_e = getenv("BLR_GEMM_RING_WAVES");
+        if (per_cu != 2 && w_e && atoi(w_e) == 8) return launch_ring<T, 256, 128, false, 8>(g, st);
+        return per_cu == 2 ? launch_ring<T, 256, 128, true>(g, st) : launch_ring<T, 256, 128>(g, st);
+      }
       if (!per_cu) per_cu = r128 >= 2 * (int64_t)cus ? 2 : 1;     // three shallow workgroups per compute unit, or two deep ones
       return per_cu == 2 ? launch_ring<T, 128, 128, true>(g, st) : launch_ring<T, 128, 128>(g, st);
     }

@@ -1,7 +1,7 @@
 """GPU parity of the GEMM kernels whose operand tiles are copied global -> LDS directly, against the oracle.
 
 They are normally chosen only for problems that fill the chip; BLR_GEMM_RING=2 selects them whenever the operands
-allow it and BLR_GEMM_RING_TILE / BLR_GEMM_RING_PER_CU pick the tile shape (256x256, 256x128 deep or shallow, 128x128), so small, ragged and tail shapes (M, N not multiples of 256; K with a 16-wide last slice; K shorter than
+allow it and BLR_GEMM_RING_TILE / BLR_GEMM_RING_PER_CU / BLR_GEMM_RING_WAVES pick the variant (256x256 with four or eight waves, 256x128 and 128x128 with deep or shallow rings), so small, ragged and tail shapes (M, N not multiples of 256; K with a 16-wide last slice; K shorter than
 the prefetch depth) run through it here.  Every case is also run with the kernel switched off and the two results
 must agree to rounding.
 """
@@ -17,14 +17,15 @@ from gpu_util import assert_close, back, blast_inputs, dev, rounded, say
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["256256", "256128", "256128/2", "128128"])
+@pytest.fixture(params=["256256", "256256/1/8", "256128", "256128/1/8", "256128/2", "128128", "128128/2"])
 def ring_forced(request):
-    """Selects the kernel for every legal problem, with one of its tile shapes (256x128 with deep rings, one workgroup
-    per compute unit, or shallow rings, two)."""
-    old = {k: os.environ.get(k) for k in ("BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU")}
+    """Selects the kernel for every legal problem, with one of its variants: tile shape / ring depth (1 deep rings, 2
+    shallow ones and more workgroups per compute unit) / waves per workgroup (256x256 only)."""
+    env = ("BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU", "BLR_GEMM_RING_WAVES")
+    old = {k: os.environ.get(k) for k in env}
+    parts = (request.param.split("/") + ["1", "4"])[:3]
     os.environ["BLR_GEMM_RING"] = "2"
-    os.environ["BLR_GEMM_RING_TILE"] = request.param.split("/")[0]
-    os.environ["BLR_GEMM_RING_PER_CU"] = "2" if request.param.endswith("/2") else "1"
+    os.environ["BLR_GEMM_RING_TILE"], os.environ["BLR_GEMM_RING_PER_CU"], os.environ["BLR_GEMM_RING_WAVES"] = parts
     yield request.param
     for k, v in old.items():
         if v is None:
