@@ -467,7 +467,7 @@ size_t blr_low_rank_workspace_bytes(int M, int in_f, int out_f, int r, int dtype
     size_t s = stream_generic_workspace(1, M, in_f, out_f, 1, r);
     return s > tiled ? s : tiled;
   }
-  return tiled;
+  return tiled + gemm_splitk_bytes(M, r, in_f, dtype);       // x.A has few output tiles and a long reduction: room to cut it along K
 }
 
 int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
@@ -495,6 +495,8 @@ int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
   GemmArgs g1 = {};
   g1.A = x; g1.lda = ldx; g1.B = A; g1.ldb = r; g1.b_kn = 1;
   g1.C = Z; g1.ldc = r; g1.cn = 1; g1.M = M; g1.N = r; g1.K = in_f; g1.batch = 1;
+  const size_t tiled = align_up((size_t)M * r * elt_size(dtype), 256);
+  if (ws && ws_bytes > tiled) { g1.splitk_ws = static_cast<char*>(ws) + tiled; g1.splitk_bytes = ws_bytes - tiled; }
   int rc = gemm_launch(g1, dtype, st);
   if (rc) return rc;
   GemmArgs g2 = {};

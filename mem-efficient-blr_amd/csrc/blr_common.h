@@ -106,9 +106,15 @@ struct GemmArgs {
   int sat8;         // 1: the fp32 result is rounded to nearest even and clamped to [-128, 127] before it is stored
   const void* bias; // optional: values of dtype added to the rounded result, indexed by the element's offset inside its row of C
   int act;          // blr_act applied after the bias
+  void* splitk_ws;  // optional scratch for splitting the reduction (gemm_splitk_bytes says how much); null: never split
+  size_t splitk_bytes;
+  int kc;           // set by gemm_launch for the split kernels: k values per slice
 };
 // dtype: blr_dtype.  Returns blr_status.
 int gemm_launch(const GemmArgs& a, int dtype, hipStream_t st);
+// Scratch a plain single GEMM M x N x K of dtype wants in GemmArgs::splitk_ws so that a problem with few output tiles and
+// a long reduction can be cut along K to fill the chip (fp32 partial results, summed in a fixed order).  0: no split.
+size_t gemm_splitk_bytes(int M, int N, int K, int dtype);
 
 // ---- BLAST rank-space mix, tiled path (blr_gemm.hip) ------------------------------------
 // Z[i, m, r] = sum_j S(i, j, r) * Y[j, m, r];  Y, Z (b, M, R) contiguous of dtype.

@@ -207,8 +207,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
   int u = blockIdx.x;
   if (per_xcd > 0) u = (u & 7) * per_xcd + (u >> 3);
   if (u >= tiles * g.batch) return;
-  const int bt = u / tiles;
-  const int ut = u - bt * tiles;
+  // interleaved columns: the batches of one tile write into the same cache lines, so they run next to each other
+  const int bt = g.cn != 1 ? u % g.batch : u / tiles;
+  const int ut = g.cn != 1 ? u / g.batch : u - bt * tiles;
   const int strip = ut / (group_m * tiles_n);
   const int rem = ut - strip * group_m * tiles_n;
   const int gm_here = min(group_m, tiles_m - strip * group_m);
@@ -392,7 +393,7 @@ __device__ __forceinline__ uint32_t ring_lds_addr(const void* p) {
   return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((void __attribute__((address_space(3)))*)(p)));
 }
 
-template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false, int NWV = 4>
+template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false, int NWV = 4, bool PARTIAL = false>
 __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
   constexpr int NA = ring_na<SHALLOW>(), NB = ring_nb<SHALLOW>();
   constexpr int ASTG = BM * 64, BSTG = BN * 64, BRING = NA * ASTG;   // stage sizes, start of the B ring
@@ -412,8 +413,10 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   int u = blockIdx.x;
   if (per_xcd > 0) u = (u & 7) * per_xcd + (u >> 3);
   if (u >= tiles * g.batch) return;
-  const int bt = u / tiles;
-  const int ut = u - bt * tiles;
+  // interleaved columns: the batches of one tile write into the same cache lines, so they run next to each other (same
+  // XCD, same time) and the lines are complete before they leave the L2
+  const int bt = g.cn != 1 ? u % g.batch : u / tiles;
+  const int ut = g.cn != 1 ? u / g.batch : u - bt * tiles;
   const int strip = ut / (group_m * tiles_n);
   const int rem = ut - strip * group_m * tiles_n;
   const int gm_here = min(group_m, tiles_m - strip * group_m);
@@ -424,8 +427,10 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   const char* Bb = reinterpret_cast<const char*>(g.B) + (int64_t)bt * g.sB * 2;
   T* C = reinterpret_cast<T*>(g.C);
 
-  const int KT = (g.K + 31) >> 5;
-  const int ktail = g.K & 31;                         // valid k of the last tile when it is partial: 8, 16 or 24
+  // PARTIAL: the batch index counts slices of the reduction (g.kc values of k each, the last one what is left of g.K)
+  const int Kloc = PARTIAL ? min(g.kc, g.K - bt * g.kc) : g.K;
+  const int KT = (Kloc + 31) >> 5;
+  const int ktail = Kloc & 31;                        // valid k of the last tile when it is partial: 8, 16 or 24
 
   // K-contiguous operand tile: rows of 32 k (64 bytes); chunk c of row r is stored at chunk c ^ ((r >> 1) & 3).
   // (k, n) operand tile: 32 rows of BN n; chunk c of row k is stored at chunk c ^ ((k & 3) << 1): the four rows a
@@ -592,6 +597,22 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
     __builtin_amdgcn_sched_barrier(0);
   }
   __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
+  if (PARTIAL) {
+    // fp32 partial sums of this slice, straight from the accumulators: an instruction stores two rows of 32 floats
+    float* P = reinterpret_cast<float*>(g.C) + (int64_t)bt * g.sC;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int gc = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int gr = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          if (gr < g.M && gc < g.N) P[(int64_t)gr * g.ldc + gc] = acc[i][j][e];
+        }
+      }
+    return;
+  }
   __syncthreads();                                                   // the epilogue reuses the tile memory
 
   constexpr int CLD = BN + 8;
@@ -608,6 +629,16 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
       }
     }
   __syncthreads();
+  if (g.cn != 1) {
+    // interleaved columns (column n of batch bt is element n * cn + bt of the row): two-byte stores, lanes along n, so
+    // that an instruction touches cn * 128 contiguous bytes; the other batches fill the gaps
+    for (int v = tid; v < BM * BN; v += NWV * 64) {
+      const int row = v / BN, col = v - row * BN;
+      const int gr = m0 + row, gc = n0 + col;
+      if (gr < g.M && gc < g.N) C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + (int64_t)gc * g.cn] = cs[row * CLD + col];
+    }
+    return;
+  }
   constexpr int VPR = BN / 8;
   for (int v = tid; v < BM * VPR; v += NWV * 64) {
     const int row = v / VPR, cvec = (v - row * VPR) * 8;
@@ -728,23 +759,75 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
 }
 
 // The ring kernels take plain row-major output and 16-byte friendly operands whose per-lane byte offsets fit 32 bits.
+// out[m, n] = sum over slices s of P[s][m][n] (fp32, fixed order), rounded once to T; 8 columns per thread
+template <typename T>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ P, T* __restrict__ C, int M, int N, int64_t ldc, int splits) {
+  using V8 = typename TypeTraits<T>::vec8;
+  const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int vpr = N >> 3;
+  if (v >= (int64_t)M * vpr) return;
+  const int m = (int)(v / vpr), n = (int)(v - (int64_t)m * vpr) * 8;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+  for (int s = 0; s < splits; ++s) {
+    const float4* p = reinterpret_cast<const float4*>(P + ((int64_t)s * M + m) * N + n);
+    const float4 a = p[0], b = p[1];
+    acc[0] += a.x; acc[1] += a.y; acc[2] += a.z; acc[3] += a.w;
+    acc[4] += b.x; acc[5] += b.y; acc[6] += b.z; acc[7] += b.w;
+  }
+  V8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = TypeTraits<T>::from_f32(acc[e]);
+  *reinterpret_cast<V8*>(&C[(int64_t)m * ldc + n]) = o;
+}
+
+// How many slices a plain single GEMM is cut into along K: only when 256 x 128 tiles leave at least half of the compute
+// units idle and every slice keeps at least 512 values of k (slices are multiples of 32).
+static int splitk_plan(int M, int N, int K, int* kc_out) {
+  const int cus = device_cus() > 0 ? device_cus() : 256;
+  const int64_t tiles = cdiv(M, 256) * cdiv(N, 128);
+  if (M < 96 || N % 8 || K % 8 || tiles * 2 > cus) return 1;
+  int splits = (int)std::min<int64_t>(8, cus / tiles);
+  while (splits > 1 && K / splits < 512) --splits;
+  if (splits <= 1) return 1;
+  const int kc = (int)cdiv(cdiv(K, splits), 32) * 32;
+  splits = (int)cdiv(K, kc);
+  if (kc_out) *kc_out = kc;
+  return splits;
+}
+
+size_t gemm_splitk_bytes(int M, int N, int K, int dtype) {
+  if (dtype != BLR_F16 && dtype != BLR_BF16) return 0;
+  const int splits = splitk_plan(M, N, K, nullptr);
+  return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
 static bool ring_ok(const GemmArgs& g) {
-  if (g.epi != EPI_PLAIN || g.cn != 1 || g.N < 8 || g.N % 8 || g.K % 8) return false;
-  if (!aligned(g.A, 16) || !aligned(g.B, 16) || !aligned(g.C, 16) || (g.bias && !aligned(g.bias, 16))) return false;
-  if (g.lda % 8 || g.sA % 8 || g.ldb % 8 || g.sB % 8 || g.ldc % 8 || g.sC % 8) return false;
+  if (g.epi != EPI_PLAIN || g.cn < 1 || g.N < 8 || g.N % 8 || g.K % 8) return false;
+  if (!aligned(g.A, 16) || !aligned(g.B, 16) || g.lda % 8 || g.sA % 8 || g.ldb % 8 || g.sB % 8) return false;
+  if (g.cn == 1) {                                   // 16-byte stores, the fused output stage reads its vector the same way
+    if (!aligned(g.C, 16) || (g.bias && !aligned(g.bias, 16)) || g.ldc % 8 || g.sC % 8) return false;
+  } else if (g.bias || g.act) {
+    return false;                                    // interleaved columns are stored one by one, without an output stage
+  }
   const int64_t lim = (int64_t)1 << 32;
   if ((int64_t)(g.M - 1) * g.lda * 2 + 64 >= lim) return false;
   if (g.b_kn ? 31 * g.ldb * 2 + (int64_t)g.N * 2 >= lim : (int64_t)(g.N - 1) * g.ldb * 2 + 64 >= lim) return false;
   return true;
 }
 
-template <typename T, int BM, int BN, bool SHALLOW = false, int NWV = 4>
+template <typename T, int BM, int BN, bool SHALLOW = false, int NWV = 4, bool PARTIAL = false>
 static int launch_ring(const GemmArgs& g, hipStream_t st) {
   int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
   const size_t lds = ring_lds_bytes<BM, BN, SHALLOW>();
   const bool ep = g.bias != nullptr || g.act != 0;
-  void* fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true, SHALLOW, NWV> : (void*)gemm_ring_kernel<T, false, BM, BN, true, SHALLOW, NWV>)
-                : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW, NWV> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW, NWV>);
+  void* fn;
+  if constexpr (PARTIAL)
+    fn = g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW, NWV, true> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW, NWV, true>;
+  else
+    fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true, SHALLOW, NWV> : (void*)gemm_ring_kernel<T, false, BM, BN, true, SHALLOW, NWV>)
+            : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW, NWV> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW, NWV>);
   static std::mutex mu;
   static std::set<void*> raised;
   {
@@ -784,6 +867,25 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   // switch them).
   const char* ring_e = getenv("BLR_GEMM_RING");
   const int ring = ring_e ? atoi(ring_e) : 1;
+  if (ring > 0 && force == 0 && ring_ok(g) && g.splitk_ws && g.batch == 1 && g.cn == 1 && !g.sat8 && !g.bias && !g.act) {
+    // few tiles, long reduction: slices of K as the batch of the partial-sum kernel, then one pass that adds them up
+    const char* sk_e = getenv("BLR_GEMM_SPLITK");
+    int kc = 0;
+    const int splits = (sk_e && atoi(sk_e) == 0) ? 1 : splitk_plan(g.M, g.N, g.K, &kc);
+    if (splits > 1 && g.splitk_bytes >= (size_t)splits * g.M * g.N * sizeof(float) && aligned(g.splitk_ws, 16)) {
+      GemmArgs p = g;
+      p.batch = splits; p.kc = kc;
+      p.sA = kc; p.sB = g.b_kn ? (int64_t)kc * g.ldb : kc;
+      p.C = g.splitk_ws; p.ldc = g.N; p.sC = (int64_t)g.M * g.N;
+      int rc = launch_ring<T, 256, 128, false, 4, true>(p, st);
+      if (rc) return rc;
+      const int64_t vecs = (int64_t)g.M * (g.N / 8);
+      hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3((unsigned)cdiv(vecs, 256)), dim3(256), 0, st,
+                         reinterpret_cast<const float*>(g.splitk_ws), reinterpret_cast<T*>(g.C), g.M, g.N, g.ldc, splits);
+      BLR_CHECK_LAUNCH("splitk_reduce");
+      return BLR_OK;
+    }
+  }
   if (ring > 0 && force == 0 && ring_ok(g)) {
     const char* rt_e = getenv("BLR_GEMM_RING_TILE");
     int rt = rt_e ? atoi(rt_e) : 0;
@@ -791,6 +893,8 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
     const char* pc_e = getenv("BLR_GEMM_RING_PER_CU");
     int per_cu = pc_e ? atoi(pc_e) : 0;
+    // interleaved columns are bound by their two-byte stores: only worth it with several tiles per compute unit
+    if (rt == 0 && g.cn != 1 && ring < 2 && t128 < 2 * (int64_t)cus) rt = -1;
     if (rt == 0) {
       // short reductions are mostly tile start-up and write-out: two workgroups per compute unit overlap those
       if (g.K <= 2048 && t128 >= 2 * (int64_t)cus) { rt = 256128; if (!per_cu) per_cu = 2; }
@@ -799,7 +903,7 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       else if (t128 >= fill) rt = 256128;
       else if (r128 >= fill || ring > 1) rt = 128128;
     }
-    if (rt && (ring > 1 || (g.M >= 96 && g.K >= 64))) {
+    if (rt > 0 && (ring > 1 || (g.M >= 96 && g.K >= 64))) {
       if (rt == 256256) {
         const char* w_e = getenv("BLR_GEMM_RING_WAVES");
         // eight waves (2 x 4, wave tile 128 x 64, two per SIMD) hide each other's barrier and LDS waits: the default

@@ -114,3 +114,30 @@ def test_low_rank_and_monarch_through_ring_kernel(dtype, ring_forced):
     ref = _ref_monarch(xm, w1_t, w2_t, dtype)
     ref = ref[0] if isinstance(ref, tuple) else ref
     assert_close(out, ref, dtype, "monarch", scale=2.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,in_f,r,out_f", [(300, 2056, 136, 264), (2048, 4096, 1024, 512), (130, 1024, 64, 128), (97, 6000, 8, 72)])
+def test_low_rank_with_the_reduction_cut_into_slices(M, in_f, r, out_f, dtype):
+    """x.A of low rank has few output tiles and a long reduction: the library cuts it along K (slices of whole 32-k
+    steps, the last one ragged), keeps fp32 partial sums and adds them in a fixed order.  Checked against the oracle and
+    against the same call with the split switched off."""
+    from triton_funcs import low_rank_kernels as LR
+    rng = np.random.default_rng(M + in_f)
+    x = rng.standard_normal((M, in_f)); a = rng.standard_normal((in_f, r)) / np.sqrt(in_f); bm = rng.standard_normal((r, out_f)) / np.sqrt(r)
+    say(f"[case] split-k low rank M={M} in={in_f} r={r} out={out_f} {dtype}")
+    xd, ad, bd = dev(x, dtype), dev(a, dtype), dev(bm, dtype)
+    out = LR.triton_low_rank_fp16(xd, ad, bd, TILED)
+    assert_close(out, (rounded(x, dtype) @ rounded(a, dtype)) @ rounded(bm, dtype), dtype, "low rank", scale=2.0)
+    again = LR.triton_low_rank_fp16(xd, ad, bd, TILED)
+    assert torch.equal(out, again), "the sum over slices must not depend on timing"
+    old = os.environ.get("BLR_GEMM_SPLITK")
+    os.environ["BLR_GEMM_SPLITK"] = "0"
+    try:
+        ref = LR.triton_low_rank_fp16(xd, ad, bd, TILED)
+    finally:
+        if old is None:
+            os.environ.pop("BLR_GEMM_SPLITK", None)
+        else:
+            os.environ["BLR_GEMM_SPLITK"] = old
+    assert_close(out, back(ref), dtype, "split vs unsplit", scale=0.5)
