@@ -794,17 +794,32 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
       dm_batch<T>(cur, a_s, ald, cv, rs, bi * DM_ROWS, acc);
     }
     TR2(1);
+    // y crosses workgroups as {two T values (ranks 2c, 2c + 1), epoch} pairs.  The totals go through LDS once more so
+    // that a wave stores 64 consecutive pairs of one token row (512 contiguous bytes) instead of 8-byte pieces 64 bytes apart.
+    constexpr int YLD = 130;
     reduce_emit(acc, [&](int col, int m0, const f32x4 (&vh)[2]) {
+      __syncthreads();                                            // every thread has read its sums out of red
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int gn = n0 + col + 4 * h;
-        if (gn < p.R) {
+      for (int h = 0; h < 2; ++h)
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (m0 + i < M) st_tag(&p.ypart[(((int64_t)ks * p.b + j) * M + m0 + i) * p.R + gn], vh[h][i], epoch);
+        for (int i = 0; i < 4; ++i) red[(m0 + i) * YLD + col + 4 * h] = vh[h][i];
+    });
+    __syncthreads();
+    {
+      const int cp = tid & 63, mq = (tid >> 6) * 4;
+      const int gn = n0 + 2 * cp;
+      if (gn < p.R) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int m = mq + i;
+          if (m < M) {
+            const unsigned long long v = ((unsigned long long)epoch << 32) |
+                                         pack2<T>(red[m * YLD + 2 * cp], (gn + 1 < p.R) ? red[m * YLD + 2 * cp + 1] : 0.0f);
+            __hip_atomic_store(&p.ypart[(((int64_t)ks * p.b + j) * M + m) * (p.R >> 1) + (gn >> 1)], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
         }
       }
-    });
+    }
     TR2(2);
   } else {
     check_in();
@@ -838,7 +853,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
           for (int m = 0; m < DM_MC; ++m) {
             if (ks < p.ks1 && mbase + m < M) {
-              yv[ks][m] = ld_tag(&p.ypart[(((int64_t)ks * p.b + yj) * M + mbase + m) * p.R + yr]);
+              yv[ks][m] = ld_tag(&p.ypart[(((int64_t)ks * p.b + yj) * M + mbase + m) * (p.R >> 1) + (yr >> 1)]);
               ok = ok && ((unsigned)(yv[ks][m] >> 32) == epoch);
             } else {
               yv[ks][m] = 0ull;
@@ -855,7 +870,11 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int m = 0; m < DM_MC; ++m) ysum[m] += __uint_as_float((unsigned)yv[ks][m]);
+        for (int m = 0; m < DM_MC; ++m) {                          // this thread's rank is one half of the pair
+          typedef T T2 __attribute__((ext_vector_type(2)));
+          const T2 pr = __builtin_bit_cast(T2, (unsigned)yv[ks][m]);
+          ysum[m] += TypeTraits<T>::to_f32((yr & 1) ? pr[1] : pr[0]);
+        }
     }
 #pragma unroll
     for (int m = 0; m < DM_MC; ++m) ys[m * 256 + tid] = ysum[m];
@@ -966,12 +985,31 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
       else dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
     }
   }
-  for (int bq = p.pfn / 8; bq * DM_ROWS < kcur2; ++bq) {          // deeper slabs: stream the rest
-    u32x4 cur[8];
+  {
+    // Deeper slabs: the rest is asked for in one go (up to DM_PF more loads per lane, into the registers the
+    // products above have freed), so it costs one trip to memory and not one per batch.  The loads are
+    // unconditional: a batch past the end of the slab gets an offset beyond the buffer, which reads as zero
+    // without touching memory, and is not multiplied.
+    const int nbq = (kcur2 + DM_ROWS - 1) / DM_ROWS;
+    for (int b0 = p.pfn / 8; b0 < nbq; b0 += DM_PF / 8) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) cur[u] = ldw16(ubuf, uoff, u_soff(bq, u));
-    if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
-    else dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+      for (int bq = 0; bq < DM_PF / 8; ++bq) {
+        const bool in_slab = b0 + bq < nbq;
+        const uint32_t vo = in_slab ? uoff : 0x80000000u;           // the per-lane offset is what the bounds check sees
+#pragma unroll
+        for (int u = 0; u < 8; ++u) pf[bq * 8 + u] = ldw16(ubuf, vo, in_slab ? u_soff(b0 + bq, u) : 0u);
+      }
+#pragma unroll
+      for (int bq = 0; bq < DM_PF / 8; ++bq) {
+        if (b0 + bq < nbq) {
+          u32x4 cur[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) cur[u] = pf[bq * 8 + u];
+          if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
+          else dm_batch<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
+        }
+      }
+    }
   }
   TR2(5);
   T* outp = reinterpret_cast<T*>(p.out);
