@@ -522,19 +522,40 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   for (int m = 0; m < MT; ++m)
 #pragma unroll
     for (int e = 0; e < EPL; ++e) acc[m][e] = 0.0f;
+  if constexpr (MT * EPL <= 32) {
+    // The activations of all register-resident rows are read from LDS up front (one wait), so the products below
+    // run back to back instead of paying an LDS round trip per row.  Slots at or beyond pfn are read but not used.
+    float av[MT][D2_PF];
 #pragma unroll
-  for (int u = 0; u < D2_PF; ++u) {
-    const int k = rs2 + u * rpp2;
-    if (u < p.pfn) {
-      float wv[EPL];
-      cvtw<T, WB>(pf[u], wv);
+    for (int u = 0; u < D2_PF; ++u)
 #pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        const float a = a_s[m * KLD + k];              // zero beyond the slice
+      for (int m = 0; m < MT; ++m) av[m][u] = a_s[m * KLD + ((rs2 + u * rpp2) & (KLD - 1))];   // zero beyond the slice
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
+    for (int u = 0; u < D2_PF; ++u) {
+      if (u < p.pfn) {
+        float wv[EPL];
+        cvtw<T, WB>(pf[u], wv);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) acc[m][e] = fmaf(av[m][u], wv[e], acc[m][e]);
       }
-      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {                                             // wide accumulators: no registers to spare for that
+#pragma unroll
+    for (int u = 0; u < D2_PF; ++u) {
+      const int k = rs2 + u * rpp2;
+      if (u < p.pfn) {
+        float wv[EPL];
+        cvtw<T, WB>(pf[u], wv);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float a = a_s[m * KLD + k];            // zero beyond the slice
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) acc[m][e] = fmaf(a, wv[e], acc[m][e]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
   {
@@ -1169,36 +1190,6 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
   const int lpr_cap = D2_NC_MAX / EPL;           // widest column chunk the reduction buffer holds
 
-  // stage 1: column chunks of EPL * lpr1 ranks; k split only as far as needed to engage the chip
-  {
-    static const int e_lpr = env_i("BLR_D2_LPR1", 16), e_ks = env_i("BLR_D2_KS1", 0);
-    int lpr = e_lpr < lpr_cap ? e_lpr : lpr_cap;
-    const int vecs = (R + EPL - 1) / EPL;
-    while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
-    if (lpr > 64) lpr = 64;
-    if (lpr > lpr_cap) lpr = lpr_cap;
-    if (lpr < 4) lpr = 4;
-    const int rpp = 256 / lpr;
-    const int nch = (vecs + lpr - 1) / lpr;
-    const int base = b * nch;
-    if (base > resident) return d2_bail(__LINE__);
-    // split k just far enough that a lane's share of a slice is one batch of loads
-    const int ks_max = d2_ks1_max(MT);
-    int ks = e_ks > 0 ? e_ks : ((P + rpp - 1) / rpp + d2_unr1(MT) - 1) / d2_unr1(MT);
-    if (ks > resident / base) ks = resident / base;
-    if (ks > ks_max) ks = ks_max;
-    if (ks > (P + rpp - 1) / rpp) ks = (P + rpp - 1) / rpp;     // at least one load per lane
-    if (ks < 1) ks = 1;
-    int kc = (P + ks - 1) / ks;
-    kc = (kc + rpp - 1) / rpp * rpp;
-    if (kc > kc_cap) kc = kc_cap / rpp * rpp;
-    if (kc < 1) return d2_bail(__LINE__);
-    ks = (P + kc - 1) / kc;
-    if (ks > ks_max || base * ks > resident) return d2_bail(__LINE__);
-    const int unr1 = d2_unr1(MT);
-    if (((kc + rpp - 1) / rpp + unr1 - 1) / unr1 * unr1 * rpp > D2_AS / MT) return d2_bail(__LINE__);   // zero padding must fit too
-    p.lpr1_log2 = ilog2(lpr); p.nch1 = nch; p.ks1 = ks; p.kc1 = kc; p.items1 = base * ks;
-  }
   if (a.u_layout == BLR_U_QR) {
     // stage 2 on U (bo, q, r): a wave takes rpw rows, a lane 8 of every 512 k; everything a lane loads stays in registers
     // shapes this geometry does not hold (rows of a wave times k pieces beyond the registers of a lane) go to the
@@ -1243,6 +1234,44 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     const int kpad2 = (pfn + (left > 0 ? (left + D2_UNR - 1) / D2_UNR * D2_UNR : 0)) * rpp;
     if (kpad2 > D2_AS / MT) return d2_bail(__LINE__);
     p.lpr2_log2 = ilog2(lpr); p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn; p.kpad2 = kpad2;
+  }
+  // stage 1: column chunks of EPL * lpr1 ranks; k split only as far as needed to engage the chip
+  {
+    static const int e_lpr = env_i("BLR_D2_LPR1", 16), e_ks = env_i("BLR_D2_KS1", 0);
+    int lpr = e_lpr < lpr_cap ? e_lpr : lpr_cap;
+    const int vecs = (R + EPL - 1) / EPL;
+    while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
+    if (lpr > 64) lpr = 64;
+    if (lpr > lpr_cap) lpr = lpr_cap;
+    if (lpr < 4) lpr = 4;
+    const int rpp = 256 / lpr;
+    const int nch = (vecs + lpr - 1) / lpr;
+    const int base = b * nch;
+    if (base > resident) return d2_bail(__LINE__);
+    // split k just far enough that a lane's share of a slice is one batch of loads
+    const int ks_max = d2_ks1_max(MT);
+    int ks = e_ks > 0 ? e_ks : ((P + rpp - 1) / rpp + d2_unr1(MT) - 1) / d2_unr1(MT);
+    if (ks > resident / base) ks = resident / base;
+    // A workgroup that owns both a stage-1 item and a slab of U starts streaming its slab only after its stage-1
+    // work and ends last: when a slightly coarser k split lets every item have a workgroup of its own, take it
+    // (as long as a lane's share of a slice still fits two batches of loads).
+    static const int e_solo = env_i("BLR_D2_SOLO", 1);
+    if (e_solo && e_ks <= 0 && base + p.items2 <= resident && base * ks + p.items2 > resident) {
+      const int ks_solo = (resident - p.items2) / base;
+      if (((P + ks_solo - 1) / ks_solo + rpp - 1) / rpp <= 2 * d2_unr1(MT)) ks = ks_solo;
+    }
+    if (ks > ks_max) ks = ks_max;
+    if (ks > (P + rpp - 1) / rpp) ks = (P + rpp - 1) / rpp;     // at least one load per lane
+    if (ks < 1) ks = 1;
+    int kc = (P + ks - 1) / ks;
+    kc = (kc + rpp - 1) / rpp * rpp;
+    if (kc > kc_cap) kc = kc_cap / rpp * rpp;
+    if (kc < 1) return d2_bail(__LINE__);
+    ks = (P + kc - 1) / kc;
+    if (ks > ks_max || base * ks > resident) return d2_bail(__LINE__);
+    const int unr1 = d2_unr1(MT);
+    if (((kc + rpp - 1) / rpp + unr1 - 1) / unr1 * unr1 * rpp > D2_AS / MT) return d2_bail(__LINE__);   // zero padding must fit too
+    p.lpr1_log2 = ilog2(lpr); p.nch1 = nch; p.ks1 = ks; p.kc1 = kc; p.items1 = base * ks;
   }
   {
     p.zrep = bo == 1 ? 16 : 1;
