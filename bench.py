@@ -35,7 +35,7 @@ B = 16
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE), scaled
 # by the same counters over a copy kernel of known size (1 FETCH_SIZE unit = 1.99978 KiB, 1 WRITE_SIZE unit = 1 KiB).
-TRAFFIC_BYTES = 71.06e6   # 70.43 MB fetched + 0.63 MB written (profiles/decode2_kernel_blast_llama7b_decode_m1.txt)
+TRAFFIC_BYTES = 70.86e6   # 70.36 MB fetched + 0.50 MB written (profiles/decode2_kernel_blast_llama7b_decode_m1.txt)
 
 
 def blast_bytes_flops(n, i, r, o, b=B, elt=2):
