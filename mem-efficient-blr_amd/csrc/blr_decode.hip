@@ -662,6 +662,43 @@ __device__ __forceinline__ void dm_batch_nk(const u32x4 (&cur)[8], const T* a_s,
   for (int e = 0; e < 8; ++e) acc[e] = TypeTraits<T>::mfma16(af, __builtin_bit_cast(V8, cur[e]), acc[e]);
 }
 
+// Two int8 codes sitting in bytes 0 and 2 of t (bytes 1 and 3 zero) -> two T values in one register.
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float a, float b);
+template <typename T>
+__device__ __forceinline__ uint32_t cvt_pair_i8(uint32_t t) {
+  if constexpr (sizeof(T) == 2 && __is_same(T, f16)) {
+    // 0x6400 | (code ^ 0x80) is the half 1024 + (code + 128); one packed subtraction gives the code exactly
+    const f16x2 v = __builtin_bit_cast(f16x2, t ^ 0x64806480u) - f16x2{(f16)1152.0f, (f16)1152.0f};
+    return __builtin_bit_cast(uint32_t, v);
+  } else {
+    return pack2<T>((float)(int8_t)(t & 0xffu), (float)(int8_t)((t >> 16) & 0xffu));
+  }
+}
+// The batch for int8 codes stored (k, n): load u is row k + u of the lane's 8 columns, 8 bytes.  Fragment e takes byte e of
+// rows 2q and 2q + 1 with one byte permute, which is the transpose and the widening to two-byte slots at once.
+template <typename T>
+__device__ __forceinline__ void dm_batch_i8(const u32x2 (&cur)[8], const T* a_s, int ald, int cv, int rs, int kbase, f32x4 (&acc)[8]) {
+  using V8 = typename TypeTraits<T>::vec8;
+  const V8 af = *reinterpret_cast<const V8*>(&a_s[cv * ald + kbase + rs * 8]);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const uint32_t sel = 0x0c000c00u | ((4u + (e & 3)) << 16) | (uint32_t)(e & 3);
+    u32x4 bb;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) bb[q] = cvt_pair_i8<T>(__builtin_amdgcn_perm(cur[2 * q + 1][e >> 2], cur[2 * q][e >> 2], sel));
+    acc[e] = TypeTraits<T>::mfma16(af, __builtin_bit_cast(V8, bb), acc[e]);
+  }
+}
+// one lane's piece of a weight row: 8 columns, 16 bytes of two-byte values or 8 bytes of int8 codes
+template <int WB> struct DmLoad { using type = u32x4; };
+template <> struct DmLoad<8> { using type = u32x2; };
+template <int WB>
+__device__ __forceinline__ typename DmLoad<WB>::type ldw8(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  if constexpr (WB == 8) return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 2));
+  else return ldw16(r, voff, soff);
+}
+
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
   typedef T T2 __attribute__((ext_vector_type(2)));
@@ -669,8 +706,12 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-template <typename T>
+template <typename T, int WB>
 __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
+  static_assert(WB == 16 || WB == 8, "two-byte weights or int8 codes");
+  constexpr int PFN = WB == 8 ? 2 * DM_PF : DM_PF;     // loads of the U slab kept in registers (the same 128 registers)
+  constexpr int WBY = WB / 8;                          // bytes per weight
+  using LV = typename DmLoad<WB>::type;
   __shared__ __attribute__((aligned(16))) T a_s[16 * (DM_KMAX + 8)];
   __shared__ __attribute__((aligned(16))) float red[4 * 4 * 64 * 4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -700,24 +741,24 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   const int n0_2 = nc2 * 128;
   const int n2 = n0_2 + cv * 8;
   const bool col_ok2 = n2 < p.Q;
-  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.bo * p.R * p.Q * 2u);
+  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.bo * p.R * p.Q * (uint32_t)WBY);
   // U (bo, r, q): load u of a batch is row k + u of the lane's 8 columns.  U (bo, q, r): load u is row q = column u of
   // the lane's 8, at the lane's 8 consecutive k - already a B fragment, so no transpose follows.
   const uint32_t uoff = p.u_nk ? (uint32_t)((((int64_t)i2 * p.Q + (col_ok2 ? n2 : 0)) * p.R + k0_2 + rs * 8) * 2)
-                               : (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs * 8) * p.Q + (col_ok2 ? n2 : 0)) * 2);
-  const uint32_t urow = (uint32_t)p.Q * 2u;
+                               : (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs * 8) * p.Q + (col_ok2 ? n2 : 0)) * WBY);
+  const uint32_t urow = (uint32_t)p.Q * (uint32_t)WBY;
   auto u_soff = [&](int batch, int u) -> uint32_t {
     return p.u_nk ? (uint32_t)((u * p.R + batch * DM_ROWS) * 2) : (uint32_t)(batch * DM_ROWS + u) * urow;
   };
-  u32x4 pf[DM_PF];
+  LV pf[PFN];
   auto issue_prefetch = [&]() {
 #pragma unroll
-    for (int u = 0; u < DM_PF; ++u) {
+    for (int u = 0; u < PFN; ++u) {
       if (u < p.pfn) {
         if (u >= 4 && p.pf_depth == 4) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
         else if (u >= 8 && p.pf_depth == 8) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
         else if (u >= 16 && p.pf_depth == 16) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
-        pf[u] = ldw16(ubuf, uoff, u_soff(u >> 3, u & 7));
+        pf[u] = ldw8<WB>(ubuf, uoff, u_soff(u >> 3, u & 7));
       }
     }
   };
@@ -768,14 +809,14 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     const int k0 = ks * p.kc1, kc = min(p.kc1, p.P - k0);
     const int n0 = nc1 * 128, n = n0 + cv * 8;
     const bool col_ok = n < p.R;
-    const __amdgpu_buffer_rsrc_t vbuf = wbuf(p.V, (uint32_t)p.b * p.P * p.R * 2u);
-    const uint32_t voff = (uint32_t)((((int64_t)j * p.P + k0 + rs * 8) * p.R + (col_ok ? n : 0)) * 2);
-    const uint32_t vrow = (uint32_t)p.R * 2u;
+    const __amdgpu_buffer_rsrc_t vbuf = wbuf(p.V, (uint32_t)p.b * p.P * p.R * (uint32_t)WBY);
+    const uint32_t voff = (uint32_t)((((int64_t)j * p.P + k0 + rs * 8) * p.R + (col_ok ? n : 0)) * WBY);
+    const uint32_t vrow = (uint32_t)p.R * (uint32_t)WBY;
     const int nbatch = (kc + DM_ROWS - 1) / DM_ROWS;
     const int kpad = nbatch * DM_ROWS, ald = kpad + 8;
-    u32x4 raw[8];
+    LV raw[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) raw[u] = ldw16(vbuf, voff, (uint32_t)u * vrow);
+    for (int u = 0; u < 8; ++u) raw[u] = ldw8<WB>(vbuf, voff, (uint32_t)u * vrow);
     // activations straight into LDS as T (zero outside the slice and beyond M)
     const T* xp = reinterpret_cast<const T*>(p.x);
     if (p.x_vec) {                                               // 16-byte pieces: one or two per thread
@@ -805,14 +846,15 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     for (int bi = 0; bi < nbatch; ++bi) {
-      u32x4 cur[8];
+      LV cur[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) cur[u] = raw[u];
       if (bi + 1 < nbatch) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) raw[u] = ldw16(vbuf, voff, (uint32_t)((bi + 1) * DM_ROWS + u) * vrow);
+        for (int u = 0; u < 8; ++u) raw[u] = ldw8<WB>(vbuf, voff, (uint32_t)((bi + 1) * DM_ROWS + u) * vrow);
       }
-      dm_batch<T>(cur, a_s, ald, cv, rs, bi * DM_ROWS, acc);
+      if constexpr (WB == 8) dm_batch_i8<T>(cur, a_s, ald, cv, rs, bi * DM_ROWS, acc);
+      else dm_batch<T>(cur, a_s, ald, cv, rs, bi * DM_ROWS, acc);
     }
     TR2(1);
     // y crosses workgroups as {two T values (ranks 2c, 2c + 1), epoch} pairs.  The totals go through LDS once more so
@@ -820,10 +862,15 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     constexpr int YLD = 130;
     reduce_emit(acc, [&](int col, int m0, const f32x4 (&vh)[2]) {
       __syncthreads();                                            // every thread has read its sums out of red
+      float vsc[2] = {1.0f, 1.0f};                                // int8 codes of V: one scale per rank
+      if constexpr (WB == 8) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) vsc[h] = (float)p.v_scales[(int64_t)j * p.R + min(n0 + col + 4 * h, p.R - 1)];
+      }
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) red[(m0 + i) * YLD + col + 4 * h] = vh[h][i];
+        for (int i = 0; i < 4; ++i) red[(m0 + i) * YLD + col + 4 * h] = vh[h][i] * vsc[h];
     });
     __syncthreads();
     {
@@ -997,12 +1044,13 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-  for (int bq = 0; bq < DM_PF / 8; ++bq) {
+  for (int bq = 0; bq < PFN / 8; ++bq) {
     if (bq * 8 < p.pfn) {
-      u32x4 cur[8];
+      LV cur[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) cur[u] = pf[bq * 8 + u];
-      if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+      if constexpr (WB == 8) dm_batch_i8<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+      else if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
       else dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
     }
   }
@@ -1012,21 +1060,22 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     // unconditional: a batch past the end of the slab gets an offset beyond the buffer, which reads as zero
     // without touching memory, and is not multiplied.
     const int nbq = (kcur2 + DM_ROWS - 1) / DM_ROWS;
-    for (int b0 = p.pfn / 8; b0 < nbq; b0 += DM_PF / 8) {
+    for (int b0 = p.pfn / 8; b0 < nbq; b0 += PFN / 8) {
 #pragma unroll
-      for (int bq = 0; bq < DM_PF / 8; ++bq) {
+      for (int bq = 0; bq < PFN / 8; ++bq) {
         const bool in_slab = b0 + bq < nbq;
         const uint32_t vo = in_slab ? uoff : 0x80000000u;           // the per-lane offset is what the bounds check sees
 #pragma unroll
-        for (int u = 0; u < 8; ++u) pf[bq * 8 + u] = ldw16(ubuf, vo, in_slab ? u_soff(b0 + bq, u) : 0u);
+        for (int u = 0; u < 8; ++u) pf[bq * 8 + u] = ldw8<WB>(ubuf, vo, in_slab ? u_soff(b0 + bq, u) : 0u);
       }
 #pragma unroll
-      for (int bq = 0; bq < DM_PF / 8; ++bq) {
+      for (int bq = 0; bq < PFN / 8; ++bq) {
         if (b0 + bq < nbq) {
-          u32x4 cur[8];
+          LV cur[8];
 #pragma unroll
           for (int u = 0; u < 8; ++u) cur[u] = pf[bq * 8 + u];
-          if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
+          if constexpr (WB == 8) dm_batch_i8<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
+          else if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
           else dm_batch<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
         }
       }
@@ -1088,9 +1137,11 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int gn = n0_2 + col + 4 * h;
+      float usc = 1.0f;                                              // int8 codes of U: one scale per output column
+      if constexpr (WB == 8) usc = (float)p.u_scales[(int64_t)i2 * p.Q + min(gn, p.Q - 1)];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (gn < p.Q && m0 + i < M) outp[(int64_t)(m0 + i) * p.ldo + (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns] = TypeTraits<T>::from_f32(tot[h][i]);
+        if (gn < p.Q && m0 + i < M) outp[(int64_t)(m0 + i) * p.ldo + (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns] = TypeTraits<T>::from_f32(tot[h][i] * usc);
     }
   });
   TR2(7);
@@ -1137,7 +1188,8 @@ bool decode2_applicable(const StreamBlastArgs& a) {
   static const int nk_on = env_i("BLR_D2_NK", 1);
   if (a.u_layout != BLR_U_RQ && !(nk_on && a.u_layout == BLR_U_QR && a.wbits == 16)) return false;
   if (a.wbits != 16 && (a.wbits != 8 && a.wbits != 4)) return false;
-  if (a.wbits != 16 && (a.M > 4 || !a.u_scales || !a.v_scales)) return false;   // the matrix-core variant takes two-byte weights only
+  if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return false;
+  if (a.wbits == 4 && a.M > 4) return false;                                     // the matrix-core variant takes two-byte weights and int8 codes
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
   if (a.M < 1 || a.M > 16) return false;
   const int P = a.in_f / a.b, Q = a.out_f / (a.bo > 0 ? a.bo : a.b);
@@ -1157,7 +1209,8 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
   static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
-  if (M >= mfma_min_m && a.wbits == 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);   // codes stay with the vector variant
+  if (M >= mfma_min_m && a.wbits == 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
+  if (M > 4 && a.wbits == 8) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);             // below that, codes stay with the vector variant
   if (M > 4) return d2_bail(__LINE__);
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int WBITS = a.wbits, EPL = 128 / WBITS;  // weights per 16-byte load
@@ -1311,7 +1364,9 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
                           unsigned* err_word, hipStream_t st) {
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
-  void* fn = a.dtype == BLR_F16 ? (void*)decode2m_kernel<f16> : (void*)decode2m_kernel<bf16>;
+  if (a.wbits != 16 && !(a.wbits == 8 && a.u_layout == BLR_U_RQ && a.u_scales && a.v_scales)) return d2_bail(__LINE__);   // two-byte weights, or int8 codes stored (k, n)
+  void* fn = a.wbits == 8 ? (a.dtype == BLR_F16 ? (void*)decode2m_kernel<f16, 8> : (void*)decode2m_kernel<bf16, 8>)
+                          : (a.dtype == BLR_F16 ? (void*)decode2m_kernel<f16, 16> : (void*)decode2m_kernel<bf16, 16>);
   static std::mutex mu;
   static std::map<void*, int> occ_cache;
   int occ = 0;
@@ -1328,10 +1383,10 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
   const int cus = device_cus() > 0 ? device_cus() : 256;
   const int resident = (occ < 2 ? occ : 2) * cus;
   if (R % 4) return d2_bail(__LINE__);
-  if (a.wbits != 16) return d2_bail(__LINE__);       // this kernel reads two-byte weights; its buffer bounds assume them
 
   Decode2Params p = {};
   p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
+  p.u_scales = (const f16*)a.u_scales; p.v_scales = (const f16*)a.v_scales;
   p.M = M; p.b = b; p.bo = bo; p.P = P; p.R = R; p.Q = Q;
   p.perm_per = a.perm_per; p.o_bs = a.out_ns ? a.out_bs : Q; p.o_ns = a.out_ns ? a.out_ns : 1;
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
@@ -1372,7 +1427,8 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     ks = (R + kc - 1) / kc;
     if (ks > 4 || base * ks > resident) return d2_bail(__LINE__);
     int pfn = (kc + DM_ROWS - 1) / DM_ROWS * 8;
-    if (pfn > DM_PF) pfn = DM_PF;
+    const int pf_cap = a.wbits == 8 ? 2 * DM_PF : DM_PF;     // 8-byte loads of codes: twice as many in the same registers
+    if (pfn > pf_cap) pfn = pf_cap;
     p.lpr2_log2 = 4; p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn;
     p.kpad2 = (kc + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
     p.u_nk = a.u_layout == BLR_U_QR;
