@@ -359,9 +359,9 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   hipStream_t st = (hipStream_t)stream;
   const bool phase_engine = algo == BLR_ALGO_STREAM || algo == BLR_ALGO_STREAM_SPLIT;
   if (M > 16 && phase_engine) { set_error("blast_q: M=%d > 16 not served by the streaming kernel", M); return BLR_ERR_UNSUPPORTED; }
-  // int8 codes at 5..16 rows go to the matrix-core decode kernel as they are (it widens them in registers)
+  // codes at 5..16 rows go to the matrix-core decode kernel as they are (it widens them in registers)
   static const bool i8_direct = !getenv("BLR_Q_DIRECT") || atoi(getenv("BLR_Q_DIRECT")) != 0;
-  const bool direct = bits == 8 && M <= 16 && i8_direct;
+  const bool direct = M <= 16 && i8_direct;
   if (M > 4 && !phase_engine && !direct) {
     size_t need = blr_blast_q_workspace_bytes(M, in_f, out_f, b, r, bits);
     if (!ws || ws_bytes < need) { set_error("blast_q: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }

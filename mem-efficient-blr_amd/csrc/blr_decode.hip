@@ -690,12 +690,45 @@ __device__ __forceinline__ void dm_batch_i8(const u32x2 (&cur)[8], const T* a_s,
     acc[e] = TypeTraits<T>::mfma16(af, __builtin_bit_cast(V8, bb), acc[e]);
   }
 }
-// one lane's piece of a weight row: 8 columns, 16 bytes of two-byte values or 8 bytes of int8 codes
+// Two int4 codes (two's complement nibbles) sitting in bytes 0 and 2 of t -> two T values in one register.
+template <typename T>
+__device__ __forceinline__ uint32_t cvt_pair_i4(uint32_t t) {
+  if constexpr (sizeof(T) == 2 && __is_same(T, f16)) {
+    // 0x6400 | (nibble ^ 8) is the half 1024 + (code + 8)
+    const f16x2 v = __builtin_bit_cast(f16x2, t ^ 0x64086408u) - f16x2{(f16)1032.0f, (f16)1032.0f};
+    return __builtin_bit_cast(uint32_t, v);
+  } else {
+    return pack2<T>((float)((int)((t & 0xfu) ^ 8u) - 8), (float)((int)(((t >> 16) & 0xfu) ^ 8u) - 8));
+  }
+}
+// The batch for packed int4 codes stored (k, n), even column in the low nibble: load u is row k + u of the lane's 8 columns,
+// 4 bytes.  Each row is split into its even and odd columns as bytes; from there it is the int8 scheme.
+template <typename T>
+__device__ __forceinline__ void dm_batch_i4(const uint32_t (&cur)[8], const T* a_s, int ald, int cv, int rs, int kbase, f32x4 (&acc)[8]) {
+  using V8 = typename TypeTraits<T>::vec8;
+  const V8 af = *reinterpret_cast<const V8*>(&a_s[cv * ald + kbase + rs * 8]);
+  uint32_t ev[8], od[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) { ev[u] = cur[u] & 0x0f0f0f0fu; od[u] = (cur[u] >> 4) & 0x0f0f0f0fu; }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int c = e >> 1;
+    const uint32_t sel = 0x0c000c00u | ((4u + c) << 16) | (uint32_t)c;
+    u32x4 bb;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      bb[q] = cvt_pair_i4<T>((e & 1) ? __builtin_amdgcn_perm(od[2 * q + 1], od[2 * q], sel) : __builtin_amdgcn_perm(ev[2 * q + 1], ev[2 * q], sel));
+    acc[e] = TypeTraits<T>::mfma16(af, __builtin_bit_cast(V8, bb), acc[e]);
+  }
+}
+// one lane's piece of a weight row: 8 columns = 16 bytes of two-byte values, 8 bytes of int8 codes or 4 bytes of int4 codes
 template <int WB> struct DmLoad { using type = u32x4; };
 template <> struct DmLoad<8> { using type = u32x2; };
+template <> struct DmLoad<4> { using type = uint32_t; };
 template <int WB>
 __device__ __forceinline__ typename DmLoad<WB>::type ldw8(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
   if constexpr (WB == 8) return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 2));
+  else if constexpr (WB == 4) return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 2);
   else return ldw16(r, voff, soff);
 }
 
@@ -708,9 +741,8 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 
 template <typename T, int WB>
 __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
-  static_assert(WB == 16 || WB == 8, "two-byte weights or int8 codes");
-  constexpr int PFN = WB == 8 ? 2 * DM_PF : DM_PF;     // loads of the U slab kept in registers (the same 128 registers)
-  constexpr int WBY = WB / 8;                          // bytes per weight
+  static_assert(WB == 16 || WB == 8 || WB == 4, "two-byte weights, int8 codes or packed int4 codes");
+  constexpr int PFN = WB == 16 ? DM_PF : 2 * DM_PF;    // loads of the U slab kept in registers (codes: a whole 1024-row slab)
   using LV = typename DmLoad<WB>::type;
   __shared__ __attribute__((aligned(16))) T a_s[16 * (DM_KMAX + 8)];
   __shared__ __attribute__((aligned(16))) float red[4 * 4 * 64 * 4];
@@ -741,12 +773,12 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   const int n0_2 = nc2 * 128;
   const int n2 = n0_2 + cv * 8;
   const bool col_ok2 = n2 < p.Q;
-  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)p.bo * p.R * p.Q * (uint32_t)WBY);
+  const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)((int64_t)p.bo * p.R * p.Q * WB / 8));
   // U (bo, r, q): load u of a batch is row k + u of the lane's 8 columns.  U (bo, q, r): load u is row q = column u of
   // the lane's 8, at the lane's 8 consecutive k - already a B fragment, so no transpose follows.
   const uint32_t uoff = p.u_nk ? (uint32_t)((((int64_t)i2 * p.Q + (col_ok2 ? n2 : 0)) * p.R + k0_2 + rs * 8) * 2)
-                               : (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs * 8) * p.Q + (col_ok2 ? n2 : 0)) * WBY);
-  const uint32_t urow = (uint32_t)p.Q * (uint32_t)WBY;
+                               : (uint32_t)((((int64_t)i2 * p.R + k0_2 + rs * 8) * p.Q + (col_ok2 ? n2 : 0)) * WB / 8);
+  const uint32_t urow = (uint32_t)p.Q * (uint32_t)WB / 8u;
   auto u_soff = [&](int batch, int u) -> uint32_t {
     return p.u_nk ? (uint32_t)((u * p.R + batch * DM_ROWS) * 2) : (uint32_t)(batch * DM_ROWS + u) * urow;
   };
@@ -809,9 +841,9 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     const int k0 = ks * p.kc1, kc = min(p.kc1, p.P - k0);
     const int n0 = nc1 * 128, n = n0 + cv * 8;
     const bool col_ok = n < p.R;
-    const __amdgpu_buffer_rsrc_t vbuf = wbuf(p.V, (uint32_t)p.b * p.P * p.R * (uint32_t)WBY);
-    const uint32_t voff = (uint32_t)((((int64_t)j * p.P + k0 + rs * 8) * p.R + (col_ok ? n : 0)) * WBY);
-    const uint32_t vrow = (uint32_t)p.R * (uint32_t)WBY;
+    const __amdgpu_buffer_rsrc_t vbuf = wbuf(p.V, (uint32_t)((int64_t)p.b * p.P * p.R * WB / 8));
+    const uint32_t voff = (uint32_t)((((int64_t)j * p.P + k0 + rs * 8) * p.R + (col_ok ? n : 0)) * WB / 8);
+    const uint32_t vrow = (uint32_t)p.R * (uint32_t)WB / 8u;
     const int nbatch = (kc + DM_ROWS - 1) / DM_ROWS;
     const int kpad = nbatch * DM_ROWS, ald = kpad + 8;
     LV raw[8];
@@ -854,6 +886,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
         for (int u = 0; u < 8; ++u) raw[u] = ldw8<WB>(vbuf, voff, (uint32_t)((bi + 1) * DM_ROWS + u) * vrow);
       }
       if constexpr (WB == 8) dm_batch_i8<T>(cur, a_s, ald, cv, rs, bi * DM_ROWS, acc);
+      else if constexpr (WB == 4) dm_batch_i4<T>(cur, a_s, ald, cv, rs, bi * DM_ROWS, acc);
       else dm_batch<T>(cur, a_s, ald, cv, rs, bi * DM_ROWS, acc);
     }
     TR2(1);
@@ -863,7 +896,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     reduce_emit(acc, [&](int col, int m0, const f32x4 (&vh)[2]) {
       __syncthreads();                                            // every thread has read its sums out of red
       float vsc[2] = {1.0f, 1.0f};                                // int8 codes of V: one scale per rank
-      if constexpr (WB == 8) {
+      if constexpr (WB != 16) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) vsc[h] = (float)p.v_scales[(int64_t)j * p.R + min(n0 + col + 4 * h, p.R - 1)];
       }
@@ -1050,6 +1083,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
       for (int u = 0; u < 8; ++u) cur[u] = pf[bq * 8 + u];
       if constexpr (WB == 8) dm_batch_i8<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
+      else if constexpr (WB == 4) dm_batch_i4<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
       else if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
       else dm_batch<T>(cur, a_s, ald2, cv, rs, bq * DM_ROWS, acc);
     }
@@ -1075,6 +1109,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 #pragma unroll
           for (int u = 0; u < 8; ++u) cur[u] = pf[bq * 8 + u];
           if constexpr (WB == 8) dm_batch_i8<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
+          else if constexpr (WB == 4) dm_batch_i4<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
           else if (p.u_nk) dm_batch_nk<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
           else dm_batch<T>(cur, a_s, ald2, cv, rs, (b0 + bq) * DM_ROWS, acc);
         }
@@ -1138,7 +1173,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     for (int h = 0; h < 2; ++h) {
       const int gn = n0_2 + col + 4 * h;
       float usc = 1.0f;                                              // int8 codes of U: one scale per output column
-      if constexpr (WB == 8) usc = (float)p.u_scales[(int64_t)i2 * p.Q + min(gn, p.Q - 1)];
+      if constexpr (WB != 16) usc = (float)p.u_scales[(int64_t)i2 * p.Q + min(gn, p.Q - 1)];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         if (gn < p.Q && m0 + i < M) outp[(int64_t)(m0 + i) * p.ldo + (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns] = TypeTraits<T>::from_f32(tot[h][i] * usc);
@@ -1189,7 +1224,6 @@ bool decode2_applicable(const StreamBlastArgs& a) {
   if (a.u_layout != BLR_U_RQ && !(nk_on && a.u_layout == BLR_U_QR && a.wbits == 16)) return false;
   if (a.wbits != 16 && (a.wbits != 8 && a.wbits != 4)) return false;
   if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return false;
-  if (a.wbits == 4 && a.M > 4) return false;                                     // the matrix-core variant takes two-byte weights and int8 codes
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
   if (a.M < 1 || a.M > 16) return false;
   const int P = a.in_f / a.b, Q = a.out_f / (a.bo > 0 ? a.bo : a.b);
@@ -1210,7 +1244,8 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
   static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
   if (M >= mfma_min_m && a.wbits == 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
-  if (M > 4 && a.wbits == 8) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);             // below that, codes stay with the vector variant
+  static const int q_mfma_min_m = env_i("BLR_D2_Q_MFMA_MIN_M", 3);
+  if ((M > 4 || M >= q_mfma_min_m) && a.wbits != 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);   // below that, codes stay with the vector variant
   if (M > 4) return d2_bail(__LINE__);
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int WBITS = a.wbits, EPL = 128 / WBITS;  // weights per 16-byte load
@@ -1364,8 +1399,9 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
                           unsigned* err_word, hipStream_t st) {
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
-  if (a.wbits != 16 && !(a.wbits == 8 && a.u_layout == BLR_U_RQ && a.u_scales && a.v_scales)) return d2_bail(__LINE__);   // two-byte weights, or int8 codes stored (k, n)
+  if (a.wbits != 16 && !((a.wbits == 8 || a.wbits == 4) && a.u_layout == BLR_U_RQ && a.u_scales && a.v_scales)) return d2_bail(__LINE__);   // two-byte weights, or codes stored (k, n)
   void* fn = a.wbits == 8 ? (a.dtype == BLR_F16 ? (void*)decode2m_kernel<f16, 8> : (void*)decode2m_kernel<bf16, 8>)
+           : a.wbits == 4 ? (a.dtype == BLR_F16 ? (void*)decode2m_kernel<f16, 4> : (void*)decode2m_kernel<bf16, 4>)
                           : (a.dtype == BLR_F16 ? (void*)decode2m_kernel<f16, 16> : (void*)decode2m_kernel<bf16, 16>);
   static std::mutex mu;
   static std::map<void*, int> occ_cache;
@@ -1427,7 +1463,7 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     ks = (R + kc - 1) / kc;
     if (ks > 4 || base * ks > resident) return d2_bail(__LINE__);
     int pfn = (kc + DM_ROWS - 1) / DM_ROWS * 8;
-    const int pf_cap = a.wbits == 8 ? 2 * DM_PF : DM_PF;     // 8-byte loads of codes: twice as many in the same registers
+    const int pf_cap = a.wbits == 16 ? DM_PF : 2 * DM_PF;    // narrower loads of codes: twice as many in no more registers
     if (pfn > pf_cap) pfn = pf_cap;
     p.lpr2_log2 = 4; p.nch2 = nch; p.ks2 = ks; p.kc2 = kc; p.items2 = base * ks; p.pfn = pfn;
     p.kpad2 = (kc + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
