@@ -334,9 +334,9 @@ int blr_blast_i8act_fwd(const void* x, int64_t ldx, const void* U, const void* V
 // ---- quantized BLAST -----------------------------------------------------------------------------
 size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits) {
   if (M <= 0 || b <= 0 || r <= 0) return 0;
-  // M <= 4 streams the codes.  Above that the factors are expanded to two-byte values once per call
-  // ([kernel workspace][U][V]) and the two-byte kernels run: the matrix-core decode kernel up to 16 rows,
-  // the tiled kernels beyond.  Requests for the phase engine (BLR_ALGO_STREAM*) stream codes up to M = 16.
+  // M <= 16 streams the codes (the decode kernels widen them in registers).  Above that - or from 5 rows with
+  // BLR_Q_DIRECT=0 - the factors are expanded to two-byte values once per call ([kernel workspace][U][V]) and the
+  // two-byte kernels run; the size covers both.  Requests for the phase engine (BLR_ALGO_STREAM*) stream codes up to M = 16.
   size_t s = stream_blast_workspace(M <= 16 ? M : 16, in_f, out_f, b, r, bits);
   if (M <= 4) return s;
   size_t sub = M <= 16 ? s : 2 * align_up((size_t)b * M * r * 2, 256);
