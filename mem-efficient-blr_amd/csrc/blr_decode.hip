@@ -1245,7 +1245,10 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
   if (M >= mfma_min_m && a.wbits == 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
   static const int q_mfma_min_m = env_i("BLR_D2_Q_MFMA_MIN_M", 3);
-  if ((M > 4 || M >= q_mfma_min_m) && a.wbits != 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);   // below that, codes stay with the vector variant
+  if ((M > 4 || M >= q_mfma_min_m) && a.wbits != 16) {   // below that, codes stay with the vector variant
+    const int rc = decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
+    if (rc != 1 || M > 4) return rc;                     // a shape it declines at 3 or 4 rows is still the vector variant's
+  }
   if (M > 4) return d2_bail(__LINE__);
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int WBITS = a.wbits, EPL = 128 / WBITS;  // weights per 16-byte load

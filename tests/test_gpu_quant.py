@@ -44,7 +44,8 @@ def test_quantizer_half_inputs_and_ties():
     np.testing.assert_array_equal(c2.cpu().numpy(), r2)
 
 
-QSHAPES = [(2, 8, 8, 32, 1), (4, 16, 24, 64, 3), (16, 32, 40, 96, 16), (16, 256, 256, 512, 4), (4, 32, 40, 96, 40), (16, 72, 288, 288, 300)]
+QSHAPES = [(2, 8, 8, 32, 1), (4, 16, 24, 64, 3), (16, 32, 40, 96, 16), (16, 256, 256, 512, 4), (4, 32, 40, 96, 40), (16, 72, 288, 288, 300),
+           (4, 32, 24, 1088, 6), (2, 136, 264, 160, 11)]   # the last two: a rank beyond one slab (stage 2 split along k), ragged blocks
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
