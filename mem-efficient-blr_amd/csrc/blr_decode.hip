@@ -1183,6 +1183,138 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   if (w == 0) finish_epoch(p, epoch, G);
 }
 
+// ---- dense layer at 5..16 token rows ---------------------------------------------------------------
+// out = x W with W (K, N) row-major: nothing crosses workgroups before the products, so this is the slab stage of the
+// kernel above on its own.  A workgroup owns 128 columns and a slice of up to 1024 rows of W: the slice of x goes to LDS,
+// the slab streams through four batches of registers (32 loads per lane in flight, a consumed batch is refilled at
+// once), the products run on the matrix cores.  With one slice the result is stored as T; otherwise every slice
+// writes fp32 partial sums P[slice][m][n] with plain stores and dense_slab_reduce_kernel adds them in fixed order
+// in a second launch: no spinning, no limit on the grid.
+struct DenseSlabParams {
+  const void* x; int64_t ldx; const void* W; void* out; int64_t ldo; float* part;
+  int M, K, N, nch, ks, kc, x_vec;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void dense_slab_kernel(DenseSlabParams p) {
+  __shared__ __attribute__((aligned(16))) T a_s[16 * (DM_KMAX + 8)];
+  __shared__ __attribute__((aligned(16))) float red[4 * 4 * 64 * 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int cv = lane & 15, kg = lane >> 4, rs = wave * 4 + kg;
+  const int nc = blockIdx.x % p.nch, sl = blockIdx.x / p.nch;
+  const int k0 = sl * p.kc, kc = min(p.kc, p.K - k0);
+  const int n0 = nc * 128, n = n0 + cv * 8;
+  const bool col_ok = n < p.N;
+  const int M = p.M;
+  const __amdgpu_buffer_rsrc_t wb = wbuf(p.W, (uint32_t)((int64_t)p.K * p.N * 2));
+  const uint32_t woff = (uint32_t)((((int64_t)k0 + rs * 8) * p.N + (col_ok ? n : 0)) * 2);
+  const uint32_t wrow = (uint32_t)p.N * 2u;
+  const int nb = (kc + DM_ROWS - 1) / DM_ROWS;          // batches of 128 rows; rows past the end of W read as zero
+  const int kpad = nb * DM_ROWS, ald = kpad + 8;
+  u32x4 pf[DM_PF];
+#pragma unroll
+  for (int bq = 0; bq < DM_PF / 8; ++bq) {
+    const uint32_t vo = bq < nb ? woff : 0x80000000u;   // a batch past the slice: offset beyond the buffer, reads as zero
+#pragma unroll
+    for (int u = 0; u < 8; ++u) pf[bq * 8 + u] = ldw16(wb, vo, bq < nb ? (uint32_t)(bq * DM_ROWS + u) * wrow : 0u);
+  }
+  // the slice of x as T, zero beyond M rows and beyond the slice
+  const T* xp = reinterpret_cast<const T*>(p.x);
+  if (p.x_vec) {                                         // 16-byte pieces: every piece aligned and inside the row
+    const int pieces = kpad >> 3;
+    for (int idx = tid; idx < 16 * pieces; idx += 256) {
+      const int m = idx / pieces, ka = (idx - m * pieces) * 8;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (m < M && ka < kc) v = *reinterpret_cast<const u32x4*>(&xp[(int64_t)m * p.ldx + k0 + ka]);
+      *reinterpret_cast<u32x4*>(&a_s[m * ald + ka]) = v;
+    }
+  } else {
+    for (int idx = tid; idx < 16 * kpad; idx += 256) {
+      const int m = idx / kpad, ka = idx - m * kpad;
+      T v = TypeTraits<T>::from_f32(0.0f);
+      if (m < M && ka < kc) v = xp[(int64_t)m * p.ldx + k0 + ka];
+      a_s[m * ald + ka] = v;
+    }
+  }
+  __syncthreads();
+  f32x4 acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  // Straight-line code: the loads are unconditional (past the slice they cost nothing), only the products are skipped,
+  // so the compiler can count the loads in flight instead of waiting for all of them at every branch.
+#pragma unroll
+  for (int bt = 0; bt < DM_KMAX / DM_ROWS; ++bt) {
+    constexpr int NSLOT = DM_PF / 8;
+    const int bq = bt % NSLOT;
+    u32x4 cur[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) cur[u] = pf[bq * 8 + u];
+    if (bt + NSLOT < DM_KMAX / DM_ROWS) {                  // refill the registers just read with the batch four ahead
+      const int nxt = bt + NSLOT;
+      const uint32_t vo = nxt < nb ? woff : 0x80000000u;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) pf[bq * 8 + u] = ldw16(wb, vo, nxt < nb ? (uint32_t)(nxt * DM_ROWS + u) * wrow : 0u);
+    }
+    if (bt < nb) dm_batch<T>(cur, a_s, ald, cv, rs, bt * DM_ROWS, acc);
+  }
+  // sum of the four waves (they hold different rows of the slice), then thread (e, l) owns rows 4 (l / 16) .. + 3 of
+  // columns 8 (l % 16) + e and + 4 of that
+  f32x4 vh[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < 4; ++e) *reinterpret_cast<f32x4*>(&red[((wave * 4 + e) * 64 + lane) * 4]) = acc[h * 4 + e];
+    __syncthreads();
+    const int e = tid >> 6, l = tid & 63;
+    f32x4 v = *reinterpret_cast<const f32x4*>(&red[((0 * 4 + e) * 64 + l) * 4]);
+    v += *reinterpret_cast<const f32x4*>(&red[((1 * 4 + e) * 64 + l) * 4]);
+    v += *reinterpret_cast<const f32x4*>(&red[((2 * 4 + e) * 64 + l) * 4]);
+    v += *reinterpret_cast<const f32x4*>(&red[((3 * 4 + e) * 64 + l) * 4]);
+    vh[h] = v;
+  }
+  // through LDS once more so that a wave writes whole rows of the 128-column chunk
+  constexpr int OLD = 132;
+  __syncthreads();
+  {
+    const int e = tid >> 6, l = tid & 63, col = (l & 15) * 8 + e, m0 = (l >> 4) * 4;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[(m0 + i) * OLD + col + 4 * h] = vh[h][i];
+  }
+  __syncthreads();
+  {
+    const int c4 = (tid & 31) * 4, mr = tid >> 5;        // 4 columns of rows mr and mr + 8
+    const int gn = n0 + c4;
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int m = mr + 8 * hh;
+      if (m < M && gn < p.N) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(&red[m * OLD + c4]);
+        if (p.ks > 1) {
+          float* dst = &p.part[((int64_t)sl * M + m) * p.N + gn];
+          if (gn + 3 < p.N && (p.N & 3) == 0) *reinterpret_cast<f32x4*>(dst) = v;
+          else { for (int e = 0; e < 4; ++e) if (gn + e < p.N) dst[e] = v[e]; }
+        } else {
+          T* dst = &reinterpret_cast<T*>(p.out)[(int64_t)m * p.ldo + gn];
+          for (int e = 0; e < 4; ++e) if (gn + e < p.N) dst[e] = TypeTraits<T>::from_f32(v[e]);
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dense_slab_reduce_kernel(const float* __restrict__ P, T* __restrict__ out, int64_t ldo, int M, int N, int ks) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * N) return;
+  const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
+  float v = 0.0f;
+  for (int s = 0; s < ks; ++s) v += P[((int64_t)s * M + m) * N + n];
+  out[(int64_t)m * ldo + n] = TypeTraits<T>::from_f32(v);
+}
+
 // ---- host side -----------------------------------------------------------------------------------
 namespace {
 
@@ -1501,6 +1633,41 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
   void* args[] = {&p};
   hipError_t e = hipLaunchKernel(fn, dim3(grid), dim3(256), args, 0, st);
   if (e != hipSuccess) { set_error("decode2m: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  return BLR_OK;
+}
+
+// Dense layer at up to 16 rows through dense_slab_kernel.  part: room for max_slices * M * N floats.
+// Returns BLR_OK, a negative status, or 1 when the call is not for this kernel.
+int dense_slab_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int K, int N, int dtype,
+                      float* part, int max_slices, hipStream_t st) {
+  static const int enabled = env_i("BLR_DENSE_SLAB", 1), min_m = env_i("BLR_DENSE_SLAB_MIN_M", 5);
+  if (!enabled || M < min_m || M > 16) return 1;
+  if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
+  if (N % 8 || !aligned(W, 16) || (int64_t)K * N * 2 >= (1ll << 31)) return d2_bail(__LINE__);   // 16-byte pieces of a row, 32-bit buffer offsets
+  const int cus = device_cus() > 0 ? device_cus() : 256;
+  const int nch = (N + 127) / 128;
+  static const int per_cu = env_i("BLR_DENSE_SLAB_WGS_PER_CU", 2);
+  int ks = (per_cu * cus + nch - 1) / nch;               // enough slices to give every compute unit its workgroups
+  if (ks > max_slices) ks = max_slices;
+  if (ks > (K + DM_ROWS - 1) / DM_ROWS) ks = (K + DM_ROWS - 1) / DM_ROWS;
+  if (ks < 1) ks = 1;
+  int kc = ((K + ks - 1) / ks + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
+  if (kc > DM_KMAX) kc = DM_KMAX;
+  ks = (K + kc - 1) / kc;
+  if (ks > max_slices) return d2_bail(__LINE__);
+  DenseSlabParams p = {};
+  p.x = x; p.ldx = ldx; p.W = W; p.out = out; p.ldo = ldo; p.part = part;
+  p.M = M; p.K = K; p.N = N; p.nch = nch; p.ks = ks; p.kc = kc;
+  p.x_vec = aligned(x, 16) && ldx % 8 == 0 && K % 8 == 0;
+  if (dtype == BLR_F16) hipLaunchKernelGGL(dense_slab_kernel<f16>, dim3((unsigned)(nch * ks)), dim3(256), 0, st, p);
+  else hipLaunchKernelGGL(dense_slab_kernel<bf16>, dim3((unsigned)(nch * ks)), dim3(256), 0, st, p);
+  if (ks > 1) {
+    const unsigned blocks = (unsigned)(((int64_t)M * N + 255) / 256);
+    if (dtype == BLR_F16) hipLaunchKernelGGL(dense_slab_reduce_kernel<f16>, dim3(blocks), dim3(256), 0, st, part, (f16*)out, ldo, M, N, ks);
+    else hipLaunchKernelGGL(dense_slab_reduce_kernel<bf16>, dim3(blocks), dim3(256), 0, st, part, (bf16*)out, ldo, M, N, ks);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_error("dense_slab: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
 }
 

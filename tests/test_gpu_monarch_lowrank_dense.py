@@ -206,3 +206,21 @@ def test_low_rank_and_dense_llama7b(layer, M):
     d = D.triton_dense_fp16(dev(x, torch.float16), dev(W, torch.float16))
     rd = rounded(x[0, rows], torch.float16) @ rounded(W, torch.float16)
     assert_close(d[rows], rd, torch.float16, f"dense {layer} M{M}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [5, 7, 12, 16])
+@pytest.mark.parametrize("shape", [(1000, 200), (1004, 136), (2600, 264), (64, 8)])
+def test_dense_few_rows_ragged(shape, M, dtype):
+    """Dense at 5..16 rows: reductions that are no multiple of a batch, of a slice or of 8; column counts that end
+    inside a 128-column chunk; x as a row-strided view."""
+    from triton_funcs import dense_kernels as D
+    in_f, out_f = shape
+    rng = np.random.default_rng(100 + M)
+    x = rng.standard_normal((M, in_f))
+    W = rng.standard_normal((out_f, in_f)) / np.sqrt(in_f)
+    say(f"[case] dense few rows {dtype} M={M} {shape}")
+    xd = torch.zeros(M, in_f + 24, device="cuda", dtype=dtype)
+    xd[:, :in_f] = dev(x, dtype)
+    d = D.triton_dense_fp16(xd[:, :in_f], dev(W.T, dtype))
+    assert_close(d, O.dense_forward(rounded(x, dtype), rounded(W, dtype)).reshape(M, out_f), dtype, f"dense M={M} {shape}")
