@@ -13,7 +13,7 @@ bool decode2_applicable(const StreamBlastArgs& a);
 int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
                          unsigned* err_word, hipStream_t st);
 
-// Dense layer out = x W (W (K, N)) at 5..16 rows: slabs of W on the matrix cores, fp32 partial sums of the k-slices in `part`
+// Dense layer out = x W (W (K, N)) at up to 16 rows: slabs of W on the matrix cores, fp32 partial sums of the k-slices in `part`
 // (room for max_slices * M * N floats) added by a second launch.  Returns BLR_OK, a negative blr_status, or 1 when the
 // call is not for this kernel.
 int dense_slab_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int K, int N, int dtype,

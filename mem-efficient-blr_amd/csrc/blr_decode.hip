@@ -1183,7 +1183,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   if (w == 0) finish_epoch(p, epoch, G);
 }
 
-// ---- dense layer at 5..16 token rows ---------------------------------------------------------------
+// ---- dense layer at up to 16 token rows ---------------------------------------------------------------
 // out = x W with W (K, N) row-major: nothing crosses workgroups before the products, so this is the slab stage of the
 // kernel above on its own.  A workgroup owns 128 columns and a slice of up to 1024 rows of W: the slice of x goes to LDS,
 // the slab streams through four batches of registers (32 loads per lane in flight, a consumed batch is refilled at
@@ -1640,20 +1640,27 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
 // Returns BLR_OK, a negative status, or 1 when the call is not for this kernel.
 int dense_slab_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int K, int N, int dtype,
                       float* part, int max_slices, hipStream_t st) {
-  static const int enabled = env_i("BLR_DENSE_SLAB", 1), min_m = env_i("BLR_DENSE_SLAB_MIN_M", 5);
+  static const int enabled = env_i("BLR_DENSE_SLAB", 1), min_m = env_i("BLR_DENSE_SLAB_MIN_M", 1);
   if (!enabled || M < min_m || M > 16) return 1;
   if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
   if (N % 8 || !aligned(W, 16) || (int64_t)K * N * 2 >= (1ll << 31)) return d2_bail(__LINE__);   // 16-byte pieces of a row, 32-bit buffer offsets
   const int cus = device_cus() > 0 ? device_cus() : 256;
   const int nch = (N + 127) / 128;
-  static const int per_cu = env_i("BLR_DENSE_SLAB_WGS_PER_CU", 2);
-  int ks = (per_cu * cus + nch - 1) / nch;               // enough slices to give every compute unit its workgroups
-  if (ks > max_slices) ks = max_slices;
-  if (ks > (K + DM_ROWS - 1) / DM_ROWS) ks = (K + DM_ROWS - 1) / DM_ROWS;
-  if (ks < 1) ks = 1;
-  int kc = ((K + ks - 1) / ks + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
-  if (kc > DM_KMAX) kc = DM_KMAX;
-  ks = (K + kc - 1) / kc;
+  // Slices: one workgroup per compute unit if its slab then fits the four register batches (512 rows: the whole slab is
+  // requested at once and the partial sums stay few), otherwise two per compute unit.
+  static const int e_per_cu = env_i("BLR_DENSE_SLAB_WGS_PER_CU", 0);
+  int ks = 1, kc = K;
+  for (int per_cu = e_per_cu > 0 ? e_per_cu : 1; per_cu <= (e_per_cu > 0 ? e_per_cu : 2); ++per_cu) {
+    ks = (per_cu * cus + nch - 1) / nch;                 // enough slices to give every compute unit its workgroups
+    if (ks > max_slices) ks = max_slices;
+    if (ks > (K + DM_ROWS - 1) / DM_ROWS) ks = (K + DM_ROWS - 1) / DM_ROWS;
+    if (ks < 1) ks = 1;
+    kc = ((K + ks - 1) / ks + DM_ROWS - 1) / DM_ROWS * DM_ROWS;
+    const bool fits = kc <= DM_PF / 8 * DM_ROWS;
+    if (kc > DM_KMAX) kc = DM_KMAX;
+    ks = (K + kc - 1) / kc;
+    if (fits) break;
+  }
   if (ks > max_slices) return d2_bail(__LINE__);
   DenseSlabParams p = {};
   p.x = x; p.ldx = ldx; p.W = W; p.out = out; p.ldo = ldo; p.part = part;

@@ -1287,7 +1287,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
   p.M = a.M;
   if (a.op == 0) {                             // dense: out = x W, W (in, out)
     WsLayout w = ws_carve(a.ws, 0);
-    if (!a.split) {                            // 5..16 rows: the slab kernel (the partial-sum area holds up to KSPLIT_MAX slices, or K / 8)
+    if (!a.split) {                            // the slab kernel (the partial-sum area holds up to KSPLIT_MAX slices, or K / 8)
       const int max_slices = (a.in_f + 7) / 8 < KSPLIT_MAX ? (a.in_f + 7) / 8 : KSPLIT_MAX;
       int rc = dense_slab_launch(a.x, a.ldx, a.W1, a.out, a.ldo, a.M, a.in_f, a.out_f, a.dtype, w.part, max_slices, st);
       if (rc != 1) return rc;
