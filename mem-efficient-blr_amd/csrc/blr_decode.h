@@ -19,4 +19,9 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
 int dense_slab_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int K, int N, int dtype,
                       float* part, int max_slices, hipStream_t st);
 
+// The same kernel for a batch of products C[bt] = A[bt] B[bt] with B (K, N) row-major (row stride ldb, batch strides in elements).
+// Without a partial-sum area (part null) the reduction is not cut and K is limited to one slab (1024 rows).
+int slab_gemm_launch(const void* A, int64_t lda, int64_t sA, const void* B, int64_t ldb, int64_t sB, void* C, int64_t ldc, int64_t sC,
+                     int M, int N, int K, int batch, int dtype, float* part, int max_slices, hipStream_t st);
+
 }  // namespace blr

@@ -1192,7 +1192,8 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
 // in a second launch: no spinning, no limit on the grid.
 struct DenseSlabParams {
   const void* x; int64_t ldx; const void* W; void* out; int64_t ldo; float* part;
-  int M, K, N, nch, ks, kc, x_vec;
+  int64_t sx, sw, so, ldw;                 // batches: element strides of x, W and out; row stride of W
+  int M, K, N, nch, ks, kc, x_vec, batch;
 };
 
 template <typename T>
@@ -1201,14 +1202,15 @@ __global__ __launch_bounds__(256, 2) void dense_slab_kernel(DenseSlabParams p) {
   __shared__ __attribute__((aligned(16))) float red[4 * 4 * 64 * 4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cv = lane & 15, kg = lane >> 4, rs = wave * 4 + kg;
-  const int nc = blockIdx.x % p.nch, sl = blockIdx.x / p.nch;
+  const int nc = blockIdx.x % p.nch, tb = blockIdx.x / p.nch;
+  const int bt = tb % p.batch, sl = tb / p.batch;
   const int k0 = sl * p.kc, kc = min(p.kc, p.K - k0);
   const int n0 = nc * 128, n = n0 + cv * 8;
   const bool col_ok = n < p.N;
   const int M = p.M;
-  const __amdgpu_buffer_rsrc_t wb = wbuf(p.W, (uint32_t)((int64_t)p.K * p.N * 2));
-  const uint32_t woff = (uint32_t)((((int64_t)k0 + rs * 8) * p.N + (col_ok ? n : 0)) * 2);
-  const uint32_t wrow = (uint32_t)p.N * 2u;
+  const __amdgpu_buffer_rsrc_t wb = wbuf(reinterpret_cast<const T*>(p.W) + (int64_t)bt * p.sw, (uint32_t)((int64_t)p.K * p.ldw * 2));
+  const uint32_t woff = (uint32_t)((((int64_t)k0 + rs * 8) * p.ldw + (col_ok ? n : 0)) * 2);
+  const uint32_t wrow = (uint32_t)p.ldw * 2u;
   const int nb = (kc + DM_ROWS - 1) / DM_ROWS;          // batches of 128 rows; rows past the end of W read as zero
   const int kpad = nb * DM_ROWS, ald = kpad + 8;
   u32x4 pf[DM_PF];
@@ -1219,7 +1221,7 @@ __global__ __launch_bounds__(256, 2) void dense_slab_kernel(DenseSlabParams p) {
     for (int u = 0; u < 8; ++u) pf[bq * 8 + u] = ldw16(wb, vo, bq < nb ? (uint32_t)(bq * DM_ROWS + u) * wrow : 0u);
   }
   // the slice of x as T, zero beyond M rows and beyond the slice
-  const T* xp = reinterpret_cast<const T*>(p.x);
+  const T* xp = reinterpret_cast<const T*>(p.x) + (int64_t)bt * p.sx;
   if (p.x_vec) {                                         // 16-byte pieces: every piece aligned and inside the row
     const int pieces = kpad >> 3;
     for (int idx = tid; idx < 16 * pieces; idx += 256) {
@@ -1293,11 +1295,11 @@ __global__ __launch_bounds__(256, 2) void dense_slab_kernel(DenseSlabParams p) {
       if (m < M && gn < p.N) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(&red[m * OLD + c4]);
         if (p.ks > 1) {
-          float* dst = &p.part[((int64_t)sl * M + m) * p.N + gn];
+          float* dst = &p.part[(((int64_t)sl * p.batch + bt) * M + m) * p.N + gn];
           if (gn + 3 < p.N && (p.N & 3) == 0) *reinterpret_cast<f32x4*>(dst) = v;
           else { for (int e = 0; e < 4; ++e) if (gn + e < p.N) dst[e] = v[e]; }
         } else {
-          T* dst = &reinterpret_cast<T*>(p.out)[(int64_t)m * p.ldo + gn];
+          T* dst = &reinterpret_cast<T*>(p.out)[(int64_t)bt * p.so + (int64_t)m * p.ldo + gn];
           for (int e = 0; e < 4; ++e) if (gn + e < p.N) dst[e] = TypeTraits<T>::from_f32(v[e]);
         }
       }
@@ -1306,13 +1308,16 @@ __global__ __launch_bounds__(256, 2) void dense_slab_kernel(DenseSlabParams p) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void dense_slab_reduce_kernel(const float* __restrict__ P, T* __restrict__ out, int64_t ldo, int M, int N, int ks) {
+__global__ __launch_bounds__(256) void dense_slab_reduce_kernel(const float* __restrict__ P, T* __restrict__ out, int64_t ldo, int64_t so,
+                                                                 int M, int N, int ks, int batch) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (int64_t)M * N) return;
-  const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
+  if (idx >= (int64_t)batch * M * N) return;
+  const int n = (int)(idx % N);
+  const int64_t t = idx / N;
+  const int m = (int)(t % M), bt = (int)(t / M);
   float v = 0.0f;
-  for (int s = 0; s < ks; ++s) v += P[((int64_t)s * M + m) * N + n];
-  out[(int64_t)m * ldo + n] = TypeTraits<T>::from_f32(v);
+  for (int s = 0; s < ks; ++s) v += P[(((int64_t)s * batch + bt) * M + m) * N + n];
+  out[(int64_t)bt * so + (int64_t)m * ldo + n] = TypeTraits<T>::from_f32(v);
 }
 
 // ---- host side -----------------------------------------------------------------------------------
@@ -1636,22 +1641,25 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
   return BLR_OK;
 }
 
-// Dense layer at up to 16 rows through dense_slab_kernel.  part: room for max_slices * M * N floats.
-// Returns BLR_OK, a negative status, or 1 when the call is not for this kernel.
-int dense_slab_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int K, int N, int dtype,
-                      float* part, int max_slices, hipStream_t st) {
+// Batched C[bt] = A[bt] B[bt] at up to 16 rows through dense_slab_kernel; B (K, N) row-major with row stride ldb.
+// part: room for max_slices * batch * M * N floats (may be null with max_slices <= 1: the reduction is then not cut, which
+// limits K to one slab).  Returns BLR_OK, a negative status, or 1 when the call is not for this kernel.
+int slab_gemm_launch(const void* A, int64_t lda, int64_t sA, const void* B, int64_t ldb, int64_t sB, void* C, int64_t ldc, int64_t sC,
+                     int M, int N, int K, int batch, int dtype, float* part, int max_slices, hipStream_t st) {
   static const int enabled = env_i("BLR_DENSE_SLAB", 1), min_m = env_i("BLR_DENSE_SLAB_MIN_M", 1);
   if (!enabled || M < min_m || M > 16) return 1;
   if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
-  if (N % 8 || !aligned(W, 16) || (int64_t)K * N * 2 >= (1ll << 31)) return d2_bail(__LINE__);   // 16-byte pieces of a row, 32-bit buffer offsets
+  if (N % 8 || ldb % 8 || sB % 8 || !aligned(B, 16) || (int64_t)K * ldb * 2 >= (1ll << 31)) return d2_bail(__LINE__);   // 16-byte pieces of a row, 32-bit buffer offsets
+  if (!part || max_slices < 1) max_slices = 1;
   const int cus = device_cus() > 0 ? device_cus() : 256;
   const int nch = (N + 127) / 128;
+  const int64_t base = (int64_t)nch * batch;
   // Slices: one workgroup per compute unit if its slab then fits the four register batches (512 rows: the whole slab is
   // requested at once and the partial sums stay few), otherwise two per compute unit.
   static const int e_per_cu = env_i("BLR_DENSE_SLAB_WGS_PER_CU", 0);
   int ks = 1, kc = K;
   for (int per_cu = e_per_cu > 0 ? e_per_cu : 1; per_cu <= (e_per_cu > 0 ? e_per_cu : 2); ++per_cu) {
-    ks = (per_cu * cus + nch - 1) / nch;                 // enough slices to give every compute unit its workgroups
+    ks = (int)(((int64_t)per_cu * cus + base - 1) / base);   // enough slices to give every compute unit its workgroups
     if (ks > max_slices) ks = max_slices;
     if (ks > (K + DM_ROWS - 1) / DM_ROWS) ks = (K + DM_ROWS - 1) / DM_ROWS;
     if (ks < 1) ks = 1;
@@ -1662,20 +1670,28 @@ int dense_slab_launch(const void* x, int64_t ldx, const void* W, void* out, int6
     if (fits) break;
   }
   if (ks > max_slices) return d2_bail(__LINE__);
+  if (base * ks >= (1ll << 31)) return d2_bail(__LINE__);
   DenseSlabParams p = {};
-  p.x = x; p.ldx = ldx; p.W = W; p.out = out; p.ldo = ldo; p.part = part;
-  p.M = M; p.K = K; p.N = N; p.nch = nch; p.ks = ks; p.kc = kc;
-  p.x_vec = aligned(x, 16) && ldx % 8 == 0 && K % 8 == 0;
-  if (dtype == BLR_F16) hipLaunchKernelGGL(dense_slab_kernel<f16>, dim3((unsigned)(nch * ks)), dim3(256), 0, st, p);
-  else hipLaunchKernelGGL(dense_slab_kernel<bf16>, dim3((unsigned)(nch * ks)), dim3(256), 0, st, p);
+  p.x = A; p.ldx = lda; p.W = B; p.out = C; p.ldo = ldc; p.part = part;
+  p.sx = sA; p.sw = sB; p.so = sC; p.ldw = ldb;
+  p.M = M; p.K = K; p.N = N; p.nch = nch; p.ks = ks; p.kc = kc; p.batch = batch;
+  p.x_vec = aligned(A, 16) && lda % 8 == 0 && sA % 8 == 0 && K % 8 == 0;
+  const unsigned grid = (unsigned)(base * ks);
+  if (dtype == BLR_F16) hipLaunchKernelGGL(dense_slab_kernel<f16>, dim3(grid), dim3(256), 0, st, p);
+  else hipLaunchKernelGGL(dense_slab_kernel<bf16>, dim3(grid), dim3(256), 0, st, p);
   if (ks > 1) {
-    const unsigned blocks = (unsigned)(((int64_t)M * N + 255) / 256);
-    if (dtype == BLR_F16) hipLaunchKernelGGL(dense_slab_reduce_kernel<f16>, dim3(blocks), dim3(256), 0, st, part, (f16*)out, ldo, M, N, ks);
-    else hipLaunchKernelGGL(dense_slab_reduce_kernel<bf16>, dim3(blocks), dim3(256), 0, st, part, (bf16*)out, ldo, M, N, ks);
+    const unsigned blocks = (unsigned)(((int64_t)batch * M * N + 255) / 256);
+    if (dtype == BLR_F16) hipLaunchKernelGGL(dense_slab_reduce_kernel<f16>, dim3(blocks), dim3(256), 0, st, part, (f16*)C, ldc, sC, M, N, ks, batch);
+    else hipLaunchKernelGGL(dense_slab_reduce_kernel<bf16>, dim3(blocks), dim3(256), 0, st, part, (bf16*)C, ldc, sC, M, N, ks, batch);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_error("dense_slab: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
+}
+
+int dense_slab_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int K, int N, int dtype,
+                      float* part, int max_slices, hipStream_t st) {
+  return slab_gemm_launch(x, ldx, 0, W, N, 0, out, ldo, 0, M, N, K, 1, dtype, part, max_slices, st);
 }
 
 }  // namespace blr

@@ -11,6 +11,7 @@
 #include <mutex>
 #include <set>
 #include "blr_common.h"
+#include "blr_decode.h"
 
 namespace blr {
 
@@ -928,6 +929,12 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
 
 int gemm_launch(const GemmArgs& g, int dtype, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0 || g.K <= 0 || g.batch <= 0) { set_error("gemm: empty problem"); return BLR_ERR_BAD_ARG; }
+  // A handful of rows is a weight-streaming problem, not a tiling problem: plain products with (k, n)-ordered weights go to
+  // the slab kernel of the decode path (it declines what it cannot take, e.g. a reduction deeper than one slab here).
+  if (g.M <= 16 && g.b_kn && g.cn == 1 && g.epi == EPI_PLAIN && !g.sat8 && !g.bias && g.act == 0 && (dtype == BLR_F16 || dtype == BLR_BF16)) {
+    int rc = slab_gemm_launch(g.A, g.lda, g.sA, g.B, g.ldb, g.sB, g.C, g.ldc, g.sC, g.M, g.N, g.K, g.batch, dtype, nullptr, 1, st);
+    if (rc != 1) return rc;
+  }
   if (dtype == BLR_F16) return pick_mfma<f16>(g, st);
   if (dtype == BLR_BF16) return pick_mfma<bf16>(g, st);
   if (dtype == BLR_F32) {
