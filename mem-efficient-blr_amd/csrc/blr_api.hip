@@ -296,6 +296,18 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
   int a = resolve_algo(algo, M, dtype, z_out || y_out);
   if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
     if (dtype == BLR_F32 || M > 16 || z_out || y_out) { set_error("blast: streaming algorithm needs f16/bf16, M <= 16, no intermediates"); return BLR_ERR_UNSUPPORTED; }
+    // Optional (off by default, BLR_BLAST_SLAB_MIN_M): three launches - slab product, mix, slab product - instead of the single
+    // launch whose workgroups hand the intermediates to each other.  Measured at 16 rows: 39.1 against 33.7 us on gate_up,
+    // 30.8 against 19.3 on qkvo - the launches and the small mix cost more than the hand-overs.  Y and Z go behind the
+    // fixed-place block of the streaming workspace, so the same workspace keeps serving the single-launch kernels.
+    static const int slab_min_m = getenv("BLR_BLAST_SLAB_MIN_M") ? atoi(getenv("BLR_BLAST_SLAB_MIN_M")) : 99;
+    if (algo == BLR_ALGO_AUTO && M >= slab_min_m && u_layout == BLR_U_RQ && P <= 1024 && r <= 1024 && r % 8 == 0 && Q % 8 == 0 &&
+        aligned(U, 16) && aligned(V, 16)) {
+      const size_t off = stream_ws_prefix_bytes(), yz = 2 * align_up((size_t)b * M * r * elt_size(dtype), 256);
+      if (ws && ws_bytes >= off + yz)
+        return blast_tiled(x, ldx, U, V, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, u_layout, s_layout, 0,
+                           reinterpret_cast<char*>(ws) + off, ws_bytes - off, st);
+    }
     StreamBlastArgs s = {};
     s.x = x; s.ldx = ldx; s.U = U; s.V = V; s.S = S; s.out = out; s.ldo = ldo;
     s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;

@@ -138,6 +138,7 @@ struct StreamBlastArgs {
   int split;                                    // 1: separate launches per phase
 };
 size_t stream_blast_workspace(int M, int in_f, int out_f, int b, int r, int wbits);
+size_t stream_ws_prefix_bytes();                // the fixed-place block at the start of a streaming workspace; per-call scratch follows
 int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st);
 
 struct StreamGenericArgs {                      // dense / low-rank / monarch at M <= 16

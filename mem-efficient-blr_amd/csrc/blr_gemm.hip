@@ -1141,8 +1141,43 @@ __global__ __launch_bounds__(256) void blast_mix_h2_kernel(const f16* __restrict
   }
 }
 
+// The mix for a handful of rows (M <= 16, b <= 16): workgroup = 16 ranks x all output blocks, thread = (block i, rank).
+// The Y values of the chunk (b x M x 16) are staged in LDS once; every thread keeps its b values of S in registers.
+template <typename T>
+__global__ __launch_bounds__(256) void blast_mix_small_kernel(const T* __restrict__ Y, const T* __restrict__ S, T* __restrict__ Z,
+                                                              int M, int b, int R, int64_t s_si, int64_t s_sj, int64_t s_sr) {
+  __shared__ float ys[16 * 16 * 16];                  // [j][m][rank in chunk]
+  const int tid = threadIdx.x, g = tid >> 4, rr = tid & 15;
+  const int r0 = blockIdx.x * 16, r = r0 + rr;
+  float sv[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    sv[j] = (g < b && j < b && r < R) ? TypeTraits<T>::to_f32(S[(int64_t)g * s_si + (int64_t)j * s_sj + (int64_t)r * s_sr]) : 0.0f;
+  const int total = b * M * 16;
+  for (int idx = tid; idx < total; idx += 256) {
+    const int c = idx & 15, jm = idx >> 4;            // jm = j * M + m
+    ys[idx] = (r0 + c < R) ? TypeTraits<T>::to_f32(Y[(int64_t)jm * R + r0 + c]) : 0.0f;
+  }
+  __syncthreads();
+  if (g < b && r < R) {
+    for (int m = 0; m < M; ++m) {
+      float z = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) z = fmaf(sv[j], j < b ? ys[(j * M + m) * 16 + rr] : 0.0f, z);
+      Z[((int64_t)g * M + m) * R + r] = TypeTraits<T>::from_f32(z);
+    }
+  }
+}
+
 int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
                      int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st, int sat8) {
+  if (M <= 16 && b <= 16 && !sat8 && (dtype == BLR_F16 || dtype == BLR_BF16)) {
+    const dim3 grid((unsigned)cdiv(R, 16));
+    if (dtype == BLR_F16) hipLaunchKernelGGL(blast_mix_small_kernel<f16>, grid, dim3(256), 0, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr);
+    else hipLaunchKernelGGL(blast_mix_small_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)Y, (const bf16*)S, (bf16*)Z, M, b, R, s_si, s_sj, s_sr);
+    BLR_CHECK_LAUNCH("blast_mix_small");
+    return BLR_OK;
+  }
   int r_chunks = (int)cdiv(R, 64);
   if (dtype != BLR_F32 && b <= 16 && R % 8 == 0 && aligned(Y, 16) && aligned(Z, 16)) {
     size_t lds = (size_t)b * b * 64 * 2;

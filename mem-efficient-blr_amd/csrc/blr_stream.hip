@@ -1198,6 +1198,10 @@ size_t part_bound(int M, int batch, int K, int N) {
 
 }  // namespace
 
+// Bytes of the fixed-place block at the start of every streaming workspace (control words, counters, Z buffers, tagged pairs);
+// what follows it is per-call scratch.
+size_t stream_ws_prefix_bytes() { return ws_total(0, 0); }
+
 size_t stream_blast_workspace(int M, int in_f, int out_f, int b, int r, int wbits) {
   (void)wbits;
   size_t buf = (size_t)b * M * r;
