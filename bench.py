@@ -49,7 +49,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-table", action="store_true", help="skip the per-layer table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--pmc", choices=["dominant", "calib", "prefill"], default=None,
+    ap.add_argument("--pmc", choices=["dominant", "calib", "prefill", "decode16"], default=None,
                     help="profiling helper: launch only the dominant decode kernel (dominant), only copy/probe kernels of "
                          "known size (calib), or only the BLAST gate_up prefill kernels at M=2048 (prefill), eagerly, and "
                          "print nothing but a note")
@@ -200,6 +200,23 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"pmc": "prefill", "launches": 24, "flops": blast_bytes_flops(2048, 4096, 1024, 22016)[1],
                           "dense_launches": 8, "dense_flops": 2.0 * 2048 * 4096 * 22016}))
+        return
+    if args.pmc == "decode16":
+        # the other decode kernels at full shape, eager launches over rotating weight copies: dense gate_up at M = 1 and 16
+        # (slab kernel + sum of the k-slices), BLAST gate_up at M = 16 (matrix-core decode kernel), int8 BLAST gate_up at M = 16
+        st = torch.cuda.current_stream().cuda_stream
+        i_f, o_f, r = LAYERS["gate_up"]
+        for mk in (lambda: mk_dense(1, i_f, o_f), lambda: mk_dense(16, i_f, o_f),
+                   lambda: mk_blast(16, i_f, o_f, r, L.U_RQ, L.S_JIR), lambda: mk_blast_q(16, i_f, o_f, r, 8)):
+            built = [mk() for _ in range(4)]
+            for i in range(12):
+                built[i % 4][0](st)
+            torch.cuda.synchronize()
+            del built
+            torch.cuda.empty_cache()
+        print(json.dumps({"pmc": "decode16", "launches_each": 12, "dense_bytes_m1": 2 * (i_f + i_f * o_f + o_f),
+                          "dense_bytes_m16": 2 * (16 * i_f + i_f * o_f + 16 * o_f),
+                          "blast_bytes_m16": blast_bytes_flops(16, i_f, r, o_f)[0]}))
         return
     if args.pmc == "dominant":
         gu = [mk_blast(1, *LAYERS["gate_up"][:2], LAYERS["gate_up"][2], L.U_RQ, L.S_JIR) for _ in range(12)]
