@@ -1315,8 +1315,17 @@ __global__ __launch_bounds__(256) void dense_slab_reduce_kernel(const float* __r
   const int n = (int)(idx % N);
   const int64_t t = idx / N;
   const int m = (int)(t % M), bt = (int)(t / M);
+  // four slices are asked for together (one trip to memory, not one per slice) and added in slice order
+  const int64_t sstride = (int64_t)batch * M * N;
+  const float* src = P + ((int64_t)bt * M + m) * N + n;
   float v = 0.0f;
-  for (int s = 0; s < ks; ++s) v += P[(((int64_t)s * batch + bt) * M + m) * N + n];
+  int s = 0;
+  for (; s + 4 <= ks; s += 4) {
+    const float a0 = src[(int64_t)s * sstride], a1 = src[(int64_t)(s + 1) * sstride];
+    const float a2 = src[(int64_t)(s + 2) * sstride], a3 = src[(int64_t)(s + 3) * sstride];
+    v += a0; v += a1; v += a2; v += a3;
+  }
+  for (; s < ks; ++s) v += src[(int64_t)s * sstride];
   out[(int64_t)bt * so + (int64_t)m * ldo + n] = TypeTraits<T>::from_f32(v);
 }
 
