@@ -1308,12 +1308,13 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
   }
   if (a.op == 1) {                             // low rank: z = x A (in, r); out = z B (r, out)
     WsLayout w = ws_carve(a.ws, (size_t)a.M * a.r);
-    static const int slab_min_m = env_int("BLR_LOWRANK_SLAB_MIN_M", 99);
+    static const int slab_min_m = env_int("BLR_LOWRANK_SLAB_MIN_M", 5);
     if (!a.split && a.M >= slab_min_m && a.r % 8 == 0 && a.out_f % 8 == 0) {
-      // Optional (off by default): two launches of the slab kernel, each followed by the sum of its k-slices: z = x A goes
-      // to the first staging buffer as T, then out = z B.  Four launches cost 24-27 us whatever M is; measured against the
-      // single launch below at 16 rows this wins on 4096 -> 4096 (27.6 against 31.2 us) and 11008 -> 4096 (29.6 against 38.6)
-      // and loses on 4096 -> 22016 (34.6 against 30.5).  The partial-sum area is sized for either product.
+      // From a handful of rows up, two launches of the slab kernel, each followed by the sum of its k-slices: z = x A goes
+      // to the first staging buffer as T, then out = z B.  Four launches, 19-29 us whatever M is; the single launch below
+      // hands up to 16 rows of intermediates between workgroups and needs 25-39 us at 5..16 rows (measured on the three
+      // Llama-7B shapes: ahead everywhere except 4096 -> 22016 at 5 and 8 rows, where it is 1.5 us behind).  The
+      // partial-sum area is sized for either product.
       const int s1 = (a.in_f + 7) / 8 < KSPLIT_MAX ? (a.in_f + 7) / 8 : KSPLIT_MAX;
       const int s2 = (a.r + 7) / 8 < KSPLIT_MAX ? (a.r + 7) / 8 : KSPLIT_MAX;
       int rc = slab_gemm_launch(a.x, a.ldx, 0, a.W1, a.r, 0, w.buf0, a.r, 0, a.M, a.r, a.in_f, 1, a.dtype, w.part, s1, st);
