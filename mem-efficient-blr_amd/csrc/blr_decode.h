@@ -13,6 +13,11 @@ bool decode2_applicable(const StreamBlastArgs& a);
 int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
                          unsigned* err_word, hipStream_t st);
 
+// The same call on the one-workgroup-per-compute-unit kernel (blr_decode3.hip; up to four token rows).  Returns BLR_OK, a
+// negative blr_status, or 1 when the call is not for it (decode2_blast_launch then serves it itself).
+int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
+                         unsigned* err_word, hipStream_t st);
+
 // Dense layer out = x W (W (K, N)) at up to 16 rows: slabs of W on the matrix cores, fp32 partial sums of the k-slices in `part`
 // (room for max_slices * M * N floats) added by a second launch.  Returns BLR_OK, a negative blr_status, or 1 when the
 // call is not for this kernel.

@@ -22,19 +22,22 @@
 #include <mutex>
 #include "blr_common.h"
 #include "blr_decode.h"
+#include "blr_decode_dev.h"
 
 namespace blr {
 
 namespace {
 // 16-byte loads of the U slab held in registers per lane (fewer when the accumulators need the room)
 constexpr int d2_pf(int MT, int WB = 16) { return MT * (128 / WB) >= 64 ? 16 : (MT <= 1 ? 32 : (MT <= 2 ? 24 : 16)); }
+#ifndef BLR_D2_FIRST
+#define BLR_D2_FIRST 8
+#endif
+constexpr int D2_FIRST = BLR_D2_FIRST;   // loads of the U slab that go out right behind the V loads of stage 1
 constexpr int D2_UNR = 8;             // loads in flight per lane while streaming the rest of a slab
 constexpr int d2_unr1(int) { return 8; }   // loads in flight per lane in stage 1
 constexpr int d2_ks1_max(int MT) { return MT <= 2 ? 8 : 4; } // most k-slices of stage 1 (the mix fetches them all at once)
-constexpr int D2_SHARDS = 16;         // check-in counters, 256 bytes apart
 constexpr int D2_AS = 4096;           // fp32 activations staged in LDS (MT * k-chunk <= this)
 constexpr int D2_NC_MAX = 512;
-constexpr unsigned D2_SPIN_LIMIT = 4000000u;
 }  // namespace
 
 #ifdef BLR_TRACE
@@ -56,45 +59,12 @@ struct Decode2Params {
   int64_t s_si, s_sj, s_sr;
   int lpr1_log2, nch1, ks1, kc1, items1;
   int lpr2_log2, nch2, ks2, kc2, items2, pfn, kpad2;
-  int itemsM, rch_log2, pf_depth, x_vec, sparse_poll;
+  int itemsM, rch_log2, pf_depth, pf_first, x_vec, sparse_poll, udelay;
   unsigned long long* ypart;           // [ks1][b][M][R] tagged
   unsigned long long* zt;              // [b][M][R] tagged
   unsigned long long* opart;           // [ks2 - 1][b][M][Q] tagged
   unsigned* epoch_word; unsigned* arrive_word; unsigned* err_word;
 };
-
-__device__ __forceinline__ unsigned long long ld_tag(const unsigned long long* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_tag(unsigned long long* p, float v, unsigned epoch) {
-  __hip_atomic_store(p, ((unsigned long long)epoch << 32) | (unsigned long long)__float_as_uint(v),
-                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// 16 bytes of weights -> fp32: 8 two-byte elements, 16 int8 codes or 32 int4 codes (low nibble first).
-template <typename T, int WB>
-__device__ __forceinline__ void cvtw(const u32x4& r, float (&w)[128 / WB]) {
-  if constexpr (WB == 16) {
-    typename TypeTraits<T>::vec8 v = __builtin_bit_cast(typename TypeTraits<T>::vec8, r);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) w[e] = TypeTraits<T>::to_f32(v[e]);
-  } else if constexpr (WB == 8) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) w[e] = (float)(int8_t)((r[e >> 2] >> ((e & 3) * 8)) & 0xFF);
-  } else {
-#pragma unroll
-    for (int e = 0; e < 32; ++e) w[e] = (float)(((int32_t)(r[e >> 3] << (28 - 4 * (e & 7)))) >> 28);
-  }
-}
-// 16-byte streaming load through a buffer descriptor that spans the whole factor: the per-lane
-// byte offset sits in one register, the per-load row offset is uniform (scalar), and a row past
-// the end of the factor reads as zero instead of faulting - no clamping, no 64-bit addresses.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t wbuf(const void* W, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(W), 0, bytes, 0x00020000);
-}
-__device__ __forceinline__ u32x4 ldw16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
-  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 2));   // nt
-}
 
 // Sum of the row slots of a wave, then of the four waves; thread `col` < NC ends up with the
 // total of column `col` for each of the MT rows (returned through `tot`, valid for tid < NC).
@@ -129,29 +99,6 @@ __device__ __forceinline__ void wg_reduce(float (&acc)[MT][EPL], int lpr, int cv
   }
 }
 
-// Workgroup 0, at its end: wait until every workgroup of the launch has checked in (each does so
-// once it holds its copy of the epoch), then clear the counters and publish the epoch of this call,
-// from which the next call derives its own.
-__device__ __forceinline__ void finish_epoch(const Decode2Params& p, unsigned epoch, int G) {
-  if (threadIdx.x < 64) {
-    const int lane = threadIdx.x;
-    unsigned spins = 0;
-    while (true) {
-      unsigned v = (lane < D2_SHARDS) ? __hip_atomic_load(&p.arrive_word[lane * 64], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-#pragma unroll
-      for (int o = 1; o < D2_SHARDS; o <<= 1) v += __shfl_xor(v, o, 64);
-      if (__shfl(v, 0, 64) == (unsigned)G) break;
-      if (++spins > D2_SPIN_LIMIT) {
-        if (lane == 0) __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(1);
-    }
-    if (lane < D2_SHARDS) __hip_atomic_store(&p.arrive_word[lane * 64], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (lane == 0) __hip_atomic_store(p.epoch_word, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-}
-
 template <typename T, int MT, int WB>
 __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   constexpr int EPL = 128 / WB;                      // weights per 16-byte load
@@ -164,10 +111,13 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   const int tid = threadIdx.x;
   const int w = blockIdx.x, G = gridDim.x;
   const int M = p.M;
+  const unsigned long long t_begin = wall_clock64();
 
   TR2(0);
   // ---- epoch of this call ------------------------------------------------------------------
-  unsigned epoch = __hip_atomic_load(p.epoch_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  // (a plain, cached load: the word was last written before this kernel began, and hundreds of workgroups asking one
+  // address for a device-scope copy would queue up at a single memory channel - with every later load of theirs behind it)
+  unsigned epoch = *reinterpret_cast<const volatile unsigned*>(p.epoch_word) + 1u;
   if (epoch == 0u) epoch = 1u;
 
   // ---- stage-2 slab of this workgroup --------------------------------------------------------
@@ -197,23 +147,26 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   };
 
   u32x4 pf[D2_PF];                                   // only slots below pfn are ever read after the prefetch
-  auto issue_prefetch = [&]() {
+  auto issue_prefetch = [&](int lo, int hi) {        // loads lo .. hi - 1 of the slab (hi is cut at pfn)
 #pragma unroll
     for (int u = 0; u < D2_PF; ++u) {
-      if (u < p.pfn) {
+      if (u >= lo && u < hi && u < p.pfn) {
         // pacing: at most pf_depth of this lane's loads in flight, so that the queues of the memory
         // system stay short enough for the small hand-over accesses of other workgroups to get through
-        if (u >= 2 && p.pf_depth == 2) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-        else if (u >= 3 && p.pf_depth == 3) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-        else if (u >= 4 && p.pf_depth == 4) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-        else if (u >= 6 && p.pf_depth == 6) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-        else if (u >= 8 && p.pf_depth == 8) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
-        else if (u >= 12 && p.pf_depth == 12) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
-        else if (u >= 16 && p.pf_depth == 16) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
+        if (u >= D2_FIRST) {
+          if (u >= 2 && p.pf_depth == 2) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+          else if (u >= 3 && p.pf_depth == 3) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+          else if (u >= 4 && p.pf_depth == 4) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+          else if (u >= 6 && p.pf_depth == 6) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+          else if (u >= 8 && p.pf_depth == 8) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+          else if (u >= 12 && p.pf_depth == 12) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
+          else if (u >= 16 && p.pf_depth == 16) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
+        }
         pf[u] = ldw16(ubuf, uoff, u_soff(u));
       }
     }
   };
+  int pf_lo = 0;                                       // loads of the slab already asked for
 
   // Mix role (the first workgroups): its S values depend on nothing, so they are asked for first.
   // S(i = g, j = u, r) for this thread's (g, r); indices are clamped so that every load is legal.
@@ -272,6 +225,15 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     u32x4 raw[D2_UNR1];
 #pragma unroll
     for (int u = 0; u < D2_UNR1; ++u) raw[u] = ldw16(vbuf, voff, (uint32_t)u * vstep);
+    // The first loads of this workgroup's slab of U go out right behind: what heads the dependency chain is asked
+    // for first by every workgroup and comes back first (loads return in order), and the U stream is under way
+    // while stage 1 is being computed and handed over.
+    // (Straight-line, unconditional loads: a slot this workgroup does not have gets an offset beyond the buffer, which
+    // reads as zero without touching memory - so the compiler knows how many loads follow the V loads and waits
+    // for exactly those.)
+#pragma unroll
+    for (int u = 0; u < D2_FIRST; ++u) pf[u] = ldw16(ubuf, (has2 && u < p.pfn) ? uoff : 0x80000000u, u_soff(u));
+    pf_lo = D2_FIRST;
 #pragma unroll
     for (int q = 0; q < XR; ++q) {
       const int idx = tid + q * 256;
@@ -396,14 +358,17 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     TR2(9);
   }
   if (!has2) {
-    if (w == 0) finish_epoch(p, epoch, G);
+    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
     return;
   }
 
   // The slab of U: asked for only now, after this workgroup's share of stage 1 (and of the mix), because
   // a wave that queues this many loads is held up until most of them have been accepted, and the
   // work heading the dependency chain must not sit behind that.
-  issue_prefetch();
+  if (p.udelay > 0 && w >= p.items1 && w >= p.itemsM) {
+    while (wall_clock64() - t_begin < (unsigned long long)p.udelay) __builtin_amdgcn_s_sleep(2);
+  }
+  issue_prefetch(pf_lo, D2_PF);
 
   // ---- stage-2 activations: this slab's slice of z, polled from the tagged pairs into LDS ---------------
   __syncthreads();                                   // earlier uses of a_s and red are over
@@ -512,7 +477,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
       }
     }
     TR2(7);
-    if (w == 0) finish_epoch(p, epoch, G);
+    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
     return;
   }
 
@@ -623,7 +588,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     }
   }
   TR2(7);
-  if (w == 0) finish_epoch(p, epoch, G);
+  if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
 }
 
 
@@ -752,7 +717,9 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   const int M = p.M;
   TR2(0);
 
-  unsigned epoch = __hip_atomic_load(p.epoch_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  // (a plain, cached load: the word was last written before this kernel began, and hundreds of workgroups asking one
+  // address for a device-scope copy would queue up at a single memory channel - with every later load of theirs behind it)
+  unsigned epoch = *reinterpret_cast<const volatile unsigned*>(p.epoch_word) + 1u;
   if (epoch == 0u) epoch = 1u;
   auto check_in = [&]() {
     if (tid == 0) {
@@ -998,7 +965,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     TR2(9);
   }
   if (!has2) {
-    if (w == 0) finish_epoch(p, epoch, G);
+    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
     return;
   }
 
@@ -1180,7 +1147,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     }
   });
   TR2(7);
-  if (w == 0) finish_epoch(p, epoch, G);
+  if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
 }
 
 // ---- dense layer at up to 16 token rows ---------------------------------------------------------------
@@ -1332,18 +1299,6 @@ __global__ __launch_bounds__(256) void dense_slab_reduce_kernel(const float* __r
 // ---- host side -----------------------------------------------------------------------------------
 namespace {
 
-int env_i(const char* name, int dflt) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
-}
-// "this shape is not for me": 1, with the place reported when BLR_D2_DEBUG is set
-int d2_bail(int line) {
-  static const int dbg = env_i("BLR_D2_DEBUG", 0);
-  if (dbg) fprintf(stderr, "decode2: falling back (blr_decode.hip:%d)\n", line);
-  return 1;
-}
-int ilog2(int v) { int l = 0; while ((1 << l) < v) ++l; return l; }
-
 template <typename T, int WB>
 void* d2_kernel_mt(int MT) {
   switch (MT) {
@@ -1388,6 +1343,10 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
                          unsigned* err_word, hipStream_t st) {
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
+  {
+    const int rc = decode3_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
+    if (rc != 1) return rc;
+  }
   static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
   if (M >= mfma_min_m && a.wbits == 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
   static const int q_mfma_min_m = env_i("BLR_D2_Q_MFMA_MIN_M", 3);
@@ -1523,6 +1482,10 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     p.pf_depth = e_depth;
     static const int e_sparse = env_i("BLR_D2_SPARSE_POLL", 0);
     p.sparse_poll = e_sparse;
+    static const int e_udelay = env_i("BLR_D2_UDELAY", 0);
+    p.udelay = e_udelay;
+    static const int e_first = env_i("BLR_D2_PF_FIRST", 0);
+    p.pf_first = e_first;
   }
   const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)(p.zrep > 1 ? p.zrep : bo) * M * R * 8, 256);
   const size_t obytes = (size_t)(p.ks2 - 1) * bo * M * Q * 8;
