@@ -18,6 +18,10 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
 int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
                          unsigned* err_word, hipStream_t st);
 
+// The same call as two launches - stage 1, then mix + stage 2 - with ordinary memory between them (blr_decode_pair.hip; up
+// to four token rows, U (b, r, q), S with the rank contiguous).  region: scratch for y as T.  Same return convention.
+int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_bytes, hipStream_t st);
+
 // Dense layer out = x W (W (K, N)) at up to 16 rows: slabs of W on the matrix cores, fp32 partial sums of the k-slices in `part`
 // (room for max_slices * M * N floats) added by a second launch.  Returns BLR_OK, a negative blr_status, or 1 when the
 // call is not for this kernel.

@@ -1344,7 +1344,9 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
   {
-    const int rc = decode3_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
+    int rc = decode_pair_launch(a, region, decode2_region_bytes(), st);
+    if (rc != 1) return rc;
+    rc = decode3_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
     if (rc != 1) return rc;
   }
   static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
