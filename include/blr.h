@@ -33,7 +33,8 @@ typedef enum {
   BLR_ERR_WORKSPACE = -3,     /* workspace missing or smaller than blr_*_workspace_bytes()  */
   BLR_ERR_UNSUPPORTED = -4,   /* combination not implemented (e.g. decode algo with fp32)   */
   BLR_ERR_LAUNCH = -5,        /* the HIP runtime refused a launch                            */
-  BLR_ERR_NO_DEVICE = -6
+  BLR_ERR_NO_DEVICE = -6,
+  BLR_ERR_TIMEOUT = -7        /* a bounded wait inside a kernel gave up (blr_workspace_status)  */
 } blr_status;
 
 typedef enum { BLR_F16 = 0, BLR_BF16 = 1, BLR_F32 = 2 } blr_dtype;
@@ -65,6 +66,34 @@ typedef enum { BLR_OUT_INTERLEAVED = 0, BLR_OUT_BLOCKED = 1 } blr_monarch_out;
 
 /* Activation of the fused output stage (the *_fwd_ep entry points). */
 typedef enum { BLR_ACT_NONE = 0, BLR_ACT_GELU_TANH = 1, BLR_ACT_SILU = 2 } blr_act;
+
+/* ---- workspaces ---------------------------------------------------------------------------
+ * Every *_fwd entry point takes a caller-owned workspace of at least blr_*_workspace_bytes(...) bytes
+ * for the same arguments.  For calls served by the streaming kernels (M <= 16 under BLR_ALGO_AUTO,
+ * BLR_ALGO_STREAM, BLR_ALGO_STREAM_SPLIT) the workspace is more than scratch:
+ *   - it must be ZERO-FILLED before its first use.  Its head (16 KiB of control words: barrier and
+ *     check-in counters, the call epoch, the error word; then 32 KiB of arrival counters, 2 MiB of
+ *     accumulation buffers and 16 MiB of tagged hand-over values) carries state from one call to the
+ *     next: every value a workgroup hands to another is stored together with the epoch of its call,
+ *     and a call recognises its own values by that tag;
+ *   - nothing else may write to it between calls, and it must not be shared by calls that can
+ *     overlap: one workspace per stream, calls on it stream-ordered;
+ *   - the single-launch kernels wait for each other's values with every workgroup resident, so
+ *     they expect the GPU to themselves while they run (a few microseconds); when another kernel
+ *     occupies compute units at that moment a wait may run into its bound (about a second), the
+ *     kernel then finishes with undefined results and records that in the workspace.  Such a
+ *     give-up is reported by blr_workspace_status(), never by the call itself (which only enqueues).
+ * Calls served by the tiled kernels (M > 16, BLR_ALGO_TILED) use the workspace as plain scratch.
+ *
+ * blr_workspace_status: SYNCHRONISES the stream, returns BLR_OK if no bounded wait gave up on this
+ * workspace since the last query and BLR_ERR_TIMEOUT otherwise (the record is cleared; later calls
+ * are valid again).  The reference's harness records a per-function FAIL in the same role
+ * (reference layer.py:211-214, utils.py:8-13).  It must not be called while the stream is being
+ * captured.
+ * blr_set_spin_limit: polls after which a wait gives up, process-wide; 0 restores the default
+ * (4,000,000, about a second).  Meant for tests of the give-up path.                          */
+int blr_workspace_status(void* ws, size_t ws_bytes, void* stream);
+void blr_set_spin_limit(unsigned polls);
 
 const char* blr_last_error(void);
 int blr_version(void);

@@ -1,4 +1,5 @@
 // extern "C" entry points of libblr: argument validation, algorithm choice, workspace carving.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <mutex>
@@ -205,7 +206,35 @@ static int with_epilogue(const void* bias, int act, void* out, int64_t ldo, int 
 
 using namespace blr;
 
+namespace blr {
+static std::atomic<unsigned> g_spin_limit{0};
+unsigned spin_limit_now() {
+  const unsigned v = g_spin_limit.load(std::memory_order_relaxed);
+  return v ? v : 4000000u;
+}
+}  // namespace blr
+
 extern "C" {
+
+void blr_set_spin_limit(unsigned polls) { blr::g_spin_limit.store(polls, std::memory_order_relaxed); }
+
+// Synchronises the stream, reads the error word of a streaming workspace and clears it.
+int blr_workspace_status(void* ws, size_t ws_bytes, void* stream) {
+  if (!ws || ws_bytes < stream_ws_prefix_bytes()) { set_error("workspace_status: not a streaming workspace (%zu bytes)", ws_bytes); return BLR_ERR_WORKSPACE; }
+  hipStream_t st = (hipStream_t)stream;
+  unsigned* word = reinterpret_cast<unsigned*>(reinterpret_cast<char*>(ws) + stream_ws_error_offset());
+  unsigned host = 0;
+  hipError_t e = hipMemcpyAsync(&host, word, sizeof(unsigned), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) { set_error("workspace_status: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  if (!host) return BLR_OK;
+  e = hipMemsetAsync(word, 0, sizeof(unsigned), st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) { set_error("workspace_status: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  set_error("a bounded wait inside a kernel gave up since the last query: the results of the calls on this workspace since then are not valid "
+            "(another kernel kept part of the GPU busy, or two calls shared the workspace)");
+  return BLR_ERR_TIMEOUT;
+}
 
 const char* blr_last_error(void) { return g_err; }
 int blr_version(void) { return 100; }

@@ -78,6 +78,8 @@ __device__ __forceinline__ float wave_sum(float v) {
 // ---- host side ------------------------------------------------------------------------
 void set_error(const char* fmt, ...);
 int device_cus();
+// Polls after which a bounded wait inside a kernel gives up and sets the error word of its workspace (blr_set_spin_limit).
+unsigned spin_limit_now();
 // true when p is aligned to `bytes`.
 static inline bool aligned(const void* p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) % bytes) == 0; }
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -138,7 +140,8 @@ struct StreamBlastArgs {
   int split;                                    // 1: separate launches per phase
 };
 size_t stream_blast_workspace(int M, int in_f, int out_f, int b, int r, int wbits);
-size_t stream_ws_prefix_bytes();                // the fixed-place block at the start of a streaming workspace; per-call scratch follows
+size_t stream_ws_prefix_bytes();
+size_t stream_ws_error_offset();                // byte offset of the error word inside a streaming workspace                // the fixed-place block at the start of a streaming workspace; per-call scratch follows
 int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st);
 
 struct StreamGenericArgs {                      // dense / low-rank / monarch at M <= 16

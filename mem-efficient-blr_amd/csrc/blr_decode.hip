@@ -64,6 +64,7 @@ struct Decode2Params {
   unsigned long long* zt;              // [b][M][R] tagged
   unsigned long long* opart;           // [ks2 - 1][b][M][Q] tagged
   unsigned* epoch_word; unsigned* arrive_word; unsigned* err_word;
+  unsigned spin_limit;
 };
 
 // Sum of the row slots of a wave, then of the four waves; thread `col` < NC ends up with the
@@ -328,7 +329,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
           }
         }
         if (ok) break;
-        if (++spins > D2_SPIN_LIMIT) {
+        if (++spins > p.spin_limit) {
           __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
@@ -358,7 +359,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     TR2(9);
   }
   if (!has2) {
-    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
+    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, p.spin_limit);
     return;
   }
 
@@ -387,7 +388,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
         ok = ok && ((unsigned)(ld_tag(&p.zt[((int64_t)zi * M + m) * p.R + r]) >> 32) == epoch);
       }
       if (__syncthreads_and(ok)) break;
-      if (++spins > D2_SPIN_LIMIT) break;              // the full fetch below reports the failure
+      if (++spins > p.spin_limit) break;              // the full fetch below reports the failure
       __builtin_amdgcn_s_sleep(2);
     }
   }
@@ -413,7 +414,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
           }
         }
         if (ok) break;
-        if (++spins > D2_SPIN_LIMIT) {
+        if (++spins > p.spin_limit) {
           __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
@@ -477,7 +478,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
       }
     }
     TR2(7);
-    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
+    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, p.spin_limit);
     return;
   }
 
@@ -572,7 +573,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
               while (true) {
                 pv = ld_tag(src);
                 if ((unsigned)(pv >> 32) == epoch) break;
-                if (++spins > D2_SPIN_LIMIT) {
+                if (++spins > p.spin_limit) {
                   __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                   break;
                 }
@@ -588,7 +589,7 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
     }
   }
   TR2(7);
-  if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
+  if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, p.spin_limit);
 }
 
 
@@ -929,7 +930,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
           }
         }
         if (ok) break;
-        if (++spins > D2_SPIN_LIMIT) {
+        if (++spins > p.spin_limit) {
           __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
@@ -965,7 +966,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     TR2(9);
   }
   if (!has2) {
-    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
+    if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, p.spin_limit);
     return;
   }
 
@@ -988,7 +989,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
         ok = ok && ((unsigned)(ld_tag(&p.zt[((int64_t)zi * M + mc * DM_MC) * (p.R >> 1) + (r >> 1)]) >> 32) == epoch);
       }
       if (__syncthreads_and(ok)) break;
-      if (++spins > D2_SPIN_LIMIT) break;
+      if (++spins > p.spin_limit) break;
       __builtin_amdgcn_s_sleep(2);
     }
   }
@@ -1014,7 +1015,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
           }
         }
         if (ok) break;
-        if (++spins > D2_SPIN_LIMIT) {
+        if (++spins > p.spin_limit) {
           __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
@@ -1123,7 +1124,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
           }
         }
         if (ok) break;
-        if (++spins > D2_SPIN_LIMIT) {
+        if (++spins > p.spin_limit) {
           __hip_atomic_store(p.err_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
@@ -1147,7 +1148,7 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
     }
   });
   TR2(7);
-  if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, D2_SPIN_LIMIT);
+  if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, p.spin_limit);
 }
 
 // ---- dense layer at up to 16 token rows ---------------------------------------------------------------
@@ -1495,7 +1496,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   p.ypart = reinterpret_cast<unsigned long long*>(region);
   p.zt = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes);
   p.opart = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes + zbytes);
-  p.epoch_word = epoch_word; p.arrive_word = arrive_word; p.err_word = err_word;
+  p.epoch_word = epoch_word; p.arrive_word = arrive_word; p.err_word = err_word; p.spin_limit = spin_limit_now();
 
   int grid = p.items1 + p.items2;
   if (grid > resident) grid = resident;
@@ -1603,7 +1604,7 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
   p.ypart = reinterpret_cast<unsigned long long*>(region);
   p.zt = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes);
   p.opart = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(region) + ybytes + zbytes);
-  p.epoch_word = epoch_word; p.arrive_word = arrive_word; p.err_word = err_word;
+  p.epoch_word = epoch_word; p.arrive_word = arrive_word; p.err_word = err_word; p.spin_limit = spin_limit_now();
   int grid = p.items1 + p.items2;
   if (grid > resident) grid = resident;
   if (grid < p.items1) grid = p.items1;

@@ -613,8 +613,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
-  static const unsigned e_spin = (unsigned)env_i("BLR_D2_SPIN_LIMIT", (int)D2_SPIN_LIMIT);
-  p.spin_limit = e_spin;
+  p.spin_limit = spin_limit_now();
   static const int e_udelay = env_i("BLR_D3_UDELAY", 0);
   p.udelay = e_udelay;
   static const int e_vec = env_i("BLR_D3_VEC", 1);

@@ -67,6 +67,7 @@ struct StreamParams {
   int zatom, first, finish;                  // Z accumulation in use; launch holds the first / the last phase of the call
   float* zbuf[2]; unsigned zextent;          // two fixed-place Z buffers (ping-pong between calls), floats used by this call
   unsigned* ctrl;                           // barrier shards / finished counters / error word (see grid_barrier)
+  unsigned spin_limit;                      // polls after which the barrier gives up
 };
 
 // ---- device-scope accessors for data exchanged between workgroups ----------------------------------
@@ -95,7 +96,7 @@ __device__ __forceinline__ unsigned shard_population(int shard) {   // workgroup
   return ((unsigned)gridDim.x + BAR_SHARDS - 1 - shard) / BAR_SHARDS;
 }
 
-__device__ __forceinline__ void grid_barrier(unsigned* ctrl, unsigned nth) {
+__device__ __forceinline__ void grid_barrier(unsigned* ctrl, unsigned nth, unsigned spin_limit) {
   drain_stores();
   __syncthreads();
   if (threadIdx.x < 64) {
@@ -109,7 +110,7 @@ __device__ __forceinline__ void grid_barrier(unsigned* ctrl, unsigned nth) {
       unsigned v = __hip_atomic_load(&ctrl[s * BAR_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (__all(v >= target)) break;
       __builtin_amdgcn_s_sleep(1);
-      if (++spins > SPIN_LIMIT) {
+      if (++spins > spin_limit) {
         if (lane == 0) __hip_atomic_store(&ctrl[BAR_ERR], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         break;
       }
@@ -958,7 +959,7 @@ __global__ __launch_bounds__(256, 2) void stream_kernel(StreamParams p) {
     }
   }
   for (int ph = 0; ph < p.nph; ++ph) {
-    if (ph > 0 && p.use_barrier) { TR(6); grid_barrier(p.ctrl, (unsigned)ph); TR(7); }
+    if (ph > 0 && p.use_barrier) { TR(6); grid_barrier(p.ctrl, (unsigned)ph, p.spin_limit); TR(7); }
     run_phase<T, MT, WB, VEC>(p.ph[ph], p.M, smem, ph == 0 ? 0 : 8, zcur);
   }
   TR(15);
@@ -1161,6 +1162,7 @@ int launch_t(StreamParams& p, int MT, int split, hipStream_t st) {
 
 int launch(StreamParams& p, int dtype, int split, hipStream_t st) {
   int MT = mt_for(p.M);
+  p.spin_limit = spin_limit_now();
   if (dtype == BLR_F16) return launch_t<f16>(p, MT, split, st);
   if (dtype == BLR_BF16) return launch_t<bf16>(p, MT, split, st);
   set_error("stream: dtype %d not supported (f16 / bf16 only)", dtype);
@@ -1201,6 +1203,7 @@ size_t part_bound(int M, int batch, int K, int N) {
 // Bytes of the fixed-place block at the start of every streaming workspace (control words, counters, Z buffers, tagged pairs);
 // what follows it is per-call scratch.
 size_t stream_ws_prefix_bytes() { return ws_total(0, 0); }
+size_t stream_ws_error_offset() { return (size_t)BAR_ERR * sizeof(unsigned); }
 
 size_t stream_blast_workspace(int M, int in_f, int out_f, int b, int r, int wbits) {
   (void)wbits;

@@ -49,6 +49,8 @@ _SIGNATURES = {
     "blr_monarch_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 9 + [_vp, _sz, _vp, _vp, _i]),
     "blr_low_rank_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 6 + [_vp, _sz, _vp, _vp, _i]),
     "blr_dense_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp, _vp, _i]),
+    "blr_workspace_status": (_i, [_vp, _sz, _vp]),
+    "blr_set_spin_limit": (None, [_c.c_uint]),
     "blr_probe_dst_words": (_i, []),
     "blr_stream_probe": (_i, [_vp, _sz, _vp, _vp]),
 }
@@ -82,9 +84,34 @@ def lib():
     return _lib
 
 
-def check(rc, what):
+ERR_TIMEOUT = -7
+
+# Debug mode (environment BLR_CHECK=1, or set_debug_checks(True)): after every call that used a streaming
+# workspace the shims synchronise the stream and ask the library whether a bounded wait inside a kernel gave
+# up; if one did, the call raises BlrError instead of returning numbers that are not valid.  Off by default:
+# the query costs a device-to-host copy and a stream synchronisation per call.
+_debug_checks = os.environ.get("BLR_CHECK", "0") not in ("", "0")
+
+
+def set_debug_checks(on):
+    global _debug_checks
+    prev, _debug_checks = _debug_checks, bool(on)
+    return prev
+
+
+def workspace_status(ws, device=None):
+    """Status of a streaming workspace since the last query (0, or ERR_TIMEOUT); synchronises the stream, clears the flag."""
+    device = ws.device if device is None else device
+    return lib().blr_workspace_status(ws.data_ptr(), ws.numel(), stream_ptr(device))
+
+
+def check(rc, what, ws=None):
     if rc != 0:
         raise BlrError(f"{what} failed ({rc}): {lib().blr_last_error().decode()}")
+    if _debug_checks and ws is not None and getattr(ws, "_blr_streaming", False):
+        rc = workspace_status(ws)
+        if rc != 0:
+            raise BlrError(f"{what}: {lib().blr_last_error().decode()} ({rc})")
 
 
 def dtype_code(dt):
@@ -125,6 +152,7 @@ def workspace(device, nbytes, algo=ALGO_AUTO, M=None, dtype=None):
     if ws is None or ws.numel() < nbytes:
         size = max(int(nbytes), 1 << 20)
         ws = torch.zeros(size, dtype=torch.uint8, device=device)
+        ws._blr_streaming = streaming
         _workspaces[key] = ws
     return ws
 

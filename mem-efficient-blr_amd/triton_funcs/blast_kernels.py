@@ -82,7 +82,7 @@ def _blast(name, x, U, V, S, u_layout, s_layout, algo, want_intermediates):
                                z.data_ptr() if z is not None else None, y.data_ptr() if y is not None else None,
                                M, in_f, out_f, b1, r, dt, u_layout, s_layout, algo,
                                ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
-    L.check(rc, name)
+    L.check(rc, name, ws)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": b1, "rank": r,
                           "algo": algo, "dtype": str(x.dtype)}
     return out.reshape(*x.shape[:-1], out_f), z, y

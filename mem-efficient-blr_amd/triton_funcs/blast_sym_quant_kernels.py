@@ -98,7 +98,7 @@ def _blast_bmm_i8act(x, U, V, S):
     rc = lib.blr_blast_i8act_fwd(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
                                  out.data_ptr(), out.stride(0), None, None, M, in_f, out_f, b1, r, dt,
                                  L.U_QR, L.S_RIJ, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
-    L.check(rc, "triton_blast_bmm_int8_fp16")
+    L.check(rc, "triton_blast_bmm_int8_fp16", ws)
     _last_config["q"] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": b1, "rank": r, "bits": 0}
     return out.reshape(*x.shape[:-1], out_f)
 
@@ -130,7 +130,7 @@ def triton_blast_bmm_int8_fp16(x, U, V, S, config=(None, None, None)):
     rc = lib.blr_blast_q_fwd(x2.data_ptr(), x2.stride(0), U.codes.data_ptr(), U.scales.data_ptr(),
                              V.codes.data_ptr(), V.scales.data_ptr(), S.data_ptr(), out.data_ptr(), out.stride(0),
                              M, in_f, out_f, b1, r, dt, U.bits, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
-    L.check(rc, "triton_blast_bmm_int8_fp16")
+    L.check(rc, "triton_blast_bmm_int8_fp16", ws)
     _last_config["q"] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": b1, "rank": r, "bits": U.bits}
     return out.reshape(*x.shape[:-1], out_f)
 

@@ -34,7 +34,7 @@ def _dense(name, x, w, algo):
     else:
         rc = lib.blr_dense_fwd(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
                                M, in_f, out_f, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
-    L.check(rc, name)
+    L.check(rc, name, ws)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "algo": algo}
     return out
 

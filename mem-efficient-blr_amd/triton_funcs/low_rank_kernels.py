@@ -37,7 +37,7 @@ def _low_rank(name, x, a, b, algo, want_z):
         rc = lib.blr_low_rank_fwd(x2.data_ptr(), x2.stride(0), a.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
                                   z.data_ptr() if z is not None else None,
                                   M, in_f, out_f, r, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
-    L.check(rc, name)
+    L.check(rc, name, ws)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "rank": r, "algo": algo}
     return out, z
 

@@ -65,7 +65,7 @@ def _monarch(name, x, w1, w2, w2_layout, out_order, algo, want_out1):
                                  out1.data_ptr() if out1 is not None else None,
                                  M, in_f, out_f, k, q, dt, w2_layout, out_order, algo,
                                  ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
-    L.check(rc, name)
+    L.check(rc, name, ws)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": k, "rank": q, "algo": algo}
     return out.reshape(*x.shape[:-1], out_f), out1
 

@@ -26,13 +26,13 @@ def _blast_case(b, p, q, r, M, name, dtype, seed):
     return (lambda: getattr(K, name)(*args)), ref
 
 
-def _low_rank_case(in_f, out_f, r, M, dtype, seed):
+def _low_rank_case(in_f, out_f, r, M, dtype, seed, config=None):
     from triton_funcs import low_rank_kernels as K
     rng = np.random.default_rng(seed)
     x = rng.standard_normal((1, M, in_f)); a = rng.standard_normal((in_f, r)) / np.sqrt(r); bm = rng.standard_normal((r, out_f)) / np.sqrt(r)
     args = [dev(x, dtype), dev(a, dtype), dev(bm, dtype)]
     ref = (rounded(x, dtype) @ rounded(a, dtype)) @ rounded(bm, dtype)
-    return (lambda: K.triton_low_rank_fp16(*args)), ref.reshape(M, out_f)
+    return (lambda: K.triton_low_rank_fp16(*args, config=config)), ref.reshape(M, out_f)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -111,3 +111,46 @@ def test_decode_call_replayed_from_a_graph():
         assert torch.equal(captured, eager), f"replay {rep} differs from the eager result"
         other()                                     # eager calls between the replays
         torch.cuda.synchronize()
+
+
+def _spinning_cases(dtype):
+    """Calls served by kernels whose workgroups wait for each other (shapes at which the wait lasts microseconds)."""
+    return {
+        "blast_full_m8": _blast_case(16, 256, 256, 512, 8, "triton_blast_full_fp16", dtype, 60),
+        "blast_bmm_m1": _blast_case(16, 256, 256, 512, 1, "triton_blast_bmm_fp16", dtype, 61),
+        # 4104 input features cannot be cut into equal blocks of whole 16-byte pieces: the phase engine serves the call
+        # (one launch, a barrier of the whole grid between the two products)
+        "low_rank_phases_m1": _low_rank_case(4104, 4096, 512, 1, dtype, 62),
+    }
+
+
+@pytest.mark.parametrize("case", ["blast_full_m8", "blast_bmm_m1", "low_rank_phases_m1"])
+def test_wait_that_gives_up_is_reported_and_leaves_the_workspace_usable(case):
+    """With the poll limit forced to 1 from the host every wait gives up at once: the kernel still ends, the status query
+    returns BLR_ERR_TIMEOUT exactly once, and the next call at the normal limit is correct and reports a clean status."""
+    from triton_funcs import _lib as L
+    fn, ref = _spinning_cases(torch.float16)[case]
+    say(f"[case] forced give-up {case}")
+    good = fn().clone()
+    assert_close(good, ref.reshape(tuple(good.shape)), torch.float16, case)
+    ws = L.workspace(good.device, 1, L.ALGO_STREAM)
+    assert L.workspace_status(ws) == 0
+    L.lib().blr_set_spin_limit(1)
+    try:
+        fn()
+        torch.cuda.synchronize()
+        assert L.workspace_status(ws) == L.ERR_TIMEOUT
+        assert b"gave up" in L.lib().blr_last_error()
+        assert L.workspace_status(ws) == 0                      # the query cleared the flag
+        prev = L.set_debug_checks(True)
+        try:
+            with pytest.raises(L.BlrError, match="gave up"):
+                fn()
+        finally:
+            L.set_debug_checks(prev)
+    finally:
+        L.lib().blr_set_spin_limit(0)                           # back to the default limit
+    for rep in range(3):
+        out = fn()
+        assert torch.equal(out, good), f"call {rep} after the give-up differs from the result before it"
+    assert L.workspace_status(ws) == 0
