@@ -212,6 +212,24 @@ int blr_dense_fwd_ep(const void* x, int64_t ldx, const void* W, void* out, int64
                      int M, int in_f, int out_f, int dtype, int algo,
                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act);
 
+/* ---- BLAST forward that allocates nothing and takes no workspace -------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory or carry a workspace
+ * around: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same
+ * arithmetic and arguments as blr_blast_fwd with BLR_ALGO_TILED (and the two-launch decode path at up
+ * to four rows of f16 / bf16), without z_out / y_out / algo / ws: the intermediates live in a device
+ * array built into the library, BLR_STATIC_SCRATCH_BYTES per GPU, held from the first call on that GPU
+ * until the process ends.  A call whose intermediates do not fit (2 * b * M * r elements of dtype, each
+ * half rounded up to 256 bytes) returns BLR_ERR_WORKSPACE; use blr_blast_fwd with a workspace then.
+ * Calls no hipMalloc / hipFree and no allocating library routine.  Every call on a GPU shares that
+ * GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls ordered on one
+ * stream are safe.  The kernels write all of the scratch they read, so nothing has to be cleared
+ * between calls.  The first call on a device resolves the array's address (hipGetSymbolAddress); make
+ * it outside a graph capture.                                                                       */
+#define BLR_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
+int blr_blast_fwd_static(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                         void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
+                         int dtype, int u_layout, int s_layout, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

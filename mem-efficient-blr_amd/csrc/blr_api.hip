@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <mutex>
 #include "blr_common.h"
+#include "blr_decode.h"
 
 namespace blr {
 
@@ -616,6 +617,68 @@ int blr_dense_fwd_ep(const void* x, int64_t ldx, const void* W, void* out, int64
   return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
     return blr_dense_fwd(x, ldx, W, out, ldo, M, in_f, out_f, dtype, algo, ws, ws_bytes, stream);
   });
+}
+
+}  // extern "C"
+
+// ---- BLAST forward that allocates nothing ----------------------------------------------------------------------------
+// The intermediates Y and Z (and, at up to four rows, the stage-1 result of the two-launch decode path) live in a
+// file-scope device array instead of a caller's workspace.  Host code never uses the array's name as an address: the
+// device address is resolved once per device with hipGetSymbolAddress and kept in g_scratch_ptr.
+namespace {
+constexpr size_t kScratchBytes = BLR_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int scratch_for_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) { blr::set_error("blast_fwd_static: no usable current device (%d)", dev); return BLR_ERR_LAUNCH; }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) { blr::set_error("blast_fwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return BLR_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int blr_blast_fwd_static(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                         void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
+                         int dtype, int u_layout, int s_layout, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!x || !U || !V || !S || !out) { set_error("blast_fwd_static: null pointer"); return BLR_ERR_BAD_ARG; }
+  if (!dtype_ok(dtype) || u_layout < 0 || u_layout > 1 || s_layout < 0 || s_layout > 2) { set_error("blast_fwd_static: bad enum"); return BLR_ERR_BAD_ARG; }
+  int rc = check_blast_shape("blast_fwd_static", M, in_f, out_f, b, r);
+  if (rc) return rc;
+  if (ldx < in_f || ldo < out_f) { set_error("blast_fwd_static: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  const size_t need = 2 * align_up((size_t)b * M * r * elt_size(dtype), 256);
+  if (need > kScratchBytes) {
+    set_error("blast_fwd_static: the intermediates of this call need %zu bytes, the built-in scratch holds %zu (2 * b * M * r elements); "
+              "use blr_blast_fwd with a workspace", need, kScratchBytes);
+    return BLR_ERR_WORKSPACE;
+  }
+  void* ptr = nullptr;
+  rc = scratch_for_current_device(&ptr);
+  if (rc) return rc;
+  if (M <= 4 && dtype != BLR_F32) {
+    // Two launches with the stage-1 result in the scratch (plain loads and stores between them, nothing to clear).
+    StreamBlastArgs s = {};
+    s.x = x; s.ldx = ldx; s.U = U; s.V = V; s.S = S; s.out = out; s.ldo = ldo;
+    s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
+    s.dtype = dtype; s.u_layout = u_layout; s.s_layout = s_layout; s.wbits = 16;
+    rc = decode_pair_launch(s, ptr, kScratchBytes, st);
+    if (rc != 1) return rc;
+  }
+  // Three launches: Y = x V, Z = mix(S, Y), out = Z U; Y and Z are written in full before they are read.
+  return blast_tiled(x, ldx, U, V, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, u_layout, s_layout, 0, ptr, kScratchBytes, st);
 }
 
 }  // extern "C"

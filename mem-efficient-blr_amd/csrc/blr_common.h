@@ -140,8 +140,8 @@ struct StreamBlastArgs {
   int split;                                    // 1: separate launches per phase
 };
 size_t stream_blast_workspace(int M, int in_f, int out_f, int b, int r, int wbits);
-size_t stream_ws_prefix_bytes();
-size_t stream_ws_error_offset();                // byte offset of the error word inside a streaming workspace                // the fixed-place block at the start of a streaming workspace; per-call scratch follows
+size_t stream_ws_prefix_bytes();                // the fixed-place block at the start of a streaming workspace; per-call scratch follows
+size_t stream_ws_error_offset();                // byte offset of the error word inside a streaming workspace
 int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st);
 
 struct StreamGenericArgs {                      // dense / low-rank / monarch at M <= 16

@@ -51,6 +51,7 @@ _SIGNATURES = {
     "blr_dense_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp, _vp, _i]),
     "blr_workspace_status": (_i, [_vp, _sz, _vp]),
     "blr_set_spin_limit": (None, [_c.c_uint]),
+    "blr_blast_fwd_static": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64] + [_i] * 8 + [_vp]),
     "blr_probe_dst_words": (_i, []),
     "blr_stream_probe": (_i, [_vp, _sz, _vp, _vp]),
 }

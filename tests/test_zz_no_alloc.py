@@ -1,0 +1,84 @@
+"""GPU test of blr_blast_fwd_static, the BLAST forward that allocates nothing (intermediates in a device array of the library).
+
+Called through the C-ABI with raw pointers, on two calls in a row - the second with a smaller input, so that it runs over
+what the first left in the shared scratch - and compared with blr_blast_fwd (caller's workspace) on the same operands and
+with the oracle.  Tolerance: the fp16 bound of the other parity tests (1e-2 of max|ref|); where both entry points run the
+same kernels the results are required to be bit-identical.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import blr_oracle as O
+from gpu_util import assert_close, blast_inputs, dev, rounded, say
+
+pytestmark = pytest.mark.gpu
+
+STATIC_SCRATCH_BYTES = 16 << 20        # BLR_STATIC_SCRATCH_BYTES of include/blr.h
+
+
+def _operands(b, p, q, r, M, dtype, seed):
+    x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=seed)
+    Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)            # U (b, r, q), V (b, p, r), S (j, i, r)
+    ref = O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0].reshape(M, b * q)
+    return dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype), ref
+
+
+def _call_static(L, x, U, V, S, b, r):
+    M, in_f = x.shape
+    out_f = b * U.shape[2]
+    out = torch.full((M, out_f), float("nan"), device=x.device, dtype=x.dtype)
+    rc = L.lib().blr_blast_fwd_static(x.data_ptr(), x.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(), out.data_ptr(), out.stride(0),
+                                      M, in_f, out_f, b, r, L.dtype_code(x.dtype), L.U_RQ, L.S_JIR, L.stream_ptr(x.device))
+    return rc, out
+
+
+def _call_workspace(L, x, U, V, S, b, r, algo):
+    M, in_f = x.shape
+    out_f = b * U.shape[2]
+    dt = L.dtype_code(x.dtype)
+    out = torch.full((M, out_f), float("nan"), device=x.device, dtype=x.dtype)
+    ws = torch.zeros(max(L.lib().blr_blast_workspace_bytes(M, in_f, out_f, b, r, dt, algo), 1 << 20), dtype=torch.uint8, device=x.device)
+    rc = L.lib().blr_blast_fwd(x.data_ptr(), x.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(), out.data_ptr(), out.stride(0), None, None,
+                               M, in_f, out_f, b, r, dt, L.U_RQ, L.S_JIR, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
+    torch.cuda.synchronize()
+    return rc, out
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_two_calls_in_a_row_the_second_smaller(dtype):
+    from triton_funcs import _lib as L
+    # (b, p, q, r, M): prefill-sized first (three launches, Y and Z in the scratch), then fewer rows of a smaller layer,
+    # then decode-sized calls (two launches at up to four rows, stage-1 result in the scratch)
+    calls = [(16, 64, 72, 128, 96, L.ALGO_TILED), (4, 48, 24, 96, 7, L.ALGO_TILED), (16, 64, 72, 128, 3, L.ALGO_AUTO),
+             (4, 48, 24, 96, 1, L.ALGO_AUTO)]
+    for n, (b, p, q, r, M, algo) in enumerate(calls):
+        say(f"[case] blast_fwd_static call {n}: b={b} p={p} q={q} r={r} M={M} {dtype}")
+        x, U, V, S, ref = _operands(b, p, q, r, M, dtype, 70 + n)
+        rc, got = _call_static(L, x, U, V, S, b, r)
+        assert rc == 0, L.lib().blr_last_error().decode()
+        torch.cuda.synchronize()
+        rc2, want = _call_workspace(L, x, U, V, S, b, r, algo)
+        assert rc2 == 0, L.lib().blr_last_error().decode()
+        assert_close(got, ref, dtype, f"static call {n} against the oracle")
+        assert_close(got, want.to(torch.float64).cpu().numpy(), dtype, f"static call {n} against blr_blast_fwd")
+        if algo == L.ALGO_TILED:
+            assert torch.equal(got, want), f"call {n}: same kernels, different bits"
+
+
+def test_oversize_call_is_refused_without_a_launch():
+    from triton_funcs import _lib as L
+    b, p, q, r = 16, 64, 72, 128
+    M = STATIC_SCRATCH_BYTES // (2 * b * r * 2) + 1              # one row more than the scratch holds
+    x, U, V, S, _ = _operands(b, p, q, r, 1, torch.float16, 80)
+    xm = x.expand(M, -1).contiguous()
+    say(f"[case] blast_fwd_static oversize M={M}")
+    rc, out = _call_static(L, xm, U, V, S, b, r)
+    assert rc == -3, rc                                          # BLR_ERR_WORKSPACE
+    assert b"scratch holds" in L.lib().blr_last_error()
+    torch.cuda.synchronize()
+    assert torch.isnan(out).all()                                # nothing was launched
+    rc, out = _call_static(L, xm[: M - 1], U, V, S, b, r)        # the largest call that fits
+    assert rc == 0, L.lib().blr_last_error().decode()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
