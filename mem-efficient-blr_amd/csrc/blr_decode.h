@@ -22,6 +22,10 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
 // to four token rows, U (b, r, q), S with the rank contiguous).  region: scratch for y as T.  Same return convention.
 int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_bytes, hipStream_t st);
 
+// The same call as three launches - y = x V and out = z U on the matrix cores with the rank-space mix between them
+// (blr_decode_rows.hip; up to 16 token rows, U (b, r, q), two-byte weights).  region: scratch for y and z as T.  Same return convention.
+int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_bytes, hipStream_t st);
+
 // Dense layer out = x W (W (K, N)) at up to 16 rows: slabs of W on the matrix cores, fp32 partial sums of the k-slices in `part`
 // (room for max_slices * M * N floats) added by a second launch.  Returns BLR_OK, a negative blr_status, or 1 when the
 // call is not for this kernel.

@@ -1344,6 +1344,11 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
                          unsigned* err_word, hipStream_t st) {
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
+  static const int rows_min_m = env_i("BLR_DECODE_ROWS_MIN_M", 2);
+  if (M >= rows_min_m) {
+    const int rc = decode_rows_launch(a, region, decode2_region_bytes(), st);
+    if (rc != 1) return rc;
+  }
   {
     int rc = decode_pair_launch(a, region, decode2_region_bytes(), st);
     if (rc != 1) return rc;

@@ -65,6 +65,7 @@ struct Decode3Params {
   int itemsM, rch_log2, udelay;
   int x_vec, s_mode;                             // activations in 16-byte pieces; S: 0 = any strides, 1 = r contiguous, 2 = j contiguous
   unsigned spin_limit;
+  int xcd_order;
   unsigned long long* ypart;           // [ks1][b][M][R] tagged
   unsigned long long* zt;              // [bo or zrep][M][R] tagged
   unsigned long long* opart;           // [ks2 - 1][bo][M][Q] tagged
@@ -400,7 +401,8 @@ __global__ __launch_bounds__(D3_NT) void decode3_kernel(Decode3Params p) {
   // The whole slab of U is asked for at once.  Slots 0 .. PF - 9 hold the first pfn - 8 loads, the last eight slots the
   // last eight loads; groups of eight slots without a load are branched around, a single slot without one gets an
   // offset outside the buffer.  The speculative fetch of this slab's slice of z sits in front of the last group.
-  const uint32_t t2 = fd_div((uint32_t)w, p.nch2), nc2 = (uint32_t)w - t2 * p.nch2.d;
+  const uint32_t ws2 = p.xcd_order ? xcd_item((uint32_t)w, (uint32_t)p.items2) : (uint32_t)w;   // slab of this workgroup
+  const uint32_t t2 = fd_div(ws2, p.nch2), nc2 = ws2 - t2 * p.nch2.d;
   const uint32_t ksi2 = fd_div(t2, p.bodiv), i2 = t2 - ksi2 * p.bodiv.d;
   const int lpr2 = 1 << p.lpr2_log2, rpp2 = D3_NT >> p.lpr2_log2;
   const int cv2 = tid & (lpr2 - 1), rs2 = tid >> p.lpr2_log2;
@@ -614,6 +616,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
   p.spin_limit = spin_limit_now();
+  { static const int e_xcd = env_i("BLR_XCD_ORDER", 1); p.xcd_order = e_xcd; }
   static const int e_udelay = env_i("BLR_D3_UDELAY", 0);
   p.udelay = e_udelay;
   static const int e_vec = env_i("BLR_D3_VEC", 1);

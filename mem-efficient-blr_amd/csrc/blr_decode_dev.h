@@ -73,6 +73,14 @@ __device__ __forceinline__ void finish_epoch(unsigned* arrive_word, unsigned* ep
   }
 }
 
+// Workgroup w of a launch runs on XCD w % 8, and each XCD has its own L2.  Item order that gives every XCD a contiguous
+// run of the G items: neighbouring items (column chunks of one factor block, whose row pieces share cache lines when they
+// are not whole lines) then meet in one L2 instead of fetching the shared lines twice.
+__device__ __forceinline__ uint32_t xcd_item(uint32_t w, uint32_t G) {
+  const uint32_t x = w & 7u, base = G >> 3, rem = G & 7u;
+  return x * base + (x < rem ? x : rem) + (w >> 3);
+}
+
 // Division of a small number (< 65536) by a launch constant d (< 65536) without the divide sequence: m = ceil(2^32 / d),
 // n / d = high word of n * m; d == 1 is flagged by m == 0.
 struct FastDiv { uint32_t d, m; };

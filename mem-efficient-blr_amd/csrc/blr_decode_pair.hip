@@ -51,6 +51,7 @@ struct PairParams {
   FastDiv nch1, bdiv;
   int lpr2_log2, pfn, kld2_log2, octs_log2, jpg;
   FastDiv nch2;
+  int xcd_order;
 };
 
 __device__ __forceinline__ void lds_barrier2() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
@@ -208,7 +209,7 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   const int tid = threadIdx.x;
   const int M = p.M, R = p.R;
   TR4(0);
-  const uint32_t w = blockIdx.x;
+  const uint32_t w = p.xcd_order ? xcd_item(blockIdx.x, gridDim.x) : blockIdx.x;
   const uint32_t i2 = fd_div(w, p.nch2), nc2 = w - i2 * p.nch2.d;
   const int lpr2 = 1 << p.lpr2_log2, rpp2 = DP_NT >> p.lpr2_log2;
   const int cv2 = tid & (lpr2 - 1), rs2 = tid >> p.lpr2_log2;
@@ -424,6 +425,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     p.lpr1_log2 = ilog2(lpr); p.nch1 = fd_make((uint32_t)nch); p.bdiv = fd_make((uint32_t)b);
     p.ks1 = ks; p.kc1 = kc; p.kpad1_log2 = ilog2(kpad);
   }
+  { static const int e_xcd = env_i("BLR_XCD_ORDER", 1); p.xcd_order = e_xcd; }
   const size_t ybytes = (size_t)p.ks1 * b * M * R * 2;
   if (ybytes > region_bytes) return d2_bail(__LINE__);
   p.y = region;

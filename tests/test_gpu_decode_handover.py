@@ -116,7 +116,7 @@ def test_decode_call_replayed_from_a_graph():
 def _spinning_cases(dtype):
     """Calls served by kernels whose workgroups wait for each other (shapes at which the wait lasts microseconds)."""
     return {
-        "blast_full_m8": _blast_case(16, 256, 256, 512, 8, "triton_blast_full_fp16", dtype, 60),
+        "blast_bmm_m8": _blast_case(16, 256, 256, 512, 8, "triton_blast_bmm_fp16", dtype, 60),
         "blast_bmm_m1": _blast_case(16, 256, 256, 512, 1, "triton_blast_bmm_fp16", dtype, 61),
         # 4104 input features cannot be cut into equal blocks of whole 16-byte pieces: the phase engine serves the call
         # (one launch, a barrier of the whole grid between the two products)
@@ -124,7 +124,7 @@ def _spinning_cases(dtype):
     }
 
 
-@pytest.mark.parametrize("case", ["blast_full_m8", "blast_bmm_m1", "low_rank_phases_m1"])
+@pytest.mark.parametrize("case", ["blast_bmm_m8", "blast_bmm_m1", "low_rank_phases_m1"])
 def test_wait_that_gives_up_is_reported_and_leaves_the_workspace_usable(case):
     """With the poll limit forced to 1 from the host every wait gives up at once: the kernel still ends, the status query
     returns BLR_ERR_TIMEOUT exactly once, and the next call at the normal limit is correct and reports a clean status."""
