@@ -38,8 +38,9 @@ __device__ unsigned long long g_trace5[1024 * 16];
 struct RowsParams {
   const void* A; int64_t lda, a_bs;       // A[m * lda + bt * a_bs + k]; rows m >= M read as zero
   uint32_t a_bytes;
-  const void* W; int64_t w_bs;            // W[bt * w_bs + k * N + n]
+  const void* W; int64_t w_bs;            // W[bt * w_bs + k * N + n]: T, int8 codes, or int4 codes two to a byte
   void* out; int64_t o_ms, o_bs, o_ns;    // out[m * o_ms + bt * o_bs + n * o_ns]
+  const f16* scales;                      // codes: the product's column n of entry bt is multiplied by scales[bt * N + n]; else null
   int M, K, N;
   int kw;                                 // rows of a wave's share (a multiple of 32)
   int npc;                                // 16-byte column pieces of a chunk (1..16)
@@ -60,8 +61,83 @@ template <> struct RowsMfma<bf16> {
   }
 };
 
-template <typename T, int STEPS>
+// A lane's piece of one weight row: eight columns, as 16 bytes of T, 8 bytes of int8 codes or 4 bytes of int4 codes (low nibble
+// first), and its expansion to eight packed T.  For f16 the codes go through the exponent trick: byte u (the code with its
+// sign bit flipped) under the high byte 0x64 is the f16 number 1024 + u, and 1024 + u - 1152 = code, exactly.
+template <typename T, int WB> struct RowsPiece;
+template <typename T> struct RowsPiece<T, 16> {
+  using raw_t = u32x4;
+  static __device__ __forceinline__ raw_t load(__amdgpu_buffer_rsrc_t r, uint32_t off) { return ldw16(r, off, 0); }
+  static __device__ __forceinline__ u32x4 expand(raw_t v) { return v; }
+};
+template <typename T, int WB> struct RowsCodes {
+  // generic: through fp32 (exact for these small integers in either 16-bit type)
+  static __device__ __forceinline__ u32x4 expand8(const int (&c)[8]) {
+    typename TypeTraits<T>::vec8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = TypeTraits<T>::from_f32((float)c[e]);
+    return __builtin_bit_cast(u32x4, v);
+  }
+};
+template <typename T> struct RowsPiece<T, 8> {
+  using raw_t = u32x2;
+  static __device__ __forceinline__ raw_t load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+    return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 2));
+  }
+  static __device__ __forceinline__ u32x4 expand(raw_t v) {
+    if constexpr (sizeof(T) == 2 && __is_same(T, f16)) {
+      const f16x2 bias = {(f16)1152.0f, (f16)1152.0f};
+      u32x4 o;
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        const uint32_t u = v[d] ^ 0x80808080u;
+        const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u), hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+        o[2 * d] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, lo) - bias);
+        o[2 * d + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, hi) - bias);
+      }
+      return o;
+    } else {
+      int c[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) c[e] = (int)(int8_t)((v[e >> 2] >> ((e & 3) * 8)) & 0xFF);
+      return RowsCodes<T, 8>::expand8(c);
+    }
+  }
+};
+template <typename T> struct RowsPiece<T, 4> {
+  using raw_t = uint32_t;
+  static __device__ __forceinline__ raw_t load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+    return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 2);
+  }
+  static __device__ __forceinline__ u32x4 expand(raw_t v) {
+    if constexpr (__is_same(T, f16)) {
+      const f16x2 bias = {(f16)1032.0f, (f16)1032.0f};
+      const uint32_t u = v ^ 0x88888888u, uh = u >> 4;
+      u32x4 o;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        // byte d of u holds the codes of columns 2d (low nibble) and 2d + 1 (high nibble)
+        const uint32_t sel = 0x0C040C00u + (uint32_t)d * 0x00010001u;      // {0, uh.byte d, 0, u.byte d}
+        const uint32_t pr = (__builtin_amdgcn_perm(uh, u, sel) & 0x000F000Fu) | 0x64006400u;
+        o[d] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, pr) - bias);
+      }
+      return o;
+    } else {
+      int c[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) c[e] = ((int32_t)(v << (28 - 4 * e))) >> 28;
+      return RowsCodes<T, 4>::expand8(c);
+    }
+  }
+};
+
+// NK: the factor is stored transposed, W[bt][n][k] with k contiguous (U of the bmm names, (b, q, r)).  A 16-byte load then is
+// a lane's matrix-core operand as it stands: the lane of slot n and k-group g loads k .. k + 7 of column 16 cg + n for each of
+// the chunk's column groups cg (p.npc of them, 16 columns each).
+template <typename T, int STEPS, int WB, bool NK>
 __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
+  using Piece = RowsPiece<T, WB>;
+  static_assert(!NK || WB == 16, "codes are stored (k, n)");
   __shared__ __attribute__((aligned(16))) float red[DR_WAVES * 16 * 128];
   const int tid = threadIdx.x, wv = tid >> 6, l = tid & 63, n = l & 15, g = l >> 4;
   TR5(0);
@@ -70,11 +146,12 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   const uint32_t item = p.xcd_span ? (blockIdx.x & 7u) * p.xcd_span + (blockIdx.x >> 3) : blockIdx.x;
   const uint32_t bt = fd_div(item, p.nch), ch = item - bt * p.nch.d;
   const int N = p.N, K = p.K;
-  const int col0 = (int)ch * p.npc * 8;                  // first column of the chunk
-  const int colp = col0 + n * 8;                         // first column of this lane's pieces
-  const bool live = n < p.npc && colp < N;
+  const int cw = p.npc * (NK ? 16 : 8);                  // columns of a chunk
+  const int col0 = (int)ch * cw;                         // first column of the chunk
+  const int colp = col0 + (NK ? n : n * 8);              // first column of this lane's pieces
+  const bool live = NK ? true : (n < p.npc && colp < N);
   const __amdgpu_buffer_rsrc_t abuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.A), 0, p.a_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t wb = wbuf(reinterpret_cast<const char*>(p.W) + (int64_t)bt * p.w_bs * 2, (uint32_t)((int64_t)K * N * 2));
+  const __amdgpu_buffer_rsrc_t wb = wbuf(reinterpret_cast<const char*>(p.W) + (int64_t)bt * p.w_bs * WB / 8, (uint32_t)((int64_t)K * N * WB / 8));
   const int kb = wv * p.kw + 8 * g;                      // first of this lane's eight k of step 0
 
   // activations: row n of A, the lane's eight k of every step (16 bytes each); weights: eight rows per step, the lane's
@@ -82,7 +159,7 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   // they only reach rows and columns of the product that are never stored), so a narrow chunk costs the load path
   // only what its live lanes fetch.
   u32x4 av[STEPS];
-  u32x4 wr[STEPS][8];
+  typename Piece::raw_t wr[STEPS][8];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     asm volatile("" : "=v"(av[s]));
@@ -100,13 +177,22 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) av[s] = u32x4{0u, 0u, 0u, 0u};
   }
-  if (live) {
-    const uint32_t wbase = (uint32_t)(kb * N + colp) * 2u;
-    const uint32_t rowb = (uint32_t)N * 2u;
+  if constexpr (NK) {
+    // column groups past the chunk or the factor, and k past K, read as zero (offset out of the buffer's bounds)
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
 #pragma unroll
-      for (int t = 0; t < 8; ++t) wr[s][t] = ldw16(wb, wbase + (uint32_t)(32 * s + t) * rowb, 0);
+      for (int t = 0; t < 8; ++t) {
+        const int c = colp + 16 * t, k = kb + 32 * s;
+        wr[s][t] = Piece::load(wb, (t < p.npc && c < N && k < K) ? (uint32_t)(c * K + k) * 2u : DR_OOB);
+      }
+  } else if (live) {
+    const uint32_t wbase = (uint32_t)(kb * N + colp) * (uint32_t)WB / 8u;
+    const uint32_t rowb = (uint32_t)N * (uint32_t)WB / 8u;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) wr[s][t] = Piece::load(wb, wbase + (uint32_t)(32 * s + t) * rowb);
   }
 
   TR5(1);
@@ -115,22 +201,38 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
+    if constexpr (NK) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
-      u32x4 bv;
+      for (int e = 0; e < 8; ++e) acc[e] = RowsMfma<T>::run(av[s], Piece::expand(wr[s][e]), acc[e]);
+    } else {
+      u32x4 wx[8];
 #pragma unroll
-      for (int h = 0; h < 4; ++h) bv[h] = __builtin_amdgcn_perm(wr[s][2 * h + 1][e >> 1], wr[s][2 * h][e >> 1], sel);
-      acc[e] = RowsMfma<T>::run(av[s], bv, acc[e]);
+      for (int t = 0; t < 8; ++t) wx[t] = Piece::expand(wr[s][t]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+        u32x4 bv;
+#pragma unroll
+        for (int h = 0; h < 4; ++h) bv[h] = __builtin_amdgcn_perm(wx[2 * h + 1][e >> 1], wx[2 * h][e >> 1], sel);
+        acc[e] = RowsMfma<T>::run(av[s], bv, acc[e]);
+      }
     }
   }
   TR5(2);
-  // acc[e][t] is row 4 g + t, column colp + e of this wave's partial product
+  if constexpr (NK) {
+    // acc[e][t] is row 4 g + t, column col0 + 16 e + n
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    float* dst = &red[((wv * 16 + 4 * g + t) * 128) + n * 8];
-    *reinterpret_cast<f32x4*>(dst) = f32x4{acc[0][t], acc[1][t], acc[2][t], acc[3][t]};
-    *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[4][t], acc[5][t], acc[6][t], acc[7][t]};
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) red[((wv * 16 + 4 * g + t) * 128) + 16 * e + n] = acc[e][t];
+  } else {
+    // acc[e][t] is row 4 g + t, column colp + e of this wave's partial product
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      float* dst = &red[((wv * 16 + 4 * g + t) * 128) + n * 8];
+      *reinterpret_cast<f32x4*>(dst) = f32x4{acc[0][t], acc[1][t], acc[2][t], acc[3][t]};
+      *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[4][t], acc[5][t], acc[6][t], acc[7][t]};
+    }
   }
   __syncthreads();
   TR5(3);
@@ -139,7 +241,13 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
 #pragma unroll
   for (int w = 1; w < DR_WAVES; ++w) tot += *reinterpret_cast<const f32x4*>(&red[(w * 16 + m) * 128 + c4]);
   const int col = col0 + c4;
-  if (m < p.M && c4 < p.npc * 8 && col < N) {
+  if (p.scales && m < p.M && c4 < cw && col < N) {
+    const f16* sc = p.scales + (int64_t)bt * N + col;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (col + e < N) tot[e] *= (float)sc[e];
+  }
+  if (m < p.M && c4 < cw && col < N) {
     T* o = reinterpret_cast<T*>(p.out) + (int64_t)m * p.o_ms + (int64_t)bt * p.o_bs;
     if (p.o_ns == 1 && col + 3 < N && ((reinterpret_cast<uintptr_t>(o + col) & 7) == 0)) {
       typename TypeTraits<T>::vec4 v;
@@ -191,7 +299,50 @@ __global__ __launch_bounds__(256) void rows_mix_kernel(const T* __restrict__ Y, 
   *reinterpret_cast<V4*>(Z + ((int64_t)i * M + m) * R + r4 * 4) = o;
 }
 
+// The same mix for S stored (r, i, j) - the input block contiguous (the layout of the bmm names and of the quantized
+// entry points).  Neighbouring threads take neighbouring output blocks i, so that a wave reads whole (r, :, :) slices of S.
+template <typename T>
+__global__ __launch_bounds__(256) void rows_mix_rij_kernel(const T* __restrict__ Y, const T* __restrict__ S, T* __restrict__ Z,
+                                                            int M, int R, FastDiv r4div, uint32_t total) {
+  constexpr int B = 16;
+  const uint32_t item = blockIdx.x * 256u + threadIdx.x;
+  if (item >= total) return;
+  const uint32_t i = item & (B - 1), t = item >> 4;
+  const uint32_t m = fd_div(t, r4div), r4 = t - m * r4div.d;
+  using V4 = typename TypeTraits<T>::vec4;
+  using V8 = typename TypeTraits<T>::vec8;
+  V8 sv[4][2];
+  V4 yv[B];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const T* sp = S + ((int64_t)(r4 * 4 + e) * B + i) * B;
+    sv[e][0] = *reinterpret_cast<const V8*>(sp); sv[e][1] = *reinterpret_cast<const V8*>(sp + 8);
+  }
+  const T* yp = Y + (int64_t)m * R + r4 * 4;
+  const int64_t y_sj = (int64_t)M * R;
+#pragma unroll
+  for (int j = 0; j < B; ++j) yv[j] = *reinterpret_cast<const V4*>(yp + j * y_sj);
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < B; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] += TypeTraits<T>::to_f32(sv[e][j >> 3][j & 7]) * TypeTraits<T>::to_f32(yv[j][e]);
+  V4 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = TypeTraits<T>::from_f32(acc[e]);
+  *reinterpret_cast<V4*>(Z + ((int64_t)i * M + m) * R + r4 * 4) = o;
+}
+
 namespace {
+
+template <typename T>
+int rows_mix_rij_t(const void* Y, const void* S, void* Z, int M, int R, hipStream_t st) {
+  const uint32_t total = (uint32_t)((int64_t)M * 16 * (R / 4));
+  hipLaunchKernelGGL((rows_mix_rij_kernel<T>), dim3((unsigned)cdiv(total, 256)), dim3(256), 0, st, (const T*)Y, (const T*)S, (T*)Z, M, R,
+                     fd_make((uint32_t)(R / 4)), total);
+  BLR_CHECK_LAUNCH("rows_mix_rij");
+  return BLR_OK;
+}
 
 template <typename T>
 int rows_mix_t(const void* Y, const void* S, void* Z, int M, int b, int R, int64_t s_si, int64_t s_sj, hipStream_t st) {
@@ -205,12 +356,12 @@ int rows_mix_t(const void* Y, const void* S, void* Z, int M, int b, int R, int64
 }
 
 // Column pieces per chunk: the busiest compute unit's bytes bound the launch (35 GB/s each), short row pieces cost DRAM efficiency.
-int plan_pieces(int batch, int K, int N, int cus) {
+int plan_pieces(int batch, int K, int N, int wbits, int cus) {
   const int pieces = N / 8;
   int best = 16; double best_t = 1e30;
   for (int npc = 16; npc >= 2; --npc) {
     const int64_t chunks = (int64_t)batch * cdiv(pieces, npc);
-    const double slab = (double)K * npc * 16.0;
+    const double slab = (double)K * npc * wbits;      // bytes: 8 columns of wbits bits per piece and row
     double t = (double)cdiv(chunks, cus) * (0.5 + slab / 35e3);
     if (npc < 8) t += 0.05 * (8 - npc);
     if (t < best_t - 1e-9) { best_t = t; best = npc; }
@@ -218,34 +369,50 @@ int plan_pieces(int batch, int K, int N, int cus) {
   return best;
 }
 
-template <typename T>
+template <typename T, int WB, bool NK = false>
 int rows_launch_t(RowsParams& p, int batch, hipStream_t st) {
   const int steps = p.kw / 32;
   const dim3 grid((unsigned)(batch * p.nch.d)), block(DR_NT);
   switch (steps) {
-    case 1: hipLaunchKernelGGL((rows_product_kernel<T, 1>), grid, block, 0, st, p); break;
-    case 2: hipLaunchKernelGGL((rows_product_kernel<T, 2>), grid, block, 0, st, p); break;
-    case 3: hipLaunchKernelGGL((rows_product_kernel<T, 3>), grid, block, 0, st, p); break;
-    default: hipLaunchKernelGGL((rows_product_kernel<T, 4>), grid, block, 0, st, p); break;
+    case 1: hipLaunchKernelGGL((rows_product_kernel<T, 1, WB, NK>), grid, block, 0, st, p); break;
+    case 2: hipLaunchKernelGGL((rows_product_kernel<T, 2, WB, NK>), grid, block, 0, st, p); break;
+    case 3: hipLaunchKernelGGL((rows_product_kernel<T, 3, WB, NK>), grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL((rows_product_kernel<T, 4, WB, NK>), grid, block, 0, st, p); break;
   }
   BLR_CHECK_LAUNCH("rows_product");
   return BLR_OK;
 }
 
 // One batch of skinny products; returns 1 when the operands do not fit the kernel.
-int rows_product(RowsParams p, int batch, int dtype, hipStream_t st) {
+int rows_product(RowsParams p, int batch, int dtype, int wbits, bool nk, hipStream_t st) {
+  if (nk && wbits != 16) return 1;
   if (p.K % 8 || p.N % 8 || p.N > 65536 || p.K > DR_WAVES * DR_MAX_STEPS * 32) return 1;
-  if (!aligned(p.A, 16) || !aligned(p.W, 16) || p.lda % 8 || p.a_bs % 8 || p.w_bs % 8) return 1;
+  if (!aligned(p.A, 16) || !aligned(p.W, 16) || p.lda % 8 || p.a_bs % 8 || p.w_bs % 32) return 1;
   if ((int64_t)p.K * p.N * 2 >= (int64_t)DR_OOB) return 1;
+  if (wbits != 16 && dtype != BLR_F16 && dtype != BLR_BF16) return 1;
   p.kw = (int)cdiv(cdiv(p.K, DR_WAVES), 32) * 32;
   const int cus = device_cus() > 0 ? device_cus() : 256;
   static const int e_npc = env_i("BLR_DR_NPC", 0);
-  p.npc = e_npc > 0 && e_npc <= 16 ? e_npc : plan_pieces(batch, p.K, p.N, cus);
-  p.nch = fd_make((uint32_t)cdiv(p.N / 8, p.npc));
+  if (nk) {
+    // column groups of 16 per chunk (at most 8): as many as keep the busiest compute unit's bytes lowest
+    int best = 8; double best_t = 1e30;
+    for (int cg = 8; cg >= 1; --cg) {
+      const double t = (double)cdiv((int64_t)batch * cdiv(p.N, 16 * cg), cus) * (0.5 + (double)p.K * cg * 32.0 / 35e3);
+      if (t < best_t - 1e-9) { best_t = t; best = cg; }
+    }
+    p.npc = best;
+    p.nch = fd_make((uint32_t)cdiv(p.N, 16 * p.npc));
+  } else {
+    p.npc = e_npc > 0 && e_npc <= 16 ? e_npc : plan_pieces(batch, p.K, p.N, wbits, cus);
+    p.nch = fd_make((uint32_t)cdiv(p.N / 8, p.npc));
+  }
   if ((int64_t)batch * p.nch.d >= 65536) return 1;
   static const int e_xcd = env_i("BLR_DR_XCD", 1);
   p.xcd_span = (e_xcd && (batch * p.nch.d) % 8 == 0) ? (uint32_t)(batch * p.nch.d / 8) : 0u;
-  return dtype == BLR_F16 ? rows_launch_t<f16>(p, batch, st) : rows_launch_t<bf16>(p, batch, st);
+  if (nk) return dtype == BLR_F16 ? rows_launch_t<f16, 16, true>(p, batch, st) : rows_launch_t<bf16, 16, true>(p, batch, st);
+  if (wbits == 16) return dtype == BLR_F16 ? rows_launch_t<f16, 16>(p, batch, st) : rows_launch_t<bf16, 16>(p, batch, st);
+  if (wbits == 8) return dtype == BLR_F16 ? rows_launch_t<f16, 8>(p, batch, st) : rows_launch_t<bf16, 8>(p, batch, st);
+  return dtype == BLR_F16 ? rows_launch_t<f16, 4>(p, batch, st) : rows_launch_t<bf16, 4>(p, batch, st);
 }
 
 }  // namespace
@@ -255,7 +422,9 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   if (!enabled) return 1;
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int b = a.b, M = a.M, R = a.r, P = a.in_f / a.b, Q = a.out_f / bo;
-  if (M < 1 || M > 16 || a.wbits != 16 || a.u_layout != BLR_U_RQ || a.perm_per > 0 || !a.S || bo != b) return 1;
+  const bool u_nk = a.u_layout == BLR_U_QR;
+  if (M < 1 || M > 16 || a.perm_per > 0 || !a.S || bo != b || (u_nk && a.wbits != 16)) return 1;
+  if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return 1;
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return 1;
   const size_t ybytes = align_up((size_t)b * M * R * 2, 256);
   if (2 * ybytes > region_bytes) return 1;
@@ -268,17 +437,17 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   s1.A = a.x; s1.lda = a.ldx; s1.a_bs = P; s1.a_bytes = (uint32_t)(x_elems * 2);
   s1.W = a.V; s1.w_bs = (int64_t)P * R;
   s1.out = Y; s1.o_ms = R; s1.o_bs = (int64_t)M * R; s1.o_ns = 1;
-  s1.M = M; s1.K = P; s1.N = R;
+  s1.M = M; s1.K = P; s1.N = R; s1.scales = a.wbits != 16 ? (const f16*)a.v_scales : nullptr;
   RowsParams s2 = {};
   s2.A = Z; s2.lda = R; s2.a_bs = (int64_t)M * R; s2.a_bytes = (uint32_t)((size_t)b * M * R * 2);
   s2.W = a.U; s2.w_bs = (int64_t)R * Q;
   s2.out = a.out; s2.o_ms = a.ldo;
   s2.o_bs = a.out_ns ? a.out_bs : Q; s2.o_ns = a.out_ns ? a.out_ns : 1;
-  s2.M = M; s2.K = R; s2.N = Q; s2.trace_base = 512;
+  s2.M = M; s2.K = R; s2.N = Q; s2.trace_base = 512; s2.scales = a.wbits != 16 ? (const f16*)a.u_scales : nullptr;
   // both products must fit before the first launch
   if (P % 8 || R % 8 || Q % 8 || P > 1024 || R > 1024 || !aligned(a.x, 16) || !aligned(a.V, 16) || !aligned(a.U, 16) || a.ldx % 8) return 1;
 
-  int rc = rows_product(s1, b, a.dtype, st);
+  int rc = rows_product(s1, b, a.dtype, a.wbits, false, st);
   if (rc) return rc;
   int64_t si, sj, sr;
   if (a.s_layout == BLR_S_JIR) { sj = (int64_t)b * R; si = R; sr = 1; }
@@ -286,10 +455,12 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   else { si = (int64_t)b * R; sj = R; sr = 1; }
   if (sr == 1 && si % 4 == 0 && sj % 4 == 0 && R % 4 == 0 && aligned(a.S, 8) && (int64_t)M * b * (R / 4) * (R / 4) < ((int64_t)1 << 32) && b < 65536)   // the multiply-high division is exact below 2^32 / divisor
     rc = a.dtype == BLR_F16 ? rows_mix_t<f16>(Y, a.S, Z, M, b, R, si, sj, st) : rows_mix_t<bf16>(Y, a.S, Z, M, b, R, si, sj, st);
+  else if (a.s_layout == BLR_S_RIJ && b == 16 && R % 4 == 0 && aligned(a.S, 16) && (int64_t)M * (R / 4) * (R / 4) < ((int64_t)1 << 32))
+    rc = a.dtype == BLR_F16 ? rows_mix_rij_t<f16>(Y, a.S, Z, M, R, st) : rows_mix_rij_t<bf16>(Y, a.S, Z, M, R, st);
   else
     rc = blast_mix_launch(Y, a.S, Z, M, b, R, si, sj, sr, a.dtype, st, 0);
   if (rc) return rc;
-  rc = rows_product(s2, b, a.dtype, st);
+  rc = rows_product(s2, b, a.dtype, a.wbits, u_nk, st);
   return rc == 1 ? BLR_ERR_UNSUPPORTED : rc;
 }
 

@@ -113,10 +113,23 @@ def test_decode_call_replayed_from_a_graph():
         torch.cuda.synchronize()
 
 
+def _monarch_case(b, p, rank, s_out, M, dtype, seed):
+    from triton_funcs import monarch_kernels as K
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((1, M, b * p))
+    w1_t = rng.standard_normal((b, rank, p)) / np.sqrt(p)
+    w2_t = rng.standard_normal((b, s_out, rank)) / np.sqrt(rank)
+    w1 = O.monarch_w1_to_kernel_layout(w1_t, b)
+    w2 = np.ascontiguousarray(np.transpose(w2_t, (0, 2, 1)))          # (b, rank, s): what the right_left name takes
+    args = [dev(x, dtype), dev(w1, dtype), dev(w2, dtype)]
+    ref = O.monarch_forward(rounded(x, dtype), rounded(w1_t, dtype), rounded(w2_t, dtype))[0]
+    return (lambda: K.triton_monarch_right_left_fp16(*args)), ref.reshape(M, b * s_out)
+
+
 def _spinning_cases(dtype):
     """Calls served by kernels whose workgroups wait for each other (shapes at which the wait lasts microseconds)."""
     return {
-        "blast_bmm_m8": _blast_case(16, 256, 256, 512, 8, "triton_blast_bmm_fp16", dtype, 60),
+        "monarch_m8": _monarch_case(4, 1024, 1024, 1024, 8, dtype, 60),
         "blast_bmm_m1": _blast_case(16, 256, 256, 512, 1, "triton_blast_bmm_fp16", dtype, 61),
         # 4104 input features cannot be cut into equal blocks of whole 16-byte pieces: the phase engine serves the call
         # (one launch, a barrier of the whole grid between the two products)
@@ -124,7 +137,7 @@ def _spinning_cases(dtype):
     }
 
 
-@pytest.mark.parametrize("case", ["blast_bmm_m8", "blast_bmm_m1", "low_rank_phases_m1"])
+@pytest.mark.parametrize("case", ["monarch_m8", "blast_bmm_m1", "low_rank_phases_m1"])
 def test_wait_that_gives_up_is_reported_and_leaves_the_workspace_usable(case):
     """With the poll limit forced to 1 from the host every wait gives up at once: the kernel still ends, the status query
     returns BLR_ERR_TIMEOUT exactly once, and the next call at the normal limit is correct and reports a clean status."""
