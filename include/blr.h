@@ -188,6 +188,13 @@ int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t 
  * low_rank_kernels.py:419-450): an empirical bandwidth ceiling for the decode kernels.        */
 int blr_probe_dst_words(void);
 int blr_stream_probe(const void* src, size_t bytes, void* dst, void* stream);
+/* The whole memory pattern of a layer without its arithmetic, as the reference's load_store kernels have it
+ * (reference triton_funcs/dense_kernels.py:150-227: load x, load w, store a zero y; low_rank_kernels.py:163-236
+ * with two factors): every byte of x, w1 and (if w2_bytes > 0) w2 is loaded with the streaming pattern and
+ * zeros are stored over all y_bytes of y.  All sizes are multiples of 16 and all pointers 16-byte aligned;
+ * dst as for blr_stream_probe.                                                                          */
+int blr_load_store_probe(const void* x, size_t x_bytes, const void* w1, size_t w1_bytes, const void* w2, size_t w2_bytes,
+                         void* y, size_t y_bytes, void* dst, void* stream);
 
 /* ---- fused output stage ---------------------------------------------------------------------
  * out = act(op(x) + bias): what the callers do right after the operator - the bias add of the wrapper

@@ -165,6 +165,13 @@ static int quantize_t(const void* w, int64_t outer, int64_t reduce, int64_t inne
 struct PendingEpilogue { const void* bias; int act; bool armed; bool used; };
 static thread_local PendingEpilogue tl_ep = {nullptr, 0, false, false};
 
+bool epilogue_pending(const void** bias, int* act) {
+  if (!tl_ep.armed || tl_ep.used) return false;
+  *bias = tl_ep.bias; *act = tl_ep.act;
+  return true;
+}
+void epilogue_taken() { tl_ep.used = true; }
+
 static void attach_epilogue(GemmArgs& g) {
   if (!tl_ep.armed) return;
   g.bias = tl_ep.bias; g.act = tl_ep.act;

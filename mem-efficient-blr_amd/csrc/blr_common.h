@@ -80,6 +80,10 @@ void set_error(const char* fmt, ...);
 int device_cus();
 // Polls after which a bounded wait inside a kernel gives up and sets the error word of its workspace (blr_set_spin_limit).
 unsigned spin_limit_now();
+// The fused output stage armed by the *_fwd_ep entry point of the running call, if any (bias of dtype or null, blr_act); a kernel
+// that applies it itself says so with epilogue_taken(), otherwise the entry point finishes with an elementwise launch.
+bool epilogue_pending(const void** bias, int* act);
+void epilogue_taken();
 // true when p is aligned to `bytes`.
 static inline bool aligned(const void* p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) % bytes) == 0; }
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -40,6 +40,9 @@ struct RowsParams {
   uint32_t a_bytes;
   const void* W; int64_t w_bs;            // W[bt * w_bs + k * N + n]: T, int8 codes, or int4 codes two to a byte
   void* out; int64_t o_ms, o_bs, o_ns;    // out[m * o_ms + bt * o_bs + n * o_ns]
+  const void* bias; int act;              // fused output stage (bias of T indexed like a row of out, or null; blr_act), applied to
+                                          // the result rounded to T - what a separate elementwise kernel would see
+  int ep;
   const f16* scales;                      // codes: the product's column n of entry bt is multiplied by scales[bt * N + n]; else null
   int M, K, N;
   int kw;                                 // rows of a wave's share (a multiple of 32)
@@ -247,6 +250,16 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
     for (int e = 0; e < 4; ++e)
       if (col + e < N) tot[e] *= (float)sc[e];
   }
+  if (p.ep && m < p.M && c4 < cw && col < N) {
+    const T* bias = reinterpret_cast<const T*>(p.bias);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (col + e < N) {
+        float v = TypeTraits<T>::to_f32(TypeTraits<T>::from_f32(tot[e]));
+        if (bias) v += TypeTraits<T>::to_f32(bias[(int64_t)bt * p.o_bs + (int64_t)(col + e) * p.o_ns]);
+        tot[e] = apply_act(v, p.act);
+      }
+  }
   if (m < p.M && c4 < cw && col < N) {
     T* o = reinterpret_cast<T*>(p.out) + (int64_t)m * p.o_ms + (int64_t)bt * p.o_bs;
     if (p.o_ns == 1 && col + 3 < N && ((reinterpret_cast<uintptr_t>(o + col) & 7) == 0)) {
@@ -447,6 +460,8 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   // both products must fit before the first launch
   if (P % 8 || R % 8 || Q % 8 || P > 1024 || R > 1024 || !aligned(a.x, 16) || !aligned(a.V, 16) || !aligned(a.U, 16) || a.ldx % 8) return 1;
 
+  const void* ep_bias = nullptr; int ep_act = 0;
+  if (epilogue_pending(&ep_bias, &ep_act)) { s2.ep = 1; s2.bias = ep_bias; s2.act = ep_act; }
   int rc = rows_product(s1, b, a.dtype, a.wbits, false, st);
   if (rc) return rc;
   int64_t si, sj, sr;
@@ -461,6 +476,7 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     rc = blast_mix_launch(Y, a.S, Z, M, b, R, si, sj, sr, a.dtype, st, 0);
   if (rc) return rc;
   rc = rows_product(s2, b, a.dtype, a.wbits, u_nk, st);
+  if (rc == BLR_OK && s2.ep) epilogue_taken();
   return rc == 1 ? BLR_ERR_UNSUPPORTED : rc;
 }
 

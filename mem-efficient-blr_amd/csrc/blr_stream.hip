@@ -1419,6 +1419,37 @@ __global__ __launch_bounds__(256) void probe_kernel(const u32x4* __restrict__ sr
   if ((threadIdx.x & 63) == 0) atomicXor(&dst[blockIdx.x], v);
 }
 
+// Loads every byte of up to three operands with the streaming pattern and stores zeros over all of y: the memory traffic
+// of a layer (activations in, factors in, result out) without its arithmetic.  The stored value depends on the loaded
+// data (it is zero unless the checksum hits one particular value), so no load can be dropped.
+struct ProbeSrc { const u32x4* p; size_t nvec; };
+__global__ __launch_bounds__(256) void load_store_probe_kernel(ProbeSrc s0, ProbeSrc s1, ProbeSrc s2, u32x4* __restrict__ y, size_t yvec,
+                                                               uint32_t* __restrict__ dst) {
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  const size_t stride = (size_t)gridDim.x * 256 * 4;
+  const ProbeSrc srcs[3] = {s0, s1, s2};
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    const u32x4* src = srcs[k].p;
+    const size_t nvec = srcs[k].nvec;
+    size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x;
+    for (; i + 3 * 256 < nvec; i += stride) {
+      u32x4 a = __builtin_nontemporal_load(&src[i]);
+      u32x4 b = __builtin_nontemporal_load(&src[i + 256]);
+      u32x4 c = __builtin_nontemporal_load(&src[i + 512]);
+      u32x4 e = __builtin_nontemporal_load(&src[i + 768]);
+      acc ^= a ^ b ^ c ^ e;
+    }
+    for (; i < nvec; i += 256) acc ^= __builtin_nontemporal_load(&src[i]);      // the last, short block of four
+  }
+  uint32_t v = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+  for (int o = 32; o > 0; o >>= 1) v ^= __shfl_xor(v, o, 64);
+  if ((threadIdx.x & 63) == 0) atomicXor(&dst[blockIdx.x], v);
+  const uint32_t z = (v == 0x9E3779B9u && acc[0] == 0x85EBCA6Bu) ? 1u : 0u;
+  const u32x4 zero = {z, z, z, z};
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < yvec; i += (size_t)gridDim.x * 256) __builtin_nontemporal_store(zero, &y[i]);
+}
+
 }  // namespace blr
 
 #ifdef BLR_TRACE
@@ -1428,6 +1459,23 @@ extern "C" int blr_debug_trace(unsigned long long* host, int n) {
 #endif
 
 extern "C" int blr_probe_dst_words(void) { return 2 * blr::device_cus() > 0 ? 2 * blr::device_cus() : 512; }
+
+extern "C" int blr_load_store_probe(const void* x, size_t x_bytes, const void* w1, size_t w1_bytes, const void* w2, size_t w2_bytes,
+                                    void* y, size_t y_bytes, void* dst, void* stream) {
+  if (!x || !w1 || !y || !dst || (w2_bytes && !w2)) { blr::set_error("load_store_probe: null pointer"); return BLR_ERR_BAD_ARG; }
+  if ((x_bytes | w1_bytes | w2_bytes | y_bytes) % 16 || !blr::aligned(x, 16) || !blr::aligned(w1, 16) || !blr::aligned(y, 16) ||
+      (w2 && !blr::aligned(w2, 16))) {
+    blr::set_error("load_store_probe: operands must be whole 16-byte pieces at 16-byte addresses");
+    return BLR_ERR_BAD_ARG;
+  }
+  const int grid = blr_probe_dst_words();
+  const blr::ProbeSrc s0 = {(const blr::u32x4*)x, x_bytes / 16}, s1 = {(const blr::u32x4*)w1, w1_bytes / 16},
+                      s2 = {(const blr::u32x4*)w2, w2 ? w2_bytes / 16 : 0};
+  hipLaunchKernelGGL(blr::load_store_probe_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, s0, s1, s2,
+                     (blr::u32x4*)y, y_bytes / 16, (uint32_t*)dst);
+  BLR_CHECK_LAUNCH("load_store_probe");
+  return BLR_OK;
+}
 
 extern "C" int blr_stream_probe(const void* src, size_t bytes, void* dst, void* stream) {
   if (!src || !dst || bytes < 16) { blr::set_error("probe: bad argument"); return BLR_ERR_BAD_ARG; }

@@ -54,6 +54,7 @@ _SIGNATURES = {
     "blr_blast_fwd_static": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64] + [_i] * 8 + [_vp]),
     "blr_probe_dst_words": (_i, []),
     "blr_stream_probe": (_i, [_vp, _sz, _vp, _vp]),
+    "blr_load_store_probe": (_i, [_vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp]),
 }
 
 _lib = None
@@ -156,6 +157,20 @@ def workspace(device, nbytes, algo=ALGO_AUTO, M=None, dtype=None):
         ws._blr_streaming = streaming
         _workspaces[key] = ws
     return ws
+
+
+def load_store_probe(x, w1, w2, out_f):
+    """The reference's *_load_store_* kernels: load x and the factors, store a zero (N, out_f) result; nothing is computed."""
+    require_gpu(x, w1)
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    y = torch.empty((x2.shape[0], out_f), device=x.device, dtype=x.dtype)
+    nb = lambda t: t.numel() * t.element_size()
+    if any(nb(t) % 16 or t.data_ptr() % 16 for t in (x2, w1, y) + ((w2,) if w2 is not None else ())):
+        raise BlrError("load_store probe: operands must be whole 16-byte pieces")
+    dst = torch.zeros(lib().blr_probe_dst_words(), dtype=torch.int32, device=x.device)
+    check(lib().blr_load_store_probe(x2.data_ptr(), nb(x2), w1.data_ptr(), nb(w1), w2.data_ptr() if w2 is not None else None,
+                                     nb(w2) if w2 is not None else 0, y.data_ptr(), nb(y), dst.data_ptr(), stream_ptr(x.device)), "load_store_probe")
+    return y
 
 
 def require_gpu(*tensors):

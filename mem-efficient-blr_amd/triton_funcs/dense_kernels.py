@@ -51,12 +51,8 @@ def triton_dense_fp16(x, w, config=None):
 
 
 def _probe(x, w):
-    """Stream W once with the decode kernels' load pattern; returns a (N, out_f) tensor of zeros."""
-    L.require_gpu(x, w)
-    lib = L.lib()
-    dst = torch.zeros(lib.blr_probe_dst_words(), dtype=torch.int32, device=w.device)
-    L.check(lib.blr_stream_probe(w.data_ptr(), w.numel() * w.element_size(), dst.data_ptr(), L.stream_ptr(w.device)), "probe")
-    return torch.zeros((x.reshape(-1, x.shape[-1]).shape[0], w.shape[1]), device=x.device, dtype=x.dtype)
+    """Load x and W, store a zero (N, out_f) result (reference triton_funcs/dense_kernels.py:150-227, 383-412)."""
+    return L.load_store_probe(x, w, None, w.shape[1])
 
 
 def triton_dense_load_store_fp32(x, w):

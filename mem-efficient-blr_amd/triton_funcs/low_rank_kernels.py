@@ -54,12 +54,8 @@ def triton_low_rank_fp16(x, a, b, config=None):
 
 
 def _probe(x, a, b):
-    L.require_gpu(x, a, b)
-    lib = L.lib()
-    dst = torch.zeros(lib.blr_probe_dst_words(), dtype=torch.int32, device=a.device)
-    for w in (a, b):
-        L.check(lib.blr_stream_probe(w.data_ptr(), w.numel() * w.element_size(), dst.data_ptr(), L.stream_ptr(w.device)), "probe")
-    return torch.zeros((x.reshape(-1, x.shape[-1]).shape[0], b.shape[1]), device=x.device, dtype=x.dtype)
+    """Load x, A and B, store a zero (N, out_f) result (reference triton_funcs/low_rank_kernels.py:163-236, 419-450)."""
+    return L.load_store_probe(x, a, b, b.shape[1])
 
 
 def triton_low_rank_load_store_fp32(x, a, b):
