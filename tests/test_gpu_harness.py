@@ -80,3 +80,24 @@ def test_dit_small_blast_matches_its_dense_assembly():
         ref = net(x, t, y).float()
     assert out.shape == (4, 8, 32, 32)
     assert (out - ref).abs().max() <= 2e-2 * ref.abs().max()
+
+
+def test_gpu_profile_traces_a_function_under_rocprofv3(tmp_path):
+    """The collection tool end to end: rocprofv3 --kernel-trace around the tool's own run mode (a child process), summary on disk."""
+    import shutil
+    import subprocess
+    import sys
+    if shutil.which("rocprofv3") is None:
+        pytest.skip("rocprofv3 is not on PATH")
+    pkg = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "mem-efficient-blr_amd")
+    say("[case] gpu_profile trace of triton_blast_full_fp16")
+    out = tmp_path / "prof"
+    cmd = [sys.executable, os.path.join(pkg, "gpu_profile.py"), "--mode", "trace", "--function_name", "triton_funcs.blast_kernels.triton_blast_full_fp16",
+           "--num_seq", "8", "--in_f", "1024", "--out_f", "1024", "--b", "16", "--rank", "128", "--num_iters", "6", "--num_warmup_iters", "2",
+           "--output_dir", str(out), "--timeout", "150"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=170, env=dict(os.environ, TMPDIR=str(tmp_path)))
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    text = (out / "triton_blast_full_fp16_kernels.txt").read_text()
+    rows = [ln for ln in text.splitlines() if "blr" in ln and "command:" not in ln]
+    assert rows, text
+    assert any(int(ln.split()[-4]) >= 8 for ln in rows), text          # 2 warm-up + 6 timed calls of at least one kernel

@@ -187,3 +187,25 @@ def test_get_config_is_picklable_and_none_before_use():
     from triton_funcs import blast_kernels as K
     assert K.get_triton_blast_partial_fp16_config() is None
     pickle.dumps(K.get_triton_blast_partial_fp16_config())
+
+
+def test_gpu_profile_summaries_from_rocprof_csv(tmp_path):
+    """The profile tool's readers of rocprofv3's csv files: per-kernel durations, counter means and the scale taken from a copy
+    of known size."""
+    import gpu_profile as G
+    kt = tmp_path / "kt_kernel_trace.csv"
+    kt.write_text('"Kind","Kernel_Name","Start_Timestamp","End_Timestamp","Workgroup_Size_X","Grid_Size_X","Grid_Size_Y","Grid_Size_Z"\n'
+                  '"KERNEL_DISPATCH","blr::a",1000,3000,256,1024,1,1\n'
+                  '"KERNEL_DISPATCH","blr::a",5000,9000,256,1024,1,1\n'
+                  '"KERNEL_DISPATCH","other",100,200,64,64,1,1\n')
+    s = G.summarize_kernel_trace(str(kt))
+    assert s[("blr::a", 1024, 256)] == {"calls": 2, "avg_us": 3.0, "min_us": 2.0, "max_us": 4.0}
+    assert "other" not in G.format_trace(s, only=["blr"]) and "blr::a" in G.format_trace(s, only=["blr"])
+    cc = tmp_path / "pmc_counter_collection.csv"
+    cc.write_text('"Dispatch_Id","Kernel_Name","Counter_Name","Counter_Value"\n'
+                  '1,"__amd_rocclr_copyBuffer","FETCH_SIZE",131072.0\n2,"__amd_rocclr_copyBuffer","FETCH_SIZE",131072.0\n'
+                  '3,"blr::a","FETCH_SIZE",1000.0\n4,"blr::a","FETCH_SIZE",3000.0\n')
+    c = G.summarize_counters(str(cc))
+    assert c[("blr::a", "FETCH_SIZE")] == {"dispatches": 2, "mean": 2000.0, "min": 1000.0, "max": 3000.0}
+    assert G.counter_unit_bytes(c, "FETCH_SIZE") == G.CALIB_BYTES / 131072.0
+    assert G.counter_unit_bytes(c, "WRITE_SIZE") is None
