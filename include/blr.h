@@ -51,8 +51,9 @@ typedef enum { BLR_S_JIR = 0, BLR_S_RIJ = 1, BLR_S_IJR = 2 } blr_s_layout;
 typedef enum {
   BLR_ALGO_AUTO = 0,
   BLR_ALGO_STREAM = 1,        /* persistent streaming kernel, one launch, M <= 16, f16/bf16 */
-  BLR_ALGO_TILED = 2,         /* MFMA tiled GEMMs with the rank-space intermediate in HBM   */
-  BLR_ALGO_FUSED = 3,         /* MFMA two-stage kernel, rank-space intermediate kept in LDS */
+  BLR_ALGO_TILED = 2,         /* MFMA tiled GEMMs; the rank-space intermediates go through HBM unless the fused first half pays */
+  BLR_ALGO_FUSED = 3,         /* BLAST: x V and the mix in one launch, Y = x V only ever in LDS; then the batched GEMM with U.
+                                 Needs f16/bf16, 4 | b <= 16, 8 | in_f / b, 8 | r, y_out == NULL; else BLR_ERR_UNSUPPORTED */
   BLR_ALGO_STREAM_SPLIT = 4   /* the STREAM phases as separate launches (no grid barrier)   */
 } blr_algo;
 

@@ -12,7 +12,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRC = ["blr_api.hip", "blr_gemm.hip", "blr_stream.hip", "blr_decode.hip", "blr_decode3.hip", "blr_decode_pair.hip", "blr_decode_rows.hip"]
+SRC = ["blr_api.hip", "blr_gemm.hip", "blr_stream.hip", "blr_decode.hip", "blr_decode3.hip", "blr_decode_pair.hip", "blr_decode_rows.hip", "blr_prefill.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-pass-failed", "-Wno-unused-function"]

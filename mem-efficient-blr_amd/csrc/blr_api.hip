@@ -281,7 +281,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
                        void* out, int64_t ldo, void* z_out, void* y_out,
                        int M, int in_f, int out_f, int b, int r,
                        int dtype, int u_layout, int s_layout, int sat8,
-                       void* ws, size_t ws_bytes, hipStream_t st) {
+                       void* ws, size_t ws_bytes, hipStream_t st, int fused = 0) {   // fused: 1 = must, 0 = where it applies, -1 = never
   const int P = in_f / b, Q = out_f / b;
   const size_t es = elt_size(dtype);
   const size_t ybytes = align_up((size_t)b * M * r * es, 256);
@@ -291,21 +291,32 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   void* Y = y_out ? y_out : (void*)wp; if (!y_out) wp += ybytes;
   void* Z = z_out ? z_out : (void*)wp;
 
-  GemmArgs g1 = {};
-  g1.A = x; g1.lda = ldx; g1.sA = P;
-  g1.B = V; g1.ldb = r; g1.sB = (int64_t)P * r; g1.b_kn = 1;
-  g1.C = Y; g1.ldc = r; g1.sC = (int64_t)M * r; g1.cn = 1;
-  g1.M = M; g1.N = r; g1.K = P; g1.batch = b;
-  g1.sat8 = sat8;
-  int rc = gemm_launch(g1, dtype, st);
-  if (rc) return rc;
-
   int64_t si, sj, sr;
   if (s_layout == BLR_S_JIR) { sj = (int64_t)b * r; si = r; sr = 1; }
   else if (s_layout == BLR_S_RIJ) { sr = (int64_t)b * b; si = b; sj = 1; }
   else { si = (int64_t)b * r; sj = r; sr = 1; }
-  rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st, sat8);
-  if (rc) return rc;
+  int rc = 1;
+  // Nobody asked for Y: x V and the mix can run as one launch with Y kept inside the compute units (BLR_ALGO_FUSED).  Chosen
+  // by itself only for narrow input blocks: the fused kernel re-reads V once per 32 rows, and from about 128 columns per
+  // block on that costs more than the round trip of Y it saves (measured at 4096 rows: 1152 -> 1152, r = 288: 64 against
+  // 68 us; 4608 -> 1152, r = 576: 154 against 122 us; Llama-7B gate_up at 2048 rows: 201 against 186 us).
+  static const int fuse_max_p = getenv("BLR_BLAST_FUSE_MAX_P") ? atoi(getenv("BLR_BLAST_FUSE_MAX_P")) : 128;
+  if (!y_out && !sat8 && fused >= 0 && (fused == 1 || P <= fuse_max_p))
+    rc = blast_ymix_launch(x, ldx, V, S, Z, M, in_f, b, r, si, sj, sr, s_layout, dtype, Y, ybytes, st);   // (the unused room of Y holds S transposed)
+  if (rc < 0) return rc;
+  if (rc == 1 && fused == 1) { set_error("blast: the fused kernel does not take this shape (b even and <= 16, block width and rank multiples of 8, f16/bf16)"); return BLR_ERR_UNSUPPORTED; }
+  if (rc == 1) {
+    GemmArgs g1 = {};
+    g1.A = x; g1.lda = ldx; g1.sA = P;
+    g1.B = V; g1.ldb = r; g1.sB = (int64_t)P * r; g1.b_kn = 1;
+    g1.C = Y; g1.ldc = r; g1.sC = (int64_t)M * r; g1.cn = 1;
+    g1.M = M; g1.N = r; g1.K = P; g1.batch = b;
+    g1.sat8 = sat8;
+    rc = gemm_launch(g1, dtype, st);
+    if (rc) return rc;
+    rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st, sat8);
+    if (rc) return rc;
+  }
 
   GemmArgs g2 = {};
   g2.A = Z; g2.lda = r; g2.sA = (int64_t)M * r;
@@ -352,8 +363,10 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
     s.ws = ws; s.ws_bytes = ws_bytes; s.split = (a == BLR_ALGO_STREAM_SPLIT);
     return stream_blast_launch(s, st);
   }
-  if (a != BLR_ALGO_TILED) { set_error("blast: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
-  return blast_tiled(x, ldx, U, V, S, out, ldo, z_out, y_out, M, in_f, out_f, b, r, dtype, u_layout, s_layout, 0, ws, ws_bytes, st);
+  if (a != BLR_ALGO_TILED && a != BLR_ALGO_FUSED) { set_error("blast: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
+  if (a == BLR_ALGO_FUSED && y_out) { set_error("blast: the fused algorithm never forms Y in memory (y_out must be null)"); return BLR_ERR_UNSUPPORTED; }
+  return blast_tiled(x, ldx, U, V, S, out, ldo, z_out, y_out, M, in_f, out_f, b, r, dtype, u_layout, s_layout, 0, ws, ws_bytes, st,
+                     a == BLR_ALGO_FUSED ? 1 : 0);
 }
 
 // ---- BLAST with int8-valued intermediates ----------------------------------------------------------

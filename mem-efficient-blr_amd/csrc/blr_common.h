@@ -128,6 +128,13 @@ size_t gemm_splitk_bytes(int M, int N, int K, int dtype);
 int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
                      int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, hipStream_t st, int sat8 = 0);
 
+// ---- BLAST above 16 rows: Z = mix(S, x V) in one launch, Y never written (blr_prefill.hip) ---------------
+// Z (b, M, R) of dtype.  Returns BLR_OK, a negative blr_status, or 1 when the shape is not for the kernel.
+// scratch: b * b * R elements for S in (r, i, j) order (not touched when S already has that layout).
+int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, void* Z, int M, int in_f, int b, int R,
+                      int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
+                      hipStream_t st);
+
 // ---- streaming (decode) engine (blr_stream.hip) -------------------------------------------
 struct StreamBlastArgs {
   const void* x; int64_t ldx;

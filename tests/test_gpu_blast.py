@@ -12,7 +12,7 @@ from gpu_util import assert_close, back, blast_inputs, dev, rounded, say
 
 pytestmark = pytest.mark.gpu
 
-ALGO = {"auto": 0, "stream": 1, "tiled": 2, "split": 4}
+ALGO = {"auto": 0, "stream": 1, "tiled": 2, "fused": 3, "split": 4}
 
 
 def _run_blast(fn_name, x, U, Vt, S, dtype, algo=None):
@@ -90,6 +90,34 @@ def test_blast_gpt2_config_fp32_and_fp16():
 
 
 LLAMA = {"qkvo": (256, 256, 512), "gate_up": (256, 1376, 1024), "down": (688, 256, 1024)}
+
+
+FUSED_SHAPES = [(16, 64, 72, 128, (96,)), (16, 72, 216, 288, (2, 75)), (4, 48, 24, 96, (37,)), (8, 256, 64, 200, (300,)),
+                (16, 688, 256, 1024, (64,)), (12, 16, 8, 40, (33,))]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("name", ["triton_blast_full_fp16", "triton_blast_bmm_fp16"])
+@pytest.mark.parametrize("shape", FUSED_SHAPES)
+def test_blast_fused_algorithm(name, shape, dtype):
+    """BLR_ALGO_FUSED: x V and the mix in one launch (Y only ever in LDS), then the batched product with U.  Row counts that
+    are not multiples of the 32-row tile, ranks that are not multiples of the 128-rank tile, k past a block's width, 4 to
+    16 blocks, S in both layouts."""
+    b, p, q, r, lead = shape
+    say(f"[case] fused {name} b={b} p={p} q={q} r={r} lead={lead} {dtype}")
+    x, U, Vt, S = blast_inputs(b, p, q, r, lead, seed=21)
+    out = _run_blast(name, x, U, Vt, S, dtype, "fused")
+    ref = _ref(x, U, Vt, S, dtype)[0]
+    assert_close(out, ref.reshape(tuple(out.shape)), dtype, f"fused {name}")
+    tiled = _run_blast(name, x, U, Vt, S, dtype, "tiled")
+    assert_close(out, back(tiled), dtype, f"fused against tiled {name}")
+
+
+def test_blast_fused_refuses_what_it_cannot_tile():
+    from triton_funcs import _lib as L
+    x, U, Vt, S = blast_inputs(2, 40, 24, 72, (5,), seed=22)              # two blocks: not a multiple of four
+    with pytest.raises(L.BlrError, match="fused"):
+        _run_blast("triton_blast_full_fp16", x, U, Vt, S, torch.float16, "fused")
 
 
 @pytest.mark.parametrize("M", [1, 4, 16])
