@@ -41,7 +41,7 @@ struct YmixParams {
   const void* V; const void* S; void* Z;
   int M, b, P, R;
   int npc;                      // 16-byte rank pieces of a tile (1..16): the tile spans BR = 8 npc ranks
-  int ksteps2;                  // pairs of 32-row k-steps that cover P
+  int ksteps;                   // 32-row k-steps that cover P
   FastDiv nmt;                  // row tiles
   const void* St;               // S as (r, i, j), the input block contiguous
 };
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
     const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.x), 0, p.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t vbuf = wbuf(reinterpret_cast<const T*>(p.V) + (int64_t)(2 * wv) * P * R, (uint32_t)((int64_t)2 * P * R * 2));
     const bool live = n < p.npc && r0 + n * 8 < R;
-    const int KS = 2 * p.ksteps2;
+    const int KS = p.ksteps;                                // 32-row steps per input block
     uint32_t h0[2][4][4];                                   // Y of the wave's first input block, packed two ranks to a dword
     f32x4 acc[2][8];
 #pragma unroll
@@ -145,24 +145,26 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
         for (int mg = 0; mg < 2; ++mg) acc[mg][e] = YmDot<T>::mfma(a[mg], bv, acc[mg][e]);
       }
     };
+    auto next_block = [&]() {                                // pack away the first block's Y, start the second from zero
+#pragma unroll
+      for (int mg = 0; mg < 2; ++mg)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) h0[mg][t][q] = ym_pack<T>(acc[mg][2 * q][t], acc[mg][2 * q + 1][t]);
+#pragma unroll
+      for (int mg = 0; mg < 2; ++mg)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[mg][e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    };
     load_ab(a0, b0, 0);
     TR6(1);
-    for (int pi = 0; pi < KS; ++pi) {                        // pairs of steps; the block changes at pi == ksteps2
-      if (pi == p.ksteps2) {
-#pragma unroll
-        for (int mg = 0; mg < 2; ++mg)
-#pragma unroll
-          for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) h0[mg][t][q] = ym_pack<T>(acc[mg][2 * q][t], acc[mg][2 * q + 1][t]);
-#pragma unroll
-        for (int mg = 0; mg < 2; ++mg)
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[mg][e] = f32x4{0.f, 0.f, 0.f, 0.f};
-      }
-      load_ab(a1, b1, 2 * pi + 1);
+    for (int q = 0; q < 2 * KS; q += 2) {                    // two steps per trip (the two register sets take turns)
+      if (q == KS) next_block();
+      load_ab(a1, b1, q + 1);
       step(a0, b0);
-      load_ab(a0, b0, 2 * pi + 2);
+      if (q + 1 == KS) next_block();
+      load_ab(a0, b0, q + 2);
       step(a1, b1);
     }
     TR6(2);
@@ -260,7 +262,7 @@ int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, 
   const int nrt = (int)cdiv(pieces, p.npc), nmt = (int)cdiv(M, YM_BM);
   if ((int64_t)nrt * nmt >= 65536 || nmt >= 65536) return 1;
   p.nmt = fd_make((uint32_t)nmt);
-  p.ksteps2 = (int)cdiv(cdiv(P, 32), 2);
+  p.ksteps = (int)cdiv(P, 32);
   if (s_layout == BLR_S_RIJ && aligned(S, 8)) {
     p.St = S;
   } else {

@@ -17,7 +17,8 @@ from utils import replace_linear_with_custom
 
 
 def modulate(x, shift, scale):
-    return x * (1 + scale.unsqueeze(1)) + shift.unsqueeze(1)
+    """x * (1 + scale) + shift (reference DiT/models.py:19-20) as one pass over x."""
+    return torch.addcmul(shift.unsqueeze(1), x, (1 + scale).unsqueeze(1))
 
 
 class TimestepEmbedder(nn.Module):
@@ -73,8 +74,9 @@ class DiTBlock(nn.Module):
 
     def forward(self, x, c):
         s1, c1, g1, s2, c2, g2 = self.adaLN_modulation(c).chunk(6, dim=1)
-        x = x + g1.unsqueeze(1) * self.attn(modulate(self.norm1(x), s1, c1))
-        x = x + g2.unsqueeze(1) * self.mlp(modulate(self.norm2(x), s2, c2))
+        # gate and residual (reference DiT/models.py:120-121) in one elementwise pass each
+        x = torch.addcmul(x, g1.unsqueeze(1), self.attn(modulate(self.norm1(x), s1, c1)))
+        x = torch.addcmul(x, g2.unsqueeze(1), self.mlp(modulate(self.norm2(x), s2, c2)))
         return x
 
 

@@ -69,17 +69,71 @@ def test_dit_small_blast_matches_its_dense_assembly():
     t = torch.randint(0, 1000, (4,), device="cuda"); y = torch.randint(0, 1000, (4,), device="cuda")
     with torch.no_grad():
         out = net(x, t, y).float()
+        say("  replays equal the eager forward; assembling the dense matrices")
+
+        def assemble(bl):                                   # W[(i,q),(j,p)] = sum_r U[i,q,r] S[r,i,j] V[j,p,r], fp32 on the GPU
+            W = torch.einsum("iqr,rij,jpr->iqjp", bl.U.float(), bl.S.float(), bl.V.float())
+            return W.reshape(bl.out_features, bl.in_features)
+
+        first = net.model.blocks[0].attn.proj                # the einsum against the oracle's assembly, once
+        S0 = first.S.detach().double().cpu().numpy().transpose(1, 2, 0)            # (r,i,j) -> (i,j,r)
+        W0 = O.blast_dense_weight(first.U.detach().double().cpu().numpy(), first.V.detach().double().cpu().numpy().transpose(0, 2, 1), S0)
+        assert np.abs(assemble(first).double().cpu().numpy() - W0).max() <= 1e-4 * np.abs(W0).max()
         for blk in net.model.blocks:
             for parent, name in ((blk.attn, "qkv"), (blk.attn, "proj"), (blk.mlp, "fc1"), (blk.mlp, "fc2")):
                 bl = getattr(parent, name)
-                S = bl.S.detach().double().cpu().numpy().transpose(1, 2, 0)            # (r,i,j) -> (i,j,r)
-                W = O.blast_dense_weight(bl.U.detach().double().cpu().numpy(), bl.V.detach().double().cpu().numpy().transpose(0, 2, 1), S)
                 lin = torch.nn.Linear(bl.in_features, bl.out_features).cuda().half()
-                lin.weight.copy_(torch.from_numpy(W)); lin.bias.copy_(bl.bias)
+                lin.weight.copy_(assemble(bl)); lin.bias.copy_(bl.bias)
                 setattr(parent, name, lin)
+        say("  dense forward")
         ref = net(x, t, y).float()
     assert out.shape == (4, 8, 32, 32)
     assert (out - ref).abs().max() <= 2e-2 * ref.abs().max()
+
+
+def test_dit_full_depth_graph_replay_is_finite_and_matches_dense_assembly():
+    """BASELINE config 5 at full size - 28 blocks, 16 latents of 256 tokens, every block linear a BLAST layer - run the way the
+    benchmark runs it (a captured forward, replayed): every replay equals the eager forward bit for bit, the output is finite,
+    and it agrees with the same network after each BLAST layer has been replaced by its assembled dense matrix."""
+    from models.dit_xl import CustomDiT, capture_forward
+    torch.manual_seed(0)
+    cfg = {k: {"rank": r, "b": 16, "func": "triton_funcs.blast_kernels.triton_blast_bmm_fp16"}
+           for k, r in (("attn.qkv", 288), ("attn.proj", 288), ("mlp.fc1", 576), ("mlp.fc2", 576))}
+    say("[case] DiT-XL/2 depth 28 batch 16, BLAST, graph replay")
+    net = CustomDiT(layer_configs=cfg, method="blast", depth=28)
+    assert net.replaced == 112
+    x = torch.randn(16, 4, 32, 32, device="cuda", dtype=torch.float16)
+    t = torch.randint(0, 1000, (16,), device="cuda"); y = torch.randint(0, 1000, (16,), device="cuda")
+    with torch.no_grad():
+        eager = net(x, t, y).clone()
+        g, out = capture_forward(net, x, t, y, warmup=1)
+        for rep in range(3):
+            out.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"replay {rep} differs from the eager forward"
+        assert eager.shape == (16, 8, 32, 32) and torch.isfinite(eager).all()
+        say("  replays equal the eager forward; assembling the dense matrices")
+
+        def assemble(bl):                                   # W[(i,q),(j,p)] = sum_r U[i,q,r] S[r,i,j] V[j,p,r], fp32 on the GPU
+            W = torch.einsum("iqr,rij,jpr->iqjp", bl.U.float(), bl.S.float(), bl.V.float())
+            return W.reshape(bl.out_features, bl.in_features)
+
+        first = net.model.blocks[0].attn.proj                # the einsum against the oracle's assembly, once
+        S0 = first.S.detach().double().cpu().numpy().transpose(1, 2, 0)            # (r,i,j) -> (i,j,r)
+        W0 = O.blast_dense_weight(first.U.detach().double().cpu().numpy(), first.V.detach().double().cpu().numpy().transpose(0, 2, 1), S0)
+        assert np.abs(assemble(first).double().cpu().numpy() - W0).max() <= 1e-4 * np.abs(W0).max()
+        for blk in net.model.blocks:
+            for parent, name in ((blk.attn, "qkv"), (blk.attn, "proj"), (blk.mlp, "fc1"), (blk.mlp, "fc2")):
+                bl = getattr(parent, name)
+                lin = torch.nn.Linear(bl.in_features, bl.out_features).cuda().half()
+                lin.weight.copy_(assemble(bl)); lin.bias.copy_(bl.bias)
+                setattr(parent, name, lin)
+        say("  dense forward")
+        ref = net(x, t, y).float()
+    err = (eager.float() - ref).abs().max().item()
+    say(f"  max |blast - dense assembly| = {err:.4g} of max |ref| = {ref.abs().max().item():.4g}")
+    assert err <= 5e-2 * ref.abs().max().item()          # 28 blocks of fp16 rounding on both sides
 
 
 def test_gpu_profile_traces_a_function_under_rocprofv3(tmp_path):
