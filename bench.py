@@ -33,9 +33,20 @@ MFMA_PEAK = 2.5e15           # FLOP/s, dense fp16/bf16
 LAYERS = {"qkvo": (4096, 4096, 512), "gate_up": (4096, 22016, 1024), "down": (11008, 4096, 1024)}
 B = 16
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE), scaled
-# by the same counters over a copy kernel of known size (1 FETCH_SIZE unit = 1.99978 KiB, 1 WRITE_SIZE unit = 1 KiB).
-TRAFFIC_BYTES = 70.86e6   # 70.36 MB fetched + 0.50 MB written (profiles/decode2_kernel_blast_llama7b_decode_m1.txt)
+# HBM bytes per launch of the dominant kernel come from the committed counter summary (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+# scaled by the same counters over a copy of known size): the line "traffic_bytes_per_launch: N" of this file.  No file, no figure.
+DOMINANT_KERNEL = "decode3_kernel<f16,1,16>"
+DOMINANT_PROFILE = os.path.join("profiles", "decode3_kernel_blast_llama7b_gate_up_m1.txt")
+
+
+def traffic_from_profile(path):
+    try:
+        for line in open(os.path.join(ROOT, path)):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def blast_bytes_flops(n, i, r, o, b=B, elt=2):
@@ -239,13 +250,20 @@ def main():
         one.append(mk_blast(M, *LAYERS["gate_up"][:2], LAYERS["gate_up"][2], L.U_RQ, L.S_JIR))
         one.append(mk_blast(M, *LAYERS["down"][:2], LAYERS["down"][2], L.U_RQ, L.S_JIR))
         sets.append(one)
+    # One graph per weight copy (one step each) and one graph that runs a step on every copy in turn: the timed region
+    # replays the long graph steps // ncopies times and finishes the remainder with single-step graphs - exactly `steps`
+    # steps, with the host out of the way between most of them.
     step_graphs = [graph_of([go for go, _ in one]) for one in sets]
+    round_graph = graph_of([go for one in sets for go, _ in one])
     for s in range(args.warmup):
         step_graphs[s % ncopies].replay()
+    round_graph.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for s in range(args.steps):
-        step_graphs[s % ncopies].replay()
+    for _ in range(args.steps // ncopies):
+        round_graph.replay()
+    for s in range(args.steps % ncopies):
+        step_graphs[s].replay()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / max(args.steps, 1)
@@ -257,10 +275,24 @@ def main():
     gu_us = time_graph(g_gu, n_l)
     gu_bytes, gu_flops = blast_bytes_flops(M, LAYERS["gate_up"][0], LAYERS["gate_up"][2], LAYERS["gate_up"][1])
     achieved = gu_bytes / (gu_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "decode2_kernel<f16,1> (BLAST gate_up 4096->22016 r=1024 b=16, M=1)",
+    roofline = {"bound": "hbm", "kernel": DOMINANT_KERNEL + " (BLAST gate_up 4096->22016 r=1024 b=16, M=1: one launch, all of V, S and U)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": round(achieved * 1e9 / HBM_PEAK, 4),
-                "us_per_launch": round(gu_us, 3), "algorithmic_bytes": gu_bytes, "traffic": TRAFFIC_BYTES}
-    del g_gu, step_graphs, sets
+                "us_per_launch": round(gu_us, 3), "algorithmic_bytes": gu_bytes, "traffic": traffic_from_profile(DOMINANT_PROFILE),
+                "traffic_source": DOMINANT_PROFILE}
+    del g_gu, step_graphs, round_graph, sets
+    torch.cuda.empty_cache()
+
+    # second roofline object: the dominant kernel at M = 2048, the ring GEMM (one launch = the dense gate_up layer), MFMA bound
+    i_f, o_f, _ = LAYERS["gate_up"]
+    dn = [mk_dense(2048, i_f, o_f) for _ in range(3)]
+    g_dn = graph_of([dn[i % 3][0] for i in range(12)])
+    dn_us = time_graph(g_dn, 12)
+    dn_flops = 2.0 * 2048 * i_f * o_f
+    roofline_prefill = {"bound": "mfma", "kernel": "gemm_ring_kernel<f16, 256x256> (dense gate_up 4096->22016, M=2048: one launch)",
+                        "achieved": round(dn_flops / (dn_us * 1e-6) / 1e12, 1), "peak": MFMA_PEAK / 1e12, "unit": "TFLOP/s",
+                        "frac": round(dn_flops / (dn_us * 1e-6) / MFMA_PEAK, 4), "us_per_launch": round(dn_us, 2),
+                        "algorithmic_flops": dn_flops, "traffic": None}
+    del g_dn, dn
     torch.cuda.empty_cache()
 
     # ---- per-layer table ----------------------------------------------------------------------------
@@ -336,6 +368,40 @@ def main():
         cpu = {"value": round(times[len(times) // 2] * 1e6, 1), "unit": "us/layer-step", "cores": cores, "kind": "port",
                "sample": f"{reps} repetitions (~{t_used:.0f} s) of the full M=1 step (6 BLAST linears) in fp32 with oracle/torch_port.blast"}
 
+    # ---- BASELINE configs[0]: the reference's own CPU-runnable case (GPT-2-small c_fc, fp32) on the host and on the GPU ---------
+    cpu1 = None
+    if not args.no_cpu:
+        from oracle import torch_port as T
+        g = torch.Generator().manual_seed(0)
+        b1, r1, i1, o1 = 4, 128, 768, 3072
+        x1 = torch.randn(1, 128, i1, generator=g)
+        U1 = torch.randn(b1, o1 // b1, r1, generator=g) * r1 ** -0.5
+        V1 = torch.randn(b1, r1, i1 // b1, generator=g) * r1 ** -0.5
+        S1 = torch.randn(b1, b1, r1, generator=g)
+        for _ in range(5):
+            T.blast(x1, U1, V1, S1)
+        reps, t_used, times = 0, 0.0, []
+        while t_used < 5.0 and reps < 20000:
+            c0 = time.perf_counter()
+            T.blast(x1, U1, V1, S1)
+            dt = time.perf_counter() - c0
+            times.append(dt); t_used += dt; reps += 1
+        times.sort()
+        from triton_funcs import blast_kernels as K
+        xg = x1.to(dev)
+        Ug, Vg, Sg = (U1.permute(0, 2, 1).contiguous().to(dev), V1.permute(0, 2, 1).contiguous().to(dev), S1.permute(1, 0, 2).contiguous().to(dev))
+        for _ in range(3):
+            K.triton_blast_full_fp32(xg, Ug, Vg, Sg)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(50):
+            K.triton_blast_full_fp32(xg, Ug, Vg, Sg)
+        e1.record(); torch.cuda.synchronize()
+        cpu1 = {"value": round(times[len(times) // 2] * 1e6, 1), "unit": "us/forward", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{reps} repetitions (~{t_used:.0f} s) of BLAST c_fc x[1,128,768] -> 3072, b=4, r=128, fp32, oracle/torch_port.blast",
+                "gpu_us": round(e0.elapsed_time(e1) * 1e3 / 50, 1), "gpu_path": "triton_blast_full_fp32 (eager calls, intermediates returned)"}
+
     result = {
         "metric": "Llama-7B layer us + %HBM/%MFMA roofline at M=1 and 2048; DiT-XL/2 img/s",
         "value": round(ms_per_step * 1e3, 2), "unit": "us/layer-step (6 BLAST linears, M=1)",
@@ -345,7 +411,8 @@ def main():
                                "triton_blast_full_fp16 layouts, HIP-graph replay, weight copies rotated past the Infinity Cache",
                    "weight_copies": ncopies, "algorithmic_bytes_per_step": step_bytes,
                    "pct_hbm_step": round(100 * step_bytes / (ms_per_step * 1e-3) / HBM_PEAK, 1)},
-        "roofline": roofline, "cpu_baseline": cpu, "layers": table, "dit_xl": dit,
+        "roofline": roofline, "roofline_prefill": roofline_prefill, "cpu_baseline": cpu, "cpu_baseline_config1": cpu1,
+        "layers": table, "dit_xl": dit,
     }
     print(json.dumps(result))
 

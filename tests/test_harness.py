@@ -209,3 +209,18 @@ def test_gpu_profile_summaries_from_rocprof_csv(tmp_path):
     assert c[("blr::a", "FETCH_SIZE")] == {"dispatches": 2, "mean": 2000.0, "min": 1000.0, "max": 3000.0}
     assert G.counter_unit_bytes(c, "FETCH_SIZE") == G.CALIB_BYTES / 131072.0
     assert G.counter_unit_bytes(c, "WRITE_SIZE") is None
+
+
+def test_bench_takes_roofline_traffic_from_the_committed_profile():
+    """bench.py's roofline.traffic is read from the counter summary under profiles/, not typed into the script."""
+    import importlib.util
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_mod", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec); spec.loader.exec_module(bench)
+    assert os.path.exists(os.path.join(root, bench.DOMINANT_PROFILE))
+    t = bench.traffic_from_profile(bench.DOMINANT_PROFILE)
+    algorithmic = bench.blast_bytes_flops(1, 4096, 1024, 22016)[0]
+    assert t is not None and algorithmic <= t <= 1.5 * algorithmic
+    assert bench.traffic_from_profile("profiles/no_such_file.txt") is None
+    text = open(os.path.join(root, bench.DOMINANT_PROFILE)).read()
+    assert bench.DOMINANT_KERNEL.split("<")[0] in text
