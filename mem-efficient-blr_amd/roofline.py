@@ -2,8 +2,10 @@
 
 Every `<function stem>_mem_flops` below is looked up by name from the function list of a Layer,
 exactly as the reference does (roofline.py:136-142): the stem is the function name without its
-trailing `_fp16` / `_fp32`.  Formulas follow roofline.py:7-99; the names that run this library's
-fused kernels are charged the fused traffic (every operand touched once).
+trailing `_fp16` / `_fp32`.  The formulas are the reference's, name by name (roofline.py:7-99), so a
+table made here is comparable with one made there: a name whose reference kernel writes an
+intermediate to memory is charged for it even though this library's kernel for that name may not
+(`library_mem_flops` gives the bytes this library's kernels are designed to move: every operand once).
 """
 import os
 
@@ -11,54 +13,95 @@ import numpy as np
 from tabulate import tabulate
 
 
-# ---- low rank / dense -------------------------------------------------------------------------
+# ---- low rank / dense (reference roofline.py:7-29) -----------------------------------------------------
 def torch_low_rank_baseline_mem_flops(n, i, r, o, e):
-    return (n * i + i * r + 2 * n * r + r * o + n * o) * e, 2 * n * r * (i + o)
+    return (n * i + i * r + n * r + r * o + n * r + n * o) * e, n * r * (i + o) * 2
 
 
 def triton_low_rank_mem_flops(n, i, r, o, e):
-    return (i * r + r * o + n * o + n * i) * e, 2 * n * r * (i + o)
+    return (i * r + r * o + n * o + n * i) * e, n * r * (i + o) * 2
 
 
 def torch_dense_baseline_mem_flops(n, i, o, e):
-    return (n * i + i * o + n * o) * e, 2 * n * i * o
+    return (n * i + i * o + n * o) * e, n * i * o * 2
 
 
-triton_dense_mem_flops = torch_dense_baseline_mem_flops
+def triton_dense_mem_flops(n, i, o, e):
+    return torch_dense_baseline_mem_flops(n, i, o, e)
 
 
-# ---- BLAST ----------------------------------------------------------------------------------------
+# ---- BLAST (reference roofline.py:31-71) -------------------------------------------------------------------
 def torch_blast_baseline_mem_flops(n, i, r, o, b1, b2, e):
-    return (n * i + b1 * b2 * r + i * r + 4 * b2 * n * r + 4 * b1 * n * r + r * o + n * o) * e, 2 * n * r * (i + o + b1 * b2)
+    return (n * i + b1 * b2 * r + i * r + 4 * b2 * n * r + 4 * b1 * n * r + r * o + n * o) * e, n * r * (i + o + b1 * b2) * 2
+
+
+def triton_blast_partial_mem_flops(n, i, r, o, b1, b2, e):
+    return (n * i + b1 * b2 * r + i * r + 2 * b2 * n * r + r * o + n * o) * e, n * r * (i + o + b1 * b2) * 2
+
+
+def triton_blast_bmm_int8_mem_flops(n, i, r, o, b1, b2, e):
+    """The reference's int8 name: factors at e bytes, the rank-space intermediates as int8 (roofline.py:46-51)."""
+    return (n * i + b1 * b2 * r + i * r + r * o + n * o) * e + 2 * b2 * n * r, n * r * (i + o + b1 * b2) * 2
+
+
+def triton_blast_partial_grouped_mem_flops(n, i, r, o, b1, b2, e):
+    return triton_blast_partial_mem_flops(n, i, r, o, b1, b2, e)
+
+
+def triton_blast_partial_grouped_persistent_mem_flops(n, i, r, o, b1, b2, e):
+    return triton_blast_partial_mem_flops(n, i, r, o, b1, b2, e)
 
 
 def triton_blast_full_mem_flops(n, i, r, o, b1, b2, e):
-    return (n * i + b1 * b2 * r + i * r + r * o + n * o) * e, 2 * n * r * (i + o + b1 * b2)
+    return (n * i + b1 * b2 * r + i * r + r * o + n * o) * e, n * r * (i + o + b1 * b2) * 2
 
 
-# all BLAST names of this library run the same kernels: one pass over the factors
-triton_blast_partial_mem_flops = triton_blast_full_mem_flops
-triton_blast_partial_grouped_mem_flops = triton_blast_full_mem_flops
-triton_blast_partial_grouped_persistent_mem_flops = triton_blast_full_mem_flops
-triton_blast_bmm_mem_flops = triton_blast_full_mem_flops
+def triton_blast_bmm_mem_flops(n, i, r, o, b1, b2, e):
+    return (n * i + b1 * b2 * r + i * r + 2 * b2 * n * r + 2 * b1 * n * r + r * o + n * o) * e, n * r * (i + o + b1 * b2) * 2
 
 
-def triton_blast_bmm_int8_mem_flops(n, i, r, o, b1, b2, e, bits=8):
-    """Weight-quantized BLAST: codes at bits/8 bytes, S / scales / activations at e bytes."""
-    return r * (i + o) * bits // 8 + e * (b1 * b2 * r + o + b1 * r + n * (i + o)), 2 * n * r * (i + o + b1 * b2)
+def blast_weight_quant_mem_flops(n, i, r, o, b1, b2, e, bits):
+    """Weight-quantized BLAST of this library (no reference counterpart): codes at bits / 8 bytes; S, the per-channel
+    scales of U (o values) and V (b1 r values) and the activations at e bytes."""
+    return r * (i + o) * bits // 8 + e * (b1 * b2 * r + o + b1 * r + n * (i + o)), n * r * (i + o + b1 * b2) * 2
 
 
-# ---- Monarch ----------------------------------------------------------------------------------------
-def torch_monarch_baseline_mem_flops(n, i, r, o, b, e):
-    return (n * i + i * r + 4 * b * n * r + r * o + 3 * n * o) * e, 2 * n * r * (i + o)
+def triton_blast_bmm_int4_mem_flops(n, i, r, o, b1, b2, e):
+    """triton_blast_bmm_int4_fp16 exists only with packed 4-bit factors."""
+    return blast_weight_quant_mem_flops(n, i, r, o, b1, b2, e, 4)
 
 
+# ---- Monarch (reference roofline.py:73-99) ------------------------------------------------------------------
 def triton_monarch_right_mem_flops(n, i, r, o, b, e):
-    return (n * i + i * r + r * o + n * o) * e, 2 * n * r * (i + o)
+    return (n * i + i * r + 2 * b * n * r + r * o + n * o + 2 * n * o) * e, n * r * (i + o) * 2
 
 
-triton_monarch_right_ideal_mem_flops = triton_monarch_right_mem_flops
-triton_monarch_right_left_mem_flops = triton_monarch_right_mem_flops
+def triton_monarch_right_ideal_mem_flops(n, i, r, o, b, e):
+    return (n * i + i * r + 2 * b * n * r + r * o + n * o) * e, n * r * (i + o) * 2
+
+
+def triton_monarch_right_left_mem_flops(n, i, r, o, b, e):
+    return triton_monarch_right_ideal_mem_flops(n, i, r, o, b, e)
+
+
+def torch_monarch_baseline_mem_flops(n, i, r, o, b, e):
+    return (n * i + i * r + 2 * b * n * r + 2 * b * n * r + r * o + n * o + 2 * n * o) * e, n * r * (i + o) * 2
+
+
+def library_mem_flops(function_name, layer, n, elt=2):
+    """(bytes, flops) with every operand moved once - what this library's kernels for `function_name` aim at."""
+    i, o = layer.in_f, layer.out_f
+    if "dense" in function_name:
+        return torch_dense_baseline_mem_flops(n, i, o, elt)
+    if "low_rank" in function_name:
+        return triton_low_rank_mem_flops(n, i, layer.low_rank["rank"], o, elt)
+    if "blast" in function_name:
+        r, b = layer.blast["rank"], layer.blast["b"]
+        if "int4" in function_name:
+            return blast_weight_quant_mem_flops(n, i, r, o, b, b, elt, 4)
+        return triton_blast_full_mem_flops(n, i, r, o, b, b, elt)
+    r = layer.monarch["rank"]
+    return (n * i + i * r + r * o + n * o) * elt, n * r * (i + o) * 2
 
 
 def mem_flops_for(function_name, layer, n, elt=2):

@@ -224,3 +224,36 @@ def test_bench_takes_roofline_traffic_from_the_committed_profile():
     assert bench.traffic_from_profile("profiles/no_such_file.txt") is None
     text = open(os.path.join(root, bench.DOMINANT_PROFILE)).read()
     assert bench.DOMINANT_KERNEL.split("<")[0] in text
+
+
+def test_roofline_formulas_are_the_references_name_by_name():
+    """Hand-evaluated values of the reference's formulas (roofline.py:7-99) at n=2, i=8, r=4, o=12, b1=b2=b=2, 2 bytes per element."""
+    import roofline as R
+    n, i, r, o, b, e = 2, 8, 4, 12, 2, 2
+    assert R.torch_low_rank_baseline_mem_flops(n, i, r, o, e) == (272, 320)
+    assert R.triton_low_rank_mem_flops(n, i, r, o, e) == (240, 320)
+    assert R.torch_dense_baseline_mem_flops(n, i, o, e) == R.triton_dense_mem_flops(n, i, o, e) == (272, 384)
+    assert R.torch_blast_baseline_mem_flops(n, i, r, o, b, b, e) == (528, 384)
+    assert R.triton_blast_partial_mem_flops(n, i, r, o, b, b, e) == (336, 384)
+    assert R.triton_blast_partial_grouped_mem_flops(n, i, r, o, b, b, e) == (336, 384)
+    assert R.triton_blast_partial_grouped_persistent_mem_flops(n, i, r, o, b, b, e) == (336, 384)
+    assert R.triton_blast_bmm_int8_mem_flops(n, i, r, o, b, b, e) == (304, 384)
+    assert R.triton_blast_full_mem_flops(n, i, r, o, b, b, e) == (272, 384)
+    assert R.triton_blast_bmm_mem_flops(n, i, r, o, b, b, e) == (400, 384)
+    assert R.triton_monarch_right_mem_flops(n, i, r, o, b, e) == (400, 320)
+    assert R.triton_monarch_right_ideal_mem_flops(n, i, r, o, b, e) == R.triton_monarch_right_left_mem_flops(n, i, r, o, b, e) == (304, 320)
+    assert R.torch_monarch_baseline_mem_flops(n, i, r, o, b, e) == (464, 320)
+    # weight-quantized BLAST (this library's own): codes r (i + o) bits / 8, the rest at e bytes
+    assert R.triton_blast_bmm_int4_mem_flops(n, i, r, o, b, b, e) == (4 * 20 // 2 + 2 * (16 + 12 + 8 + 2 * 20), 384)
+
+
+def test_every_exported_operator_name_has_a_roofline_formula():
+    import importlib
+    import roofline as R
+    for mod in ("blast_kernels", "blast_sym_quant_kernels", "monarch_kernels", "low_rank_kernels", "dense_kernels"):
+        m = importlib.import_module(f"triton_funcs.{mod}")
+        for name in m.__all__:
+            if not name.startswith("triton_") or "load_store" in name:
+                continue
+            stem = name.rsplit("_", 1)[0]
+            assert hasattr(R, f"{stem}_mem_flops"), f"{name}: no {stem}_mem_flops in roofline.py"
