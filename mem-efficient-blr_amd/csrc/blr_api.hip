@@ -414,8 +414,11 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   if (dtype != BLR_F16 && dtype != BLR_BF16) { set_error("blast_q: dtype must be f16 or bf16"); return BLR_ERR_UNSUPPORTED; }
   int rc = check_blast_shape("blast_q", M, in_f, out_f, b, r);
   if (rc) return rc;
-  if (r % 32) { set_error("blast_q: r=%d must be a multiple of 32", r); return BLR_ERR_BAD_SHAPE; }
+  if (r % 8) { set_error("blast_q: r=%d must be a multiple of 8", r); return BLR_ERR_BAD_SHAPE; }
   if ((out_f / b) % 8) { set_error("blast_q: out_f / b = %d must be a multiple of 8", out_f / b); return BLR_ERR_BAD_SHAPE; }
+  // rows of codes that are not whole 16-byte pieces (r = 1488 at 4 bits: 744 bytes) are served by the three-launch path only,
+  // whose lanes fetch 8 columns (8 or 4 bytes) at a time
+  const bool whole16 = ((int64_t)r * bits) % 128 == 0 && ((int64_t)(out_f / b) * bits) % 128 == 0;
   if (ldx < in_f || ldo < out_f) { set_error("blast_q: leading dimension too small"); return BLR_ERR_BAD_ARG; }
   if (!aligned(u_codes, 16) || !aligned(v_codes, 16)) { set_error("blast_q: code buffers must be 16-byte aligned"); return BLR_ERR_BAD_ARG; }
   hipStream_t st = (hipStream_t)stream;
@@ -424,7 +427,7 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   // codes at 5..16 rows go to the matrix-core decode kernel as they are (it widens them in registers)
   static const bool i8_direct = !getenv("BLR_Q_DIRECT") || atoi(getenv("BLR_Q_DIRECT")) != 0;
   const bool direct = M <= 16 && i8_direct;
-  if (M > 4 && !phase_engine && !direct) {
+  if ((M > 16 || (M > 4 && !phase_engine && !direct)) && !(M <= 16 && !whole16)) {
     size_t need = blr_blast_q_workspace_bytes(M, in_f, out_f, b, r, bits);
     if (!ws || ws_bytes < need) { set_error("blast_q: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
     const size_t sub = align_up(M <= 16 ? stream_blast_workspace(M, in_f, out_f, b, r, bits) : 2 * align_up((size_t)b * M * r * 2, 256), 256);
@@ -449,6 +452,7 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   s.out = out; s.ldo = ldo; s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
   s.dtype = dtype; s.u_layout = BLR_U_RQ; s.s_layout = BLR_S_RIJ; s.wbits = bits;
   s.ws = ws; s.ws_bytes = ws_bytes; s.split = (algo == BLR_ALGO_STREAM_SPLIT);
+  s.rows_only = whole16 ? 0 : 1;
   return stream_blast_launch(s, st);
 }
 

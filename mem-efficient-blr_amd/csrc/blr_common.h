@@ -149,6 +149,7 @@ struct StreamBlastArgs {
   int wbits;                                    // 16 = floating weights, 8 / 4 = codes
   void* ws; size_t ws_bytes;
   int split;                                    // 1: separate launches per phase
+  int rows_only;                                // 1: only the three-launch matrix-core path may serve the call (codes whose rows are not whole 16-byte pieces)
 };
 size_t stream_blast_workspace(int M, int in_f, int out_f, int b, int r, int wbits);
 size_t stream_ws_prefix_bytes();                // the fixed-place block at the start of a streaming workspace; per-call scratch follows

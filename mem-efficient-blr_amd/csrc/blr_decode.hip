@@ -1345,10 +1345,11 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
   static const int rows_min_m = env_i("BLR_DECODE_ROWS_MIN_M", 2);
-  if (M >= rows_min_m || a.wbits == 4) {          // (4-bit codes at one row too: 15.8 against 16.9 - 20.6 us on the single-row kernels)
+  if (M >= rows_min_m || a.wbits == 4 || a.rows_only) {   // (4-bit codes at one row too: 15.8 against 16.9 - 20.6 us on the single-row kernels)
     const int rc = decode_rows_launch(a, region, decode2_region_bytes(), st);
     if (rc != 1) return rc;
   }
+  if (a.rows_only) { set_error("blast_q: code rows that are not whole 16-byte pieces need in_f / b, r and out_f / b to be multiples of 8 and at most 4096"); return BLR_ERR_UNSUPPORTED; }
   {
     int rc = decode_pair_launch(a, region, decode2_region_bytes(), st);
     if (rc != 1) return rc;

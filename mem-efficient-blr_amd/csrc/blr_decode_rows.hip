@@ -45,7 +45,8 @@ struct RowsParams {
   int ep;
   const f16* scales;                      // codes: the product's column n of entry bt is multiplied by scales[bt * N + n]; else null
   int M, K, N;
-  int kw;                                 // rows of a wave's share (a multiple of 32)
+  int kw;                                 // rows of a wave's share per round (a multiple of 32)
+  int rounds;                             // passes of the eight waves over the rows
   int npc;                                // 16-byte column pieces of a chunk (1..16)
   FastDiv nch;                            // chunks per batch entry
   uint32_t xcd_span;                      // items per XCD when the grid is a multiple of 8, else 0 (plain order)
@@ -155,7 +156,13 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   const bool live = NK ? true : (n < p.npc && colp < N);
   const __amdgpu_buffer_rsrc_t abuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.A), 0, p.a_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t wb = wbuf(reinterpret_cast<const char*>(p.W) + (int64_t)bt * p.w_bs * WB / 8, (uint32_t)((int64_t)K * N * WB / 8));
-  const int kb = wv * p.kw + 8 * g;                      // first of this lane's eight k of step 0
+  f32x4 acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // More than 8 waves x STEPS x 32 rows: the workgroup passes over the rows in rounds (the loads of a round are issued when
+  // the products of the one before are done - one more trip to memory per extra round).
+  for (int ro = 0; ro < p.rounds; ++ro) {
+  const int kb = (ro * DR_WAVES + wv) * p.kw + 8 * g;    // first of this lane's eight k of step 0
 
   // activations: row n of A, the lane's eight k of every step (16 bytes each); weights: eight rows per step, the lane's
   // 16-byte piece of each.  Lanes without a row / without a column piece issue nothing (their registers stay undefined:
@@ -199,9 +206,6 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   }
 
   TR5(1);
-  f32x4 acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     if constexpr (NK) {
@@ -221,6 +225,7 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
       }
     }
   }
+  }  // rounds
   TR5(2);
   if constexpr (NK) {
     // acc[e][t] is row 4 g + t, column col0 + 16 e + n
@@ -399,11 +404,12 @@ int rows_launch_t(RowsParams& p, int batch, hipStream_t st) {
 // One batch of skinny products; returns 1 when the operands do not fit the kernel.
 int rows_product(RowsParams p, int batch, int dtype, int wbits, bool nk, hipStream_t st) {
   if (nk && wbits != 16) return 1;
-  if (p.K % 8 || p.N % 8 || p.N > 65536 || p.K > DR_WAVES * DR_MAX_STEPS * 32) return 1;
+  if (p.K % 8 || p.N % 8 || p.N > 65536 || p.K > 4 * DR_WAVES * DR_MAX_STEPS * 32) return 1;
   if (!aligned(p.A, 16) || !aligned(p.W, 16) || p.lda % 8 || p.a_bs % 8 || p.w_bs % 32) return 1;
   if ((int64_t)p.K * p.N * 2 >= (int64_t)DR_OOB) return 1;
   if (wbits != 16 && dtype != BLR_F16 && dtype != BLR_BF16) return 1;
-  p.kw = (int)cdiv(cdiv(p.K, DR_WAVES), 32) * 32;
+  p.rounds = (int)cdiv(p.K, DR_WAVES * DR_MAX_STEPS * 32);
+  p.kw = (int)cdiv(cdiv(p.K, DR_WAVES * p.rounds), 32) * 32;
   const int cus = device_cus() > 0 ? device_cus() : 256;
   static const int e_npc = env_i("BLR_DR_NPC", 0);
   if (nk) {
@@ -458,7 +464,7 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   s2.o_bs = a.out_ns ? a.out_bs : Q; s2.o_ns = a.out_ns ? a.out_ns : 1;
   s2.M = M; s2.K = R; s2.N = Q; s2.trace_base = 512; s2.scales = a.wbits != 16 ? (const f16*)a.u_scales : nullptr;
   // both products must fit before the first launch
-  if (P % 8 || R % 8 || Q % 8 || P > 1024 || R > 1024 || !aligned(a.x, 16) || !aligned(a.V, 16) || !aligned(a.U, 16) || a.ldx % 8) return 1;
+  if (P % 8 || R % 8 || Q % 8 || P > 4096 || R > 4096 || !aligned(a.x, 16) || !aligned(a.V, 16) || !aligned(a.U, 16) || a.ldx % 8) return 1;
 
   const void* ep_bias = nullptr; int ep_act = 0;
   if (epilogue_pending(&ep_bias, &ep_act)) { s2.ep = 1; s2.bias = ep_bias; s2.act = ep_act; }

@@ -1218,10 +1218,11 @@ int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st) {
   size_t need = stream_blast_workspace(a.M, a.in_f, a.out_f, a.b, a.r, a.wbits);
   if (!a.ws || a.ws_bytes < need) { set_error("blast stream: workspace %zu < %zu", a.ws_bytes, need); return BLR_ERR_WORKSPACE; }
   WsLayout w = ws_carve(a.ws, (size_t)a.b * a.M * a.r);
-  if (decode2_applicable(a)) {
+  if (decode2_applicable(a) || a.rows_only) {
     int rc = decode2_blast_launch(a, w.d2, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
     if (rc <= 0) return rc;                    // served (or failed); 1 = shape outside its tiling
   }
+  if (a.rows_only) return BLR_ERR_UNSUPPORTED;
   const int MT = mt_for(a.M), target = target_items();
   const bool zatom = a.M <= zatom_max_m() && (size_t)a.b * a.M * a.r <= ZCAP_FLOATS;
   const bool inline_mix = !zatom && a.M <= mix_inline_max_m();

@@ -103,12 +103,12 @@ def test_blast_q_llama7b(layer, bits, M):
 def test_blast_q_rejects_bad_input():
     from triton_funcs import blast_sym_quant_kernels as Q, _lib as L
     x = torch.zeros(1, 1, 16, device="cuda", dtype=torch.float16)
-    U = torch.randn(2, 8, 24, device="cuda"); V = torch.randn(2, 8, 24, device="cuda")
+    U = torch.randn(2, 8, 20, device="cuda"); V = torch.randn(2, 8, 20, device="cuda")
     Uq, Vq = Q.quantize_blast_factors(U, V, 8)
     with pytest.raises(L.BlrError):      # one plain tensor, one QuantFactor
-        Q.triton_blast_bmm_int8_fp16(x, U.half(), Vq, torch.zeros(24, 2, 2, device="cuda", dtype=torch.float16))
-    with pytest.raises(L.BlrError):      # r = 24 is not a multiple of 32
-        Q.triton_blast_bmm_int8_fp16(x, Uq, Vq, torch.zeros(24, 2, 2, device="cuda", dtype=torch.float16))
+        Q.triton_blast_bmm_int8_fp16(x, U.half(), Vq, torch.zeros(20, 2, 2, device="cuda", dtype=torch.float16))
+    with pytest.raises(L.BlrError):      # r = 20 is not a multiple of 8
+        Q.triton_blast_bmm_int8_fp16(x, Uq, Vq, torch.zeros(20, 2, 2, device="cuda", dtype=torch.float16))
 
 
 def test_packed_factors_round_trip_through_a_checkpoint(tmp_path):
