@@ -47,6 +47,7 @@ struct RowsParams {
   int M, K, N;
   int kw;                                 // rows of a wave's share per round (a multiple of 32)
   int rounds;                             // passes of the eight waves over the rows
+  int per; int64_t o_ls; FastDiv perdiv;  // per > 0: Monarch scatter - column c of entry bt goes to out[(c / per) * o_ls + m * o_ms + bt * per + c % per]
   int npc;                                // 16-byte column pieces of a chunk (1..16)
   FastDiv nch;                            // chunks per batch entry
   uint32_t xcd_span;                      // items per XCD when the grid is a multiple of 8, else 0 (plain order)
@@ -267,15 +268,21 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   }
   if (m < p.M && c4 < cw && col < N) {
     T* o = reinterpret_cast<T*>(p.out) + (int64_t)m * p.o_ms + (int64_t)bt * p.o_bs;
-    if (p.o_ns == 1 && col + 3 < N && ((reinterpret_cast<uintptr_t>(o + col) & 7) == 0)) {
+    int ocol = col;
+    if (p.per > 0) {                                     // (per is a multiple of 4: the four columns stay together)
+      const uint32_t l = fd_div((uint32_t)col, p.perdiv);
+      o = reinterpret_cast<T*>(p.out) + (int64_t)l * p.o_ls + (int64_t)m * p.o_ms + (int64_t)bt * p.per;
+      ocol = col - (int)l * p.per;
+    }
+    if (p.o_ns == 1 && col + 3 < N && ((reinterpret_cast<uintptr_t>(o + ocol) & 7) == 0)) {
       typename TypeTraits<T>::vec4 v;
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = TypeTraits<T>::from_f32(tot[e]);
-      *reinterpret_cast<typename TypeTraits<T>::vec4*>(o + col) = v;
+      *reinterpret_cast<typename TypeTraits<T>::vec4*>(o + ocol) = v;
     } else {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (col + e < N) o[(int64_t)(col + e) * p.o_ns] = TypeTraits<T>::from_f32(tot[e]);
+        if (col + e < N) o[(int64_t)(ocol + e) * p.o_ns] = TypeTraits<T>::from_f32(tot[e]);
     }
   }
   TR5(4);
@@ -382,6 +389,9 @@ int plan_pieces(int batch, int K, int N, int wbits, int cus) {
     const double slab = (double)K * npc * wbits;      // bytes: 8 columns of wbits bits per piece and row
     double t = (double)cdiv(chunks, cus) * (0.5 + slab / 35e3);
     if (npc < 8) t += 0.05 * (8 - npc);
+    // rows that start on cache-line boundaries: chunks whose row piece is not whole lines make neighbours fetch lines twice
+    // (measured on 4 x (1024 x 5504): 176-byte pieces 24.4 us, 256-byte pieces 21.5 us for the whole call)
+    if (((int64_t)N * wbits / 8) % 128 == 0 && (npc * wbits) % 128 != 0) t *= 1.45;
     if (t < best_t - 1e-9) { best_t = t; best = npc; }
   }
   return best;
@@ -442,7 +452,9 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int b = a.b, M = a.M, R = a.r, P = a.in_f / a.b, Q = a.out_f / bo;
   const bool u_nk = a.u_layout == BLR_U_QR;
-  if (M < 1 || M > 16 || a.perm_per > 0 || !a.S || bo != b || (u_nk && a.wbits != 16)) return 1;
+  const bool monarch = a.perm_per > 0;                  // the mix is a permutation, folded into the store of the first product
+  if (M < 1 || M > 16 || (!monarch && !a.S) || bo != b || (u_nk && a.wbits != 16)) return 1;
+  if (monarch && (a.wbits != 16 || a.perm_per % 4 || R % a.perm_per || R / a.perm_per != b || a.perm_per >= 65536)) return 1;
   if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return 1;
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return 1;
   const size_t ybytes = align_up((size_t)b * M * R * 2, 256);
@@ -457,6 +469,7 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   s1.W = a.V; s1.w_bs = (int64_t)P * R;
   s1.out = Y; s1.o_ms = R; s1.o_bs = (int64_t)M * R; s1.o_ns = 1;
   s1.M = M; s1.K = P; s1.N = R; s1.scales = a.wbits != 16 ? (const f16*)a.v_scales : nullptr;
+  if (monarch) { s1.out = Z; s1.o_bs = 0; s1.per = a.perm_per; s1.o_ls = (int64_t)M * R; s1.perdiv = fd_make((uint32_t)a.perm_per); }
   RowsParams s2 = {};
   s2.A = Z; s2.lda = R; s2.a_bs = (int64_t)M * R; s2.a_bytes = (uint32_t)((size_t)b * M * R * 2);
   s2.W = a.U; s2.w_bs = (int64_t)R * Q;
@@ -474,7 +487,9 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   if (a.s_layout == BLR_S_JIR) { sj = (int64_t)b * R; si = R; sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { sr = (int64_t)b * b; si = b; sj = 1; }
   else { si = (int64_t)b * R; sj = R; sr = 1; }
-  if (sr == 1 && si % 4 == 0 && sj % 4 == 0 && R % 4 == 0 && aligned(a.S, 8) && (int64_t)M * b * (R / 4) * (R / 4) < ((int64_t)1 << 32) && b < 65536)   // the multiply-high division is exact below 2^32 / divisor
+  if (monarch)
+    rc = BLR_OK;
+  else if (sr == 1 && si % 4 == 0 && sj % 4 == 0 && R % 4 == 0 && aligned(a.S, 8) && (int64_t)M * b * (R / 4) * (R / 4) < ((int64_t)1 << 32) && b < 65536)   // the multiply-high division is exact below 2^32 / divisor
     rc = a.dtype == BLR_F16 ? rows_mix_t<f16>(Y, a.S, Z, M, b, R, si, sj, st) : rows_mix_t<bf16>(Y, a.S, Z, M, b, R, si, sj, st);
   else if (a.s_layout == BLR_S_RIJ && b == 16 && R % 4 == 0 && aligned(a.S, 16) && (int64_t)M * (R / 4) * (R / 4) < ((int64_t)1 << 32))
     rc = a.dtype == BLR_F16 ? rows_mix_rij_t<f16>(Y, a.S, Z, M, R, st) : rows_mix_rij_t<bf16>(Y, a.S, Z, M, R, st);

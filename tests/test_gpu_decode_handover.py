@@ -129,7 +129,8 @@ def _monarch_case(b, p, rank, s_out, M, dtype, seed):
 def _spinning_cases(dtype):
     """Calls served by kernels whose workgroups wait for each other (shapes at which the wait lasts microseconds)."""
     return {
-        "monarch_m8": _monarch_case(4, 1024, 1024, 1024, 8, dtype, 60),
+        # a permutation period of 254 (not a multiple of 4) keeps this call on the single-launch kernels
+        "monarch_m8": _monarch_case(4, 1024, 1016, 1024, 8, dtype, 60),
         "blast_bmm_m1": _blast_case(16, 256, 256, 512, 1, "triton_blast_bmm_fp16", dtype, 61),
         # 4104 input features cannot be cut into equal blocks of whole 16-byte pieces: the phase engine serves the call
         # (one launch, a barrier of the whole grid between the two products)
