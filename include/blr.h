@@ -95,6 +95,10 @@ typedef enum { BLR_ACT_NONE = 0, BLR_ACT_GELU_TANH = 1, BLR_ACT_SILU = 2 } blr_a
  * (4,000,000, about a second).  Meant for tests of the give-up path.                          */
 int blr_workspace_status(void* ws, size_t ws_bytes, void* stream);
 void blr_set_spin_limit(unsigned polls);
+/* Tuning options the tests switch at run time (no counterpart in the reference): BLR_GEMM_RING, BLR_GEMM_RING_TILE,
+ * BLR_GEMM_RING_PER_CU, BLR_GEMM_RING_WAVES, BLR_GEMM_SPLITK.  Each starts from the environment variable of its name
+ * (read once); unset != 0 returns it to "not set".  Returns BLR_ERR_BAD_ARG for an unknown name.                  */
+int blr_set_option(const char* name, int value, int unset);
 
 const char* blr_last_error(void);
 int blr_version(void);

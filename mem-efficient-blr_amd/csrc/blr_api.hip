@@ -2,6 +2,7 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <cstring>
 #include <mutex>
 #include "blr_common.h"
 #include "blr_decode.h"
@@ -215,6 +216,23 @@ static int with_epilogue(const void* bias, int act, void* out, int64_t ldo, int 
 using namespace blr;
 
 namespace blr {
+namespace {
+constexpr int kOptUnset = -2147483647 - 1;
+const char* const kOptNames[OPT_COUNT] = {"BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU", "BLR_GEMM_RING_WAVES", "BLR_GEMM_SPLITK"};
+std::atomic<int> g_opts[OPT_COUNT];
+std::once_flag g_opts_once;
+void opts_init() {
+  for (int i = 0; i < OPT_COUNT; ++i) {
+    const char* e = getenv(kOptNames[i]);
+    g_opts[i].store(e ? atoi(e) : kOptUnset, std::memory_order_relaxed);
+  }
+}
+}  // namespace
+int option_value(int id, int dflt) {
+  std::call_once(g_opts_once, opts_init);
+  const int v = g_opts[id].load(std::memory_order_relaxed);
+  return v == kOptUnset ? dflt : v;
+}
 static std::atomic<unsigned> g_spin_limit{0};
 unsigned spin_limit_now() {
   const unsigned v = g_spin_limit.load(std::memory_order_relaxed);
@@ -225,6 +243,17 @@ unsigned spin_limit_now() {
 extern "C" {
 
 void blr_set_spin_limit(unsigned polls) { blr::g_spin_limit.store(polls, std::memory_order_relaxed); }
+
+int blr_set_option(const char* name, int value, int unset) {
+  std::call_once(blr::g_opts_once, blr::opts_init);
+  for (int i = 0; name && i < blr::OPT_COUNT; ++i)
+    if (!strcmp(name, blr::kOptNames[i])) {
+      blr::g_opts[i].store(unset ? blr::kOptUnset : value, std::memory_order_relaxed);
+      return BLR_OK;
+    }
+  set_error("set_option: unknown option %s", name ? name : "(null)");
+  return BLR_ERR_BAD_ARG;
+}
 
 // Synchronises the stream, reads the error word of a streaming workspace and clears it.
 int blr_workspace_status(void* ws, size_t ws_bytes, void* stream) {
@@ -344,18 +373,6 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
   int a = resolve_algo(algo, M, dtype, z_out || y_out);
   if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
     if (dtype == BLR_F32 || M > 16 || z_out || y_out) { set_error("blast: streaming algorithm needs f16/bf16, M <= 16, no intermediates"); return BLR_ERR_UNSUPPORTED; }
-    // Optional (off by default, BLR_BLAST_SLAB_MIN_M): three launches - slab product, mix, slab product - instead of the single
-    // launch whose workgroups hand the intermediates to each other.  Measured at 16 rows: 39.1 against 33.7 us on gate_up,
-    // 30.8 against 19.3 on qkvo - the launches and the small mix cost more than the hand-overs.  Y and Z go behind the
-    // fixed-place block of the streaming workspace, so the same workspace keeps serving the single-launch kernels.
-    static const int slab_min_m = getenv("BLR_BLAST_SLAB_MIN_M") ? atoi(getenv("BLR_BLAST_SLAB_MIN_M")) : 99;
-    if (algo == BLR_ALGO_AUTO && M >= slab_min_m && u_layout == BLR_U_RQ && P <= 1024 && r <= 1024 && r % 8 == 0 && Q % 8 == 0 &&
-        aligned(U, 16) && aligned(V, 16)) {
-      const size_t off = stream_ws_prefix_bytes(), yz = 2 * align_up((size_t)b * M * r * elt_size(dtype), 256);
-      if (ws && ws_bytes >= off + yz)
-        return blast_tiled(x, ldx, U, V, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, u_layout, s_layout, 0,
-                           reinterpret_cast<char*>(ws) + off, ws_bytes - off, st);
-    }
     StreamBlastArgs s = {};
     s.x = x; s.ldx = ldx; s.U = U; s.V = V; s.S = S; s.out = out; s.ldo = ldo;
     s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
@@ -396,9 +413,8 @@ int blr_blast_i8act_fwd(const void* x, int64_t ldx, const void* U, const void* V
 // ---- quantized BLAST -----------------------------------------------------------------------------
 size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits) {
   if (M <= 0 || b <= 0 || r <= 0) return 0;
-  // M <= 16 streams the codes (the decode kernels widen them in registers).  Above that - or from 5 rows with
-  // BLR_Q_DIRECT=0 - the factors are expanded to two-byte values once per call ([kernel workspace][U][V]) and the
-  // two-byte kernels run; the size covers both.  Requests for the phase engine (BLR_ALGO_STREAM*) stream codes up to M = 16.
+  // M <= 16 streams the codes (the decode kernels widen them in registers).  Above that the factors are expanded to two-byte
+  // values once per call ([kernel workspace][U][V]) and the two-byte kernels run; the size covers both.
   size_t s = stream_blast_workspace(M <= 16 ? M : 16, in_f, out_f, b, r, bits);
   if (M <= 4) return s;
   size_t sub = M <= 16 ? s : 2 * align_up((size_t)b * M * r * 2, 256);
@@ -425,9 +441,7 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   const bool phase_engine = algo == BLR_ALGO_STREAM || algo == BLR_ALGO_STREAM_SPLIT;
   if (M > 16 && phase_engine) { set_error("blast_q: M=%d > 16 not served by the streaming kernel", M); return BLR_ERR_UNSUPPORTED; }
   // codes at 5..16 rows go to the matrix-core decode kernel as they are (it widens them in registers)
-  static const bool i8_direct = !getenv("BLR_Q_DIRECT") || atoi(getenv("BLR_Q_DIRECT")) != 0;
-  const bool direct = M <= 16 && i8_direct;
-  if ((M > 16 || (M > 4 && !phase_engine && !direct)) && !(M <= 16 && !whole16)) {
+  if (M > 16) {
     size_t need = blr_blast_q_workspace_bytes(M, in_f, out_f, b, r, bits);
     if (!ws || ws_bytes < need) { set_error("blast_q: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
     const size_t sub = align_up(M <= 16 ? stream_blast_workspace(M, in_f, out_f, b, r, bits) : 2 * align_up((size_t)b * M * r * 2, 256), 256);

@@ -84,6 +84,9 @@ unsigned spin_limit_now();
 // that applies it itself says so with epilogue_taken(), otherwise the entry point finishes with an elementwise launch.
 bool epilogue_pending(const void** bias, int* act);
 void epilogue_taken();
+// Tuning options that tests switch at run time (blr_set_option); each starts from the environment variable of its name, read once.
+enum { OPT_GEMM_RING = 0, OPT_GEMM_RING_TILE, OPT_GEMM_RING_PER_CU, OPT_GEMM_RING_WAVES, OPT_GEMM_SPLITK, OPT_COUNT };
+int option_value(int id, int dflt);             // the option's value, or dflt when it is unset
 // true when p is aligned to `bytes`.
 static inline bool aligned(const void* p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) % bytes) == 0; }
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -59,7 +59,7 @@ struct Decode2Params {
   int64_t s_si, s_sj, s_sr;
   int lpr1_log2, nch1, ks1, kc1, items1;
   int lpr2_log2, nch2, ks2, kc2, items2, pfn, kpad2;
-  int itemsM, rch_log2, pf_depth, pf_first, x_vec, sparse_poll, udelay;
+  int itemsM, rch_log2, pf_depth, pf_first, x_vec;
   unsigned long long* ypart;           // [ks1][b][M][R] tagged
   unsigned long long* zt;              // [b][M][R] tagged
   unsigned long long* opart;           // [ks2 - 1][b][M][Q] tagged
@@ -366,32 +366,11 @@ __global__ __launch_bounds__(256, 2) void decode2_kernel(Decode2Params p) {
   // The slab of U: asked for only now, after this workgroup's share of stage 1 (and of the mix), because
   // a wave that queues this many loads is held up until most of them have been accepted, and the
   // work heading the dependency chain must not sit behind that.
-  if (p.udelay > 0 && w >= p.items1 && w >= p.itemsM) {
-    while (wall_clock64() - t_begin < (unsigned long long)p.udelay) __builtin_amdgcn_s_sleep(2);
-  }
   issue_prefetch(pf_lo, D2_PF);
 
   // ---- stage-2 activations: this slab's slice of z, polled from the tagged pairs into LDS ---------------
   __syncthreads();                                   // earlier uses of a_s and red are over
   TR2(3);
-  if (p.sparse_poll) {
-    // Wait on one representative pair per chunk of ranks that a mix workgroup publishes before asking
-    // for the whole slice: the waiting slabs then re-read a few hundred bytes per round, not kilobytes.
-    const int RCH = 1 << p.rch_log2;
-    const int nch = (kcur2 + RCH - 1) >> p.rch_log2;
-    const int nrep = nch * M;
-    unsigned spins = 0;
-    while (true) {
-      bool ok = true;
-      for (int idx = tid; idx < nrep; idx += 256) {
-        const int m = idx / nch, r = k0_2 + (idx - m * nch) * RCH;
-        ok = ok && ((unsigned)(ld_tag(&p.zt[((int64_t)zi * M + m) * p.R + r]) >> 32) == epoch);
-      }
-      if (__syncthreads_and(ok)) break;
-      if (++spins > p.spin_limit) break;              // the full fetch below reports the failure
-      __builtin_amdgcn_s_sleep(2);
-    }
-  }
   {
     const int pairs = kcur2 >> 1;
     const int total = M * pairs;
@@ -976,23 +955,6 @@ __global__ __launch_bounds__(256, 2) void decode2m_kernel(Decode2Params p) {
   __syncthreads();
   TR2(3);
   const int kpad2 = p.kpad2, ald2 = kpad2 + 8;
-  if (p.sparse_poll) {
-    // one representative pair per patch (chunk of ranks x group of token rows) a mix item publishes
-    const int RCH = 1 << p.rch_log2;
-    const int nch = (kcur2 + RCH - 1) >> p.rch_log2;
-    const int nrep = nch * ((M + DM_MC - 1) / DM_MC);
-    unsigned spins = 0;
-    while (true) {
-      bool ok = true;
-      for (int idx = tid; idx < nrep; idx += 256) {
-        const int mc = idx / nch, r = k0_2 + (idx - mc * nch) * RCH;
-        ok = ok && ((unsigned)(ld_tag(&p.zt[((int64_t)zi * M + mc * DM_MC) * (p.R >> 1) + (r >> 1)]) >> 32) == epoch);
-      }
-      if (__syncthreads_and(ok)) break;
-      if (++spins > p.spin_limit) break;
-      __builtin_amdgcn_s_sleep(2);
-    }
-  }
   {
     const int quads = kcur2 >> 2;                                 // 16-byte units (4 ranks) per token row
     const int total = M * quads;
@@ -1489,12 +1451,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     if (p.itemsM > resident) return d2_bail(__LINE__);
     static const int e_depth = env_i("BLR_D2_PF_DEPTH", 4);
     p.pf_depth = e_depth;
-    static const int e_sparse = env_i("BLR_D2_SPARSE_POLL", 0);
-    p.sparse_poll = e_sparse;
-    static const int e_udelay = env_i("BLR_D2_UDELAY", 0);
-    p.udelay = e_udelay;
-    static const int e_first = env_i("BLR_D2_PF_FIRST", 0);
-    p.pf_first = e_first;
+    p.pf_first = 0;
   }
   const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)(p.zrep > 1 ? p.zrep : bo) * M * R * 8, 256);
   const size_t obytes = (size_t)(p.ks2 - 1) * bo * M * Q * 8;
@@ -1601,8 +1558,6 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     if (p.itemsM > resident) return d2_bail(__LINE__);
     static const int e_depth = env_i("BLR_DM_PF_DEPTH", 4);
     p.pf_depth = e_depth;
-    static const int e_sparse = env_i("BLR_D2_SPARSE_POLL", 0);
-    p.sparse_poll = e_sparse;
   }
   const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)(p.zrep > 1 ? p.zrep : bo) * M * (R / 2) * 8, 256);
   const size_t obytes = (size_t)(p.ks2 - 1) * bo * M * Q * 8;

@@ -62,7 +62,7 @@ struct Decode3Params {
   FastDiv nch1, bdiv;
   int lpr2_log2, ks2, kc2, items2, pfn, kpad2, kld2_log2, zspec;
   FastDiv nch2, bodiv;
-  int itemsM, rch_log2, udelay;
+  int itemsM, rch_log2;
   int x_vec, s_mode;                             // activations in 16-byte pieces; S: 0 = any strides, 1 = r contiguous, 2 = j contiguous
   unsigned spin_limit;
   int xcd_order;
@@ -428,10 +428,6 @@ __global__ __launch_bounds__(D3_NT) void decode3_kernel(Decode3Params p) {
         }
       }
   };
-  if (p.udelay > 0) {
-    const unsigned long long t0 = wall_clock64();
-    while (wall_clock64() - t0 < (unsigned long long)p.udelay) __builtin_amdgcn_s_sleep(2);
-  }
   u32x4 pf[D3_PF];
   u32x4 zv[MT][ZR];
 #pragma unroll
@@ -446,9 +442,6 @@ __global__ __launch_bounds__(D3_NT) void decode3_kernel(Decode3Params p) {
   for (int u = 0; u < D3_PFB; ++u) pf[D3_PFA + u] = ldw16(ubuf, u < nbq ? uoff : D3_OOB, (uint32_t)(naq + u) * ustep);
   TR3(12);
   check_in();
-#ifdef BLR_TRACE
-  if (p.udelay < 0) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); TR3(3); }
-#endif
 
   // ---- this slab's slice of z into LDS: the speculative fetch if it caught this call's values, else polled ----
   const int kld2 = 1 << p.kld2_log2;
@@ -617,12 +610,9 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
   p.spin_limit = spin_limit_now();
   { static const int e_xcd = env_i("BLR_XCD_ORDER", 1); p.xcd_order = e_xcd; }
-  static const int e_udelay = env_i("BLR_D3_UDELAY", 0);
-  p.udelay = e_udelay;
-  static const int e_vec = env_i("BLR_D3_VEC", 1);
-  p.x_vec = e_vec && aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0;
+  p.x_vec = aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0;
   p.s_mode = 0;
-  if (e_vec && a.S && aligned(a.S, 16) && b <= 16 && R % 8 == 0) {
+  if (a.S && aligned(a.S, 16) && b <= 16 && R % 8 == 0) {
     if (p.s_sr == 1 && p.s_si % 8 == 0 && p.s_sj % 8 == 0) p.s_mode = 1;
     else if (p.s_sj == 1 && b == 16 && p.s_si % 8 == 0 && p.s_sr % 8 == 0) p.s_mode = 2;
   }
@@ -737,11 +727,10 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   }
   {
     // the speculative fetch of z pays when the chain is expected to deliver before the last eight loads of a slab land
-    static const int e_zspec = env_i("BLR_D3_ZSPEC", -1);
     const double t_z = s1.t_chain + 2.2;
     const double slab_bytes = (double)p.kc2 * (1 << p.lpr2_log2) * 16.0;
     const double t_a = d3_stream_us((slab_bytes + s1.extra_slab) * (p.pfn > D3_PFB ? (double)(p.pfn - D3_PFB) / p.pfn : 0.0));
-    p.zspec = e_zspec >= 0 ? e_zspec : (p.pfn > D3_PFB && t_z + 0.5 < t_a ? 1 : 0);
+    p.zspec = (p.pfn > D3_PFB && t_z + 0.5 < t_a) ? 1 : 0;
   }
 
   const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)(p.zrep > 1 ? p.zrep : bo) * M * R * 8, 256);

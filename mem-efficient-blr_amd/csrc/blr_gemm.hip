@@ -864,15 +864,13 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   // Problems with enough work go to the ring kernels, with the largest of their tiles that still gives every compute unit
   // one (BLR_GEMM_RING: 0 never, 1 by this rule, 2 whenever the operands allow it; BLR_GEMM_RING_TILE = 256256, 256128
   // or 128128 picks the tile, BLR_GEMM_RING_PER_CU = 1 or 2 the deep or the shallow variant of the two smaller tiles,
-  // BLR_GEMM_RING_WAVES = 4 or 8 the workgroup size of the two larger ones - all read at every call so that tests can
-  // switch them).
-  const char* ring_e = getenv("BLR_GEMM_RING");
-  const int ring = ring_e ? atoi(ring_e) : 1;
+  // BLR_GEMM_RING_WAVES = 4 or 8 the workgroup size of the two larger ones - options that tests switch with
+  // blr_set_option).
+  const int ring = option_value(OPT_GEMM_RING, 1);
   if (ring > 0 && force == 0 && ring_ok(g) && g.splitk_ws && g.batch == 1 && g.cn == 1 && !g.sat8 && !g.bias && !g.act) {
     // few tiles, long reduction: slices of K as the batch of the partial-sum kernel, then one pass that adds them up
-    const char* sk_e = getenv("BLR_GEMM_SPLITK");
     int kc = 0;
-    const int splits = (sk_e && atoi(sk_e) == 0) ? 1 : splitk_plan(g.M, g.N, g.K, &kc);
+    const int splits = option_value(OPT_GEMM_SPLITK, 1) == 0 ? 1 : splitk_plan(g.M, g.N, g.K, &kc);
     if (splits > 1 && g.splitk_bytes >= (size_t)splits * g.M * g.N * sizeof(float) && aligned(g.splitk_ws, 16)) {
       GemmArgs p = g;
       p.batch = splits; p.kc = kc;
@@ -888,12 +886,10 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     }
   }
   if (ring > 0 && force == 0 && ring_ok(g)) {
-    const char* rt_e = getenv("BLR_GEMM_RING_TILE");
-    int rt = rt_e ? atoi(rt_e) : 0;
+    int rt = option_value(OPT_GEMM_RING_TILE, 0);
     const int64_t fill = ((int64_t)cus * 9 + 9) / 10;
     const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
-    const char* pc_e = getenv("BLR_GEMM_RING_PER_CU");
-    int per_cu = pc_e ? atoi(pc_e) : 0;
+    int per_cu = option_value(OPT_GEMM_RING_PER_CU, 0);
     // interleaved columns are bound by their two-byte stores: only worth it with several tiles per compute unit
     if (rt == 0 && g.cn != 1 && ring < 2 && t128 < 2 * (int64_t)cus) rt = -1;
     if (rt == 0) {
@@ -906,13 +902,11 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     }
     if (rt > 0 && (ring > 1 || (g.M >= 96 && g.K >= 64))) {
       if (rt == 256256) {
-        const char* w_e = getenv("BLR_GEMM_RING_WAVES");
         // eight waves (2 x 4, wave tile 128 x 64, two per SIMD) hide each other's barrier and LDS waits: the default
-        return (w_e && atoi(w_e) == 4) ? launch_ring<T, 256, 256>(g, st) : launch_ring<T, 256, 256, false, 8>(g, st);
+        return option_value(OPT_GEMM_RING_WAVES, 8) == 4 ? launch_ring<T, 256, 256>(g, st) : launch_ring<T, 256, 256, false, 8>(g, st);
       }
       if (rt == 256128) {
-        const char* w_e = getenv("BLR_GEMM_RING_WAVES");
-        if (per_cu != 2 && w_e && atoi(w_e) == 8) return launch_ring<T, 256, 128, false, 8>(g, st);
+        if (per_cu != 2 && option_value(OPT_GEMM_RING_WAVES, 4) == 8) return launch_ring<T, 256, 128, false, 8>(g, st);
         return per_cu == 2 ? launch_ring<T, 256, 128, true>(g, st) : launch_ring<T, 256, 128>(g, st);
       }
       if (!per_cu) per_cu = r128 >= 2 * (int64_t)cus ? 2 : 1;     // three shallow workgroups per compute unit, or two deep ones

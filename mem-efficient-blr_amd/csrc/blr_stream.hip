@@ -984,11 +984,11 @@ int env_int(const char* name, int dflt) {
 // Workgroups kept resident per CU (tuning aid: BLR_STREAM_WGS_PER_CU).
 int wgs_per_cu() { static int v = env_int("BLR_STREAM_WGS_PER_CU", 2); return v < 1 ? 1 : v; }
 // Largest M for which the BLAST mix is recomputed inside the last phase instead of run as its own phase.
-int mix_inline_max_m() { static int v = env_int("BLR_MIX_INLINE_MAX_M", 0); return v; }
+int mix_inline_max_m() { return 0; }
 // Largest M for which BLAST stage 1 adds its S-weighted result straight into Z with float atomics
 // (one grid barrier instead of two, no separate mix phase; the summation order over j is then not fixed).
 // Off by default: measured slower on MI355X, device-scope float atomics being the bottleneck.
-int zatom_max_m() { static int v = env_int("BLR_ZATOM_MAX_M", 0); return v; }
+int zatom_max_m() { return 0; }
 
 int nk_kstep(int wbits) { return wbits == 16 ? 32 : (wbits == 8 ? 64 : 128); }
 
@@ -1043,7 +1043,7 @@ bool plan_kn(PhaseDesc& d, int MT, int target, int M = 0) {
   // Option 1: each workgroup owns all of K for a narrower column chunk (row segments of at least
   // 128 bytes).  No partial sums cross workgroups, which takes three memory round trips off the
   // end of the phase.  Taken when it still yields enough workgroups to keep HBM busy.
-  static const bool allow_nosplit = env_int("BLR_STREAM_NOSPLIT", 0) != 0;
+  const bool allow_nosplit = false;
   if (allow_nosplit && d.K <= kc_max) {
     for (int lg = lg_full; lg >= 3; --lg) {
       const int lpr = 1 << lg;

@@ -51,6 +51,7 @@ _SIGNATURES = {
     "blr_dense_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp, _vp, _i]),
     "blr_workspace_status": (_i, [_vp, _sz, _vp]),
     "blr_set_spin_limit": (None, [_c.c_uint]),
+    "blr_set_option": (_i, [_c.c_char_p, _i, _i]),
     "blr_blast_fwd_static": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64] + [_i] * 8 + [_vp]),
     "blr_probe_dst_words": (_i, []),
     "blr_stream_probe": (_i, [_vp, _sz, _vp, _vp]),
@@ -99,6 +100,23 @@ def set_debug_checks(on):
     global _debug_checks
     prev, _debug_checks = _debug_checks, bool(on)
     return prev
+
+
+class options:
+    """with options(BLR_GEMM_RING=2, BLR_GEMM_RING_TILE=256128): ... - library tuning options for the block, unset afterwards."""
+
+    def __init__(self, **kw):
+        self.kw = kw
+
+    def __enter__(self):
+        for k, v in self.kw.items():
+            check(lib().blr_set_option(k.encode(), int(v), 0), "blr_set_option")
+        return self
+
+    def __exit__(self, *exc):
+        for k in self.kw:
+            lib().blr_set_option(k.encode(), 0, 1)
+        return False
 
 
 def workspace_status(ws, device=None):

@@ -29,8 +29,7 @@ def _act(v, act):
 @pytest.mark.parametrize("M", [3, 16, 40, 300])
 def test_blast_bias_activation(M, act, ring):
     from triton_funcs import blast_kernels as K, _lib as L
-    os.environ["BLR_GEMM_RING"] = ring
-    try:
+    with L.options(BLR_GEMM_RING=ring):
         b, p, q, r = 4, 32, 40, 64
         dtype = torch.float16
         x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=M)
@@ -43,8 +42,6 @@ def test_blast_bias_activation(M, act, ring):
         assert_close(out, _act(ref + rounded(bias, dtype), act), dtype, "blast + bias + act")
         plain = K.triton_blast_full_fp16(dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype))   # context closed: no epilogue
         assert_close(plain, ref, dtype, "plain call after the context")
-    finally:
-        os.environ.pop("BLR_GEMM_RING", None)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])

@@ -1,6 +1,6 @@
 """GPU parity of the GEMM kernels whose operand tiles are copied global -> LDS directly, against the oracle.
 
-They are normally chosen only for problems that fill the chip; BLR_GEMM_RING=2 selects them whenever the operands
+They are normally chosen only for problems that fill the chip; the option BLR_GEMM_RING=2 (blr_set_option) selects them whenever the operands
 allow it and BLR_GEMM_RING_TILE / BLR_GEMM_RING_PER_CU / BLR_GEMM_RING_WAVES pick the variant (256x256 with four or eight waves, 256x128 and 128x128 with deep or shallow rings), so small, ragged and tail shapes (M, N not multiples of 256; K with a 16-wide last slice; K shorter than
 the prefetch depth) run through it here.  Every case is also run with the kernel switched off and the two results
 must agree to rounding.
@@ -21,26 +21,16 @@ pytestmark = pytest.mark.gpu
 def ring_forced(request):
     """Selects the kernel for every legal problem, with one of its variants: tile shape / ring depth (1 deep rings, 2
     shallow ones and more workgroups per compute unit) / waves per workgroup (256x256 only)."""
-    env = ("BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU", "BLR_GEMM_RING_WAVES")
-    old = {k: os.environ.get(k) for k in env}
+    from triton_funcs import _lib as L
     parts = (request.param.split("/") + ["1", "4"])[:3]
-    os.environ["BLR_GEMM_RING"] = "2"
-    os.environ["BLR_GEMM_RING_TILE"], os.environ["BLR_GEMM_RING_PER_CU"], os.environ["BLR_GEMM_RING_WAVES"] = parts
-    yield request.param
-    for k, v in old.items():
-        if v is None:
-            os.environ.pop(k, None)
-        else:
-            os.environ[k] = v
+    with L.options(BLR_GEMM_RING=2, BLR_GEMM_RING_TILE=parts[0], BLR_GEMM_RING_PER_CU=parts[1], BLR_GEMM_RING_WAVES=parts[2]):
+        yield request.param
 
 
 def _without_ring(fn):
-    old = os.environ.get("BLR_GEMM_RING")
-    os.environ["BLR_GEMM_RING"] = "0"
-    try:
+    from triton_funcs import _lib as L
+    with L.options(BLR_GEMM_RING=0):
         return fn()
-    finally:
-        os.environ["BLR_GEMM_RING"] = old
 
 
 TILED = {"algo": 2}
@@ -131,13 +121,7 @@ def test_low_rank_with_the_reduction_cut_into_slices(M, in_f, r, out_f, dtype):
     assert_close(out, (rounded(x, dtype) @ rounded(a, dtype)) @ rounded(bm, dtype), dtype, "low rank", scale=2.0)
     again = LR.triton_low_rank_fp16(xd, ad, bd, TILED)
     assert torch.equal(out, again), "the sum over slices must not depend on timing"
-    old = os.environ.get("BLR_GEMM_SPLITK")
-    os.environ["BLR_GEMM_SPLITK"] = "0"
-    try:
+    from triton_funcs import _lib as L
+    with L.options(BLR_GEMM_SPLITK=0):
         ref = LR.triton_low_rank_fp16(xd, ad, bd, TILED)
-    finally:
-        if old is None:
-            os.environ.pop("BLR_GEMM_SPLITK", None)
-        else:
-            os.environ["BLR_GEMM_SPLITK"] = old
     assert_close(out, back(ref), dtype, "split vs unsplit", scale=0.5)
