@@ -324,6 +324,29 @@ __global__ __launch_bounds__(256) void rows_mix_kernel(const T* __restrict__ Y, 
   *reinterpret_cast<V4*>(Z + ((int64_t)i * M + m) * R + r4 * 4) = o;
 }
 
+// Low rank seen as BLAST with one output block and S = 1: z[m][r] = sum_j y[j][m][r] (the k-slices of x A), fp32 sums in slice order.
+template <typename T>
+__global__ __launch_bounds__(256) void rows_sum_kernel(const T* __restrict__ Y, T* __restrict__ Z, int b, int64_t MR4) {
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= MR4) return;
+  using V4 = typename TypeTraits<T>::vec4;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int j0 = 0; j0 < b; j0 += 8) {
+    V4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const V4*>(Y + ((int64_t)min(j0 + u, b - 1) * MR4 + item) * 4);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (j0 + u < b)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += TypeTraits<T>::to_f32(v[u][e]);
+  }
+  V4 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = TypeTraits<T>::from_f32(acc[e]);
+  *reinterpret_cast<V4*>(Z + item * 4) = o;
+}
+
 // The same mix for S stored (r, i, j) - the input block contiguous (the layout of the bmm names and of the quantized
 // entry points).  Neighbouring threads take neighbouring output blocks i, so that a wave reads whole (r, :, :) slices of S.
 template <typename T>
@@ -453,7 +476,9 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   const int b = a.b, M = a.M, R = a.r, P = a.in_f / a.b, Q = a.out_f / bo;
   const bool u_nk = a.u_layout == BLR_U_QR;
   const bool monarch = a.perm_per > 0;                  // the mix is a permutation, folded into the store of the first product
-  if (M < 1 || M > 16 || (!monarch && !a.S) || bo != b || (u_nk && a.wbits != 16)) return 1;
+  const bool lowrank = !monarch && !a.S && bo == 1;     // one output block, S = 1: the mix is the sum over the input slices
+  if (M < 1 || M > 16 || (!monarch && !lowrank && !a.S) || (bo != b && !lowrank) || (u_nk && a.wbits != 16)) return 1;
+  if (lowrank && a.wbits != 16) return 1;
   if (monarch && (a.wbits != 16 || a.perm_per % 4 || R % a.perm_per || R / a.perm_per != b || a.perm_per >= 65536)) return 1;
   if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return 1;
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return 1;
@@ -471,7 +496,7 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   s1.M = M; s1.K = P; s1.N = R; s1.scales = a.wbits != 16 ? (const f16*)a.v_scales : nullptr;
   if (monarch) { s1.out = Z; s1.o_bs = 0; s1.per = a.perm_per; s1.o_ls = (int64_t)M * R; s1.perdiv = fd_make((uint32_t)a.perm_per); }
   RowsParams s2 = {};
-  s2.A = Z; s2.lda = R; s2.a_bs = (int64_t)M * R; s2.a_bytes = (uint32_t)((size_t)b * M * R * 2);
+  s2.A = Z; s2.lda = R; s2.a_bs = (int64_t)M * R; s2.a_bytes = (uint32_t)((size_t)bo * M * R * 2);
   s2.W = a.U; s2.w_bs = (int64_t)R * Q;
   s2.out = a.out; s2.o_ms = a.ldo;
   s2.o_bs = a.out_ns ? a.out_bs : Q; s2.o_ns = a.out_ns ? a.out_ns : 1;
@@ -489,14 +514,19 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   else { si = (int64_t)b * R; sj = R; sr = 1; }
   if (monarch)
     rc = BLR_OK;
-  else if (sr == 1 && si % 4 == 0 && sj % 4 == 0 && R % 4 == 0 && aligned(a.S, 8) && (int64_t)M * b * (R / 4) * (R / 4) < ((int64_t)1 << 32) && b < 65536)   // the multiply-high division is exact below 2^32 / divisor
+  else if (lowrank) {
+    const int64_t mr4 = (int64_t)M * R / 4;
+    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_sum_kernel<f16>, dim3((unsigned)cdiv(mr4, 256)), dim3(256), 0, st, (const f16*)Y, (f16*)Z, b, mr4);
+    else hipLaunchKernelGGL(rows_sum_kernel<bf16>, dim3((unsigned)cdiv(mr4, 256)), dim3(256), 0, st, (const bf16*)Y, (bf16*)Z, b, mr4);
+    BLR_CHECK_LAUNCH("rows_sum");
+  } else if (sr == 1 && si % 4 == 0 && sj % 4 == 0 && R % 4 == 0 && aligned(a.S, 8) && (int64_t)M * b * (R / 4) * (R / 4) < ((int64_t)1 << 32) && b < 65536)   // the multiply-high division is exact below 2^32 / divisor
     rc = a.dtype == BLR_F16 ? rows_mix_t<f16>(Y, a.S, Z, M, b, R, si, sj, st) : rows_mix_t<bf16>(Y, a.S, Z, M, b, R, si, sj, st);
   else if (a.s_layout == BLR_S_RIJ && b == 16 && R % 4 == 0 && aligned(a.S, 16) && (int64_t)M * (R / 4) * (R / 4) < ((int64_t)1 << 32))
     rc = a.dtype == BLR_F16 ? rows_mix_rij_t<f16>(Y, a.S, Z, M, R, st) : rows_mix_rij_t<bf16>(Y, a.S, Z, M, R, st);
   else
     rc = blast_mix_launch(Y, a.S, Z, M, b, R, si, sj, sr, a.dtype, st, 0);
   if (rc) return rc;
-  rc = rows_product(s2, b, a.dtype, a.wbits, u_nk, st);
+  rc = rows_product(s2, bo, a.dtype, a.wbits, u_nk, st);
   if (rc == BLR_OK && s2.ep) epilogue_taken();
   return rc == 1 ? BLR_ERR_UNSUPPORTED : rc;
 }

@@ -1312,6 +1312,22 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
   }
   if (a.op == 1) {                             // low rank: z = x A (in, r); out = z B (r, out)
     WsLayout w = ws_carve(a.ws, (size_t)a.M * a.r);
+    static const int rows_min_m = env_int("BLR_LOWRANK_ROWS_MIN_M", 2);
+    if (!a.split && a.M >= rows_min_m) {
+      // From two rows up: the three-launch matrix-core path, low rank being BLAST with the input cut into 16 (or 8, 4, 2) slices of
+      // rows of A, one output block and S = 1 (the mix is the sum over the slices).
+      int bi = 0;
+      for (int c = 16; c >= 2 && !bi; c >>= 1)
+        if (a.in_f % c == 0 && (a.in_f / c) % 8 == 0) bi = c;
+      if (bi) {
+        StreamBlastArgs bl = {};
+        bl.x = a.x; bl.ldx = a.ldx; bl.U = a.W2; bl.V = a.W1; bl.S = nullptr; bl.out = a.out; bl.ldo = a.ldo;
+        bl.M = a.M; bl.in_f = a.in_f; bl.out_f = a.out_f; bl.b = bi; bl.bo = 1; bl.r = a.r;
+        bl.dtype = a.dtype; bl.u_layout = BLR_U_RQ; bl.s_layout = BLR_S_IJR; bl.wbits = 16;
+        const int rc = decode_rows_launch(bl, w.d2, decode2_region_bytes(), st);
+        if (rc != 1) return rc;
+      }
+    }
     static const int slab_min_m = env_int("BLR_LOWRANK_SLAB_MIN_M", 5);
     if (!a.split && a.M >= slab_min_m && a.r % 8 == 0 && a.out_f % 8 == 0) {
       // From a handful of rows up, two launches of the slab kernel, each followed by the sum of its k-slices: z = x A goes
