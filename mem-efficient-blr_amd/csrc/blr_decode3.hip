@@ -66,6 +66,7 @@ struct Decode3Params {
   int x_vec, s_mode;                             // activations in 16-byte pieces; S: 0 = any strides, 1 = r contiguous, 2 = j contiguous
   unsigned spin_limit;
   int xcd_order;
+  const void* bias; int act, ep;                 // fused output stage: bias of T (indexed like a row of out) or null, blr_act
   unsigned long long* ypart;           // [ks1][b][M][R] tagged
   unsigned long long* zt;              // [bo or zrep][M][R] tagged
   unsigned long long* opart;           // [ks2 - 1][bo][M][Q] tagged
@@ -546,7 +547,16 @@ __global__ __launch_bounds__(D3_NT) void decode3_kernel(Decode3Params p) {
             }
             v += __uint_as_float((unsigned)pv);
           }
-          outp[(int64_t)m * p.ldo + (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns] = TypeTraits<T>::from_f32(v * usc);
+          {
+            const int64_t oc = (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns;
+            T r = TypeTraits<T>::from_f32(v * usc);
+            if (p.ep) {                                  // on the rounded result, as a separate elementwise kernel would see it
+              float e = TypeTraits<T>::to_f32(r);
+              if (p.bias) e += TypeTraits<T>::to_f32(reinterpret_cast<const T*>(p.bias)[oc]);
+              r = TypeTraits<T>::from_f32(apply_act(e, p.act));
+            }
+            outp[(int64_t)m * p.ldo + oc] = r;
+          }
         }
       }
     }
@@ -610,6 +620,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
   p.spin_limit = spin_limit_now();
   { static const int e_xcd = env_i("BLR_XCD_ORDER", 1); p.xcd_order = e_xcd; }
+  { const void* eb = nullptr; int ea = 0; if (epilogue_pending(&eb, &ea)) { p.ep = 1; p.bias = eb; p.act = ea; } }
   p.x_vec = aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0;
   p.s_mode = 0;
   if (a.S && aligned(a.S, 16) && b <= 16 && R % 8 == 0) {
@@ -748,6 +759,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   void* args[] = {&p};
   hipError_t e = hipLaunchKernel(fn, dim3(grid), dim3(D3_NT), args, 0, st);
   if (e != hipSuccess) { set_error("decode3: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  if (p.ep) epilogue_taken();
   return BLR_OK;
 }
 

@@ -52,6 +52,7 @@ struct PairParams {
   int lpr2_log2, pfn, kld2_log2, octs_log2, jpg;
   FastDiv nch2;
   int xcd_order;
+  const void* bias; int act, ep;                 // fused output stage: bias of T (indexed like a row of out) or null, blr_act
 };
 
 __device__ __forceinline__ void lds_barrier2() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
@@ -338,7 +339,16 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
     T* outp = reinterpret_cast<T*>(p.out);
 #pragma unroll
     for (int m = 0; m < MT; ++m)
-      if (m < M) outp[(int64_t)m * p.ldo + (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns] = TypeTraits<T>::from_f32(tot[m] * usc);
+      if (m < M) {
+        const int64_t oc = (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns;
+        T r = TypeTraits<T>::from_f32(tot[m] * usc);
+        if (p.ep) {                                      // on the rounded result, as a separate elementwise kernel would see it
+          float v = TypeTraits<T>::to_f32(r);
+          if (p.bias) v += TypeTraits<T>::to_f32(reinterpret_cast<const T*>(p.bias)[oc]);
+          r = TypeTraits<T>::from_f32(apply_act(v, p.act));
+        }
+        outp[(int64_t)m * p.ldo + oc] = r;
+      }
   }
   TR4(4);
 }
@@ -426,6 +436,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     p.ks1 = ks; p.kc1 = kc; p.kpad1_log2 = ilog2(kpad);
   }
   { static const int e_xcd = env_i("BLR_XCD_ORDER", 1); p.xcd_order = e_xcd; }
+  { const void* eb = nullptr; int ea = 0; if (epilogue_pending(&eb, &ea)) { p.ep = 1; p.bias = eb; p.act = ea; } }
   const size_t ybytes = (size_t)p.ks1 * b * M * R * 2;
   if (ybytes > region_bytes) return d2_bail(__LINE__);
   p.y = region;
@@ -486,6 +497,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   hipError_t e = hipLaunchKernel(f1, dim3(grid1), dim3(DP_NT), args, 0, st);
   if (e == hipSuccess) e = hipLaunchKernel(f2, dim3(grid2), dim3(DP_NT), args, 0, st);
   if (e != hipSuccess) { set_error("decode pair: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  if (p.ep) epilogue_taken();
   return BLR_OK;
 }
 

@@ -44,6 +44,24 @@ def test_blast_bias_activation(M, act, ring):
         assert_close(plain, ref, dtype, "plain call after the context")
 
 
+@pytest.mark.parametrize("act", [None, "silu"])
+@pytest.mark.parametrize("shape", [(16, 64, 72, 128), (16, 256, 1376, 1024)], ids=["short-slabs", "gate_up"])
+def test_blast_single_row_bias_activation_in_the_kernel(shape, act):
+    """One row: the two-launch kernel (short slabs) and the single-launch kernel (gate_up-sized slabs) apply bias and activation
+    in their own output stage."""
+    from triton_funcs import blast_kernels as K, _lib as L
+    b, p, q, r = shape
+    dtype = torch.float16
+    x, U, Vt, S = blast_inputs(b, p, q, r, (1,), seed=11)
+    bias = np.random.default_rng(11).standard_normal(b * q)
+    Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+    say(f"[case] epilogue blast M=1 shape={shape} act={act}")
+    with L.fused_epilogue(dev(bias, dtype), act):
+        out = K.triton_blast_full_fp16(dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype))
+    ref = O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0]
+    assert_close(out, _act(ref + rounded(bias, dtype), act), dtype, "blast M=1 + bias + act")
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M", [5, 130])
 def test_dense_low_rank_monarch_bias_activation(M, dtype):
