@@ -224,6 +224,31 @@ int blr_dense_fwd_ep(const void* x, int64_t ldx, const void* W, void* out, int64
                      int M, int in_f, int out_f, int dtype, int algo,
                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act);
 
+/* The same with a gate and a residual on top: out = resid + gate[m / gate_rows] * act(op(x) + bias), the adaLN-Zero update of a
+ * DiT block (reference DiT/models.py:120-121: x = x + gate.unsqueeze(1) * attn(...) / mlp(...)), which the callers otherwise run as
+ * separate elementwise kernels over the M x out_f result.  gate: (ceil(M / gate_rows), out_f) of dtype with row stride ld_gate, one
+ * row per group of gate_rows consecutive rows (the tokens of one image), or NULL; resid: (M, out_f) of dtype with row stride
+ * ld_resid, or NULL (it may be the same memory as out only if ldo == ld_resid: every element is read before it is written by the
+ * same thread).  Fused into the write-out of the last GEMM at M > 16, an elementwise launch after the operator otherwise.   */
+int blr_blast_fwd_ep2(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                      void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
+                      int dtype, int u_layout, int s_layout, int algo,
+                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
+                      const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid);
+int blr_monarch_fwd_ep2(const void* x, int64_t ldx, const void* w1, const void* w2,
+                        void* out, int64_t ldo, int M, int in_f, int out_f, int b, int rank,
+                        int dtype, int w2_layout, int out_order, int algo,
+                        void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
+                        const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid);
+int blr_low_rank_fwd_ep2(const void* x, int64_t ldx, const void* A, const void* B,
+                         void* out, int64_t ldo, int M, int in_f, int out_f, int r, int dtype, int algo,
+                         void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
+                         const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid);
+int blr_dense_fwd_ep2(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
+                      int M, int in_f, int out_f, int dtype, int algo,
+                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
+                      const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid);
+
 /* ---- BLAST forward that allocates nothing and takes no workspace -------------------------------
  * No counterpart in the reference.  For callers that cannot allocate device memory or carry a workspace
  * around: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same

@@ -163,11 +163,11 @@ static int quantize_t(const void* w, int64_t outer, int64_t reduce, int64_t inne
 // ---- fused output stage ------------------------------------------------------------------------------
 // The *_fwd_ep entry points arm this per-thread record and call the plain entry point; the tiled path attaches it
 // to its last GEMM (attach_epilogue), any other path leaves it and the entry point finishes with bias_act_kernel.
-struct PendingEpilogue { const void* bias; int act; bool armed; bool used; };
-static thread_local PendingEpilogue tl_ep = {nullptr, 0, false, false};
+struct PendingEpilogue { const void* bias; int act; bool armed; bool used; const void* gate; int gate_rows; int64_t ld_gate; const void* resid; int64_t ld_resid; };
+static thread_local PendingEpilogue tl_ep = {nullptr, 0, false, false, nullptr, 0, 0, nullptr, 0};
 
 bool epilogue_pending(const void** bias, int* act) {
-  if (!tl_ep.armed || tl_ep.used) return false;
+  if (!tl_ep.armed || tl_ep.used || tl_ep.gate || tl_ep.resid) return false;
   *bias = tl_ep.bias; *act = tl_ep.act;
   return true;
 }
@@ -176,39 +176,53 @@ void epilogue_taken() { tl_ep.used = true; }
 static void attach_epilogue(GemmArgs& g) {
   if (!tl_ep.armed) return;
   g.bias = tl_ep.bias; g.act = tl_ep.act;
+  g.gate = tl_ep.gate; g.gate_rows = tl_ep.gate_rows; g.ld_gate = tl_ep.ld_gate; g.resid = tl_ep.resid; g.ld_resid = tl_ep.ld_resid;
   tl_ep.used = true;
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void bias_act_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ bias, int act, int M, int N) {
+__global__ __launch_bounds__(256) void bias_act_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ bias, int act, int M, int N,
+                                                        const T* __restrict__ gate, int gate_rows, int64_t ld_gate, const T* __restrict__ resid, int64_t ld_resid) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (int64_t)M * N) return;
   const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
   float v = TypeTraits<T>::to_f32(out[(int64_t)m * ldo + n]);
   if (bias) v += TypeTraits<T>::to_f32(bias[n]);
-  out[(int64_t)m * ldo + n] = TypeTraits<T>::from_f32(apply_act(v, act));
+  v = apply_act(v, act);
+  if (gate || resid) {
+    v = TypeTraits<T>::to_f32(TypeTraits<T>::from_f32(v));
+    if (gate) v *= TypeTraits<T>::to_f32(gate[(int64_t)(m / gate_rows) * ld_gate + n]);
+    if (resid) v += TypeTraits<T>::to_f32(resid[(int64_t)m * ld_resid + n]);
+  }
+  out[(int64_t)m * ldo + n] = TypeTraits<T>::from_f32(v);
 }
 
-static int bias_act_launch(void* out, int64_t ldo, const void* bias, int act, int M, int N, int dtype, hipStream_t st) {
-  if (!bias && !act) return BLR_OK;
+static int bias_act_launch(void* out, int64_t ldo, const PendingEpilogue& ep, int M, int N, int dtype, hipStream_t st) {
+  if (!ep.bias && !ep.act && !ep.gate && !ep.resid) return BLR_OK;
   const unsigned grid = (unsigned)cdiv((int64_t)M * N, 256);
-  if (dtype == BLR_F16) hipLaunchKernelGGL(bias_act_kernel<f16>, dim3(grid), dim3(256), 0, st, (f16*)out, ldo, (const f16*)bias, act, M, N);
-  else if (dtype == BLR_BF16) hipLaunchKernelGGL(bias_act_kernel<bf16>, dim3(grid), dim3(256), 0, st, (bf16*)out, ldo, (const bf16*)bias, act, M, N);
-  else hipLaunchKernelGGL(bias_act_kernel<float>, dim3(grid), dim3(256), 0, st, (float*)out, ldo, (const float*)bias, act, M, N);
+  if (dtype == BLR_F16) hipLaunchKernelGGL(bias_act_kernel<f16>, dim3(grid), dim3(256), 0, st, (f16*)out, ldo, (const f16*)ep.bias, ep.act, M, N, (const f16*)ep.gate, ep.gate_rows, ep.ld_gate, (const f16*)ep.resid, ep.ld_resid);
+  else if (dtype == BLR_BF16) hipLaunchKernelGGL(bias_act_kernel<bf16>, dim3(grid), dim3(256), 0, st, (bf16*)out, ldo, (const bf16*)ep.bias, ep.act, M, N, (const bf16*)ep.gate, ep.gate_rows, ep.ld_gate, (const bf16*)ep.resid, ep.ld_resid);
+  else hipLaunchKernelGGL(bias_act_kernel<float>, dim3(grid), dim3(256), 0, st, (float*)out, ldo, (const float*)ep.bias, ep.act, M, N, (const float*)ep.gate, ep.gate_rows, ep.ld_gate, (const float*)ep.resid, ep.ld_resid);
   BLR_CHECK_LAUNCH("bias_act");
   return BLR_OK;
 }
 
 // Runs `call` (a plain entry point) with the epilogue armed and finishes whatever the call did not fuse.
+struct GateResidual { const void* gate; int gate_rows; int64_t ld_gate; const void* resid; int64_t ld_resid; };
 template <typename F>
-static int with_epilogue(const void* bias, int act, void* out, int64_t ldo, int M, int out_f, int dtype, void* stream, F&& call) {
+static int with_epilogue(const void* bias, int act, void* out, int64_t ldo, int M, int out_f, int dtype, void* stream, F&& call,
+                         GateResidual gr = {nullptr, 0, 0, nullptr, 0}) {
   if (act < BLR_ACT_NONE || act > BLR_ACT_SILU) { set_error("epilogue: unknown activation %d", act); return BLR_ERR_BAD_ARG; }
-  tl_ep = {bias, act, (bias != nullptr) || act != BLR_ACT_NONE, false};
+  if (gr.gate && (gr.gate_rows <= 0 || gr.ld_gate < out_f)) { set_error("epilogue: gate needs gate_rows > 0 and ld_gate >= out_f"); return BLR_ERR_BAD_ARG; }
+  if (gr.resid && gr.ld_resid < out_f) { set_error("epilogue: ld_resid < out_f"); return BLR_ERR_BAD_ARG; }
+  const PendingEpilogue ep = {bias, act, bias != nullptr || act != BLR_ACT_NONE || gr.gate != nullptr || gr.resid != nullptr, false,
+                              gr.gate, gr.gate_rows, gr.ld_gate, gr.resid, gr.ld_resid};
+  tl_ep = ep;
   const int rc = call();
   const bool used = tl_ep.used, armed = tl_ep.armed;
-  tl_ep = {nullptr, 0, false, false};
+  tl_ep = {nullptr, 0, false, false, nullptr, 0, 0, nullptr, 0};
   if (rc != BLR_OK || !armed || used) return rc;
-  return bias_act_launch(out, ldo, bias, act, M, out_f, dtype, (hipStream_t)stream);
+  return bias_act_launch(out, ldo, ep, M, out_f, dtype, (hipStream_t)stream);
 }
 
 }  // namespace blr
@@ -656,6 +670,46 @@ int blr_dense_fwd_ep(const void* x, int64_t ldx, const void* W, void* out, int64
     return blr_dense_fwd(x, ldx, W, out, ldo, M, in_f, out_f, dtype, algo, ws, ws_bytes, stream);
   });
 }
+
+// ---- the same with a gate and a residual: out = resid + gate[row group] * act(op(x) + bias) -------------------------------------
+int blr_blast_fwd_ep2(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
+                      void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
+                      int dtype, int u_layout, int s_layout, int algo,
+                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
+                      const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid) {
+  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
+    return blr_blast_fwd(x, ldx, U, V, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, u_layout, s_layout, algo, ws, ws_bytes, stream);
+  }, {gate, gate_rows, ld_gate, resid, ld_resid});
+}
+
+int blr_monarch_fwd_ep2(const void* x, int64_t ldx, const void* w1, const void* w2,
+                        void* out, int64_t ldo, int M, int in_f, int out_f, int b, int rank,
+                        int dtype, int w2_layout, int out_order, int algo,
+                        void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
+                        const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid) {
+  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
+    return blr_monarch_fwd(x, ldx, w1, w2, out, ldo, nullptr, M, in_f, out_f, b, rank, dtype, w2_layout, out_order, algo, ws, ws_bytes, stream);
+  }, {gate, gate_rows, ld_gate, resid, ld_resid});
+}
+
+int blr_low_rank_fwd_ep2(const void* x, int64_t ldx, const void* A, const void* B,
+                         void* out, int64_t ldo, int M, int in_f, int out_f, int r, int dtype, int algo,
+                         void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
+                         const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid) {
+  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
+    return blr_low_rank_fwd(x, ldx, A, B, out, ldo, nullptr, M, in_f, out_f, r, dtype, algo, ws, ws_bytes, stream);
+  }, {gate, gate_rows, ld_gate, resid, ld_resid});
+}
+
+int blr_dense_fwd_ep2(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
+                      int M, int in_f, int out_f, int dtype, int algo,
+                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
+                      const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid) {
+  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
+    return blr_dense_fwd(x, ldx, W, out, ldo, M, in_f, out_f, dtype, algo, ws, ws_bytes, stream);
+  }, {gate, gate_rows, ld_gate, resid, ld_resid});
+}
+
 
 }  // extern "C"
 

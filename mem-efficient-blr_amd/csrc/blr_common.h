@@ -82,7 +82,7 @@ int device_cus();
 unsigned spin_limit_now();
 // The fused output stage armed by the *_fwd_ep entry point of the running call, if any (bias of dtype or null, blr_act); a kernel
 // that applies it itself says so with epilogue_taken(), otherwise the entry point finishes with an elementwise launch.
-bool epilogue_pending(const void** bias, int* act);
+bool epilogue_pending(const void** bias, int* act);   // (false when a gate or a residual is armed: only the tiled path fuses those)
 void epilogue_taken();
 // Tuning options that tests switch at run time (blr_set_option); each starts from the environment variable of its name, read once.
 enum { OPT_GEMM_RING = 0, OPT_GEMM_RING_TILE, OPT_GEMM_RING_PER_CU, OPT_GEMM_RING_WAVES, OPT_GEMM_SPLITK, OPT_COUNT };
@@ -115,6 +115,8 @@ struct GemmArgs {
   int sat8;         // 1: the fp32 result is rounded to nearest even and clamped to [-128, 127] before it is stored
   const void* bias; // optional: values of dtype added to the rounded result, indexed by the element's offset inside its row of C
   int act;          // blr_act applied after the bias
+  const void* gate; int gate_rows; int64_t ld_gate;   // optional: after the activation, the value is multiplied by gate[(m / gate_rows) * ld_gate + offset in row]
+  const void* resid; int64_t ld_resid;   // optional: and resid[m * ld_resid + offset in row] is added (DiT: x + g * h, reference DiT/models.py:120-121)
   void* splitk_ws;  // optional scratch for splitting the reduction (gemm_splitk_bytes says how much); null: never split
   size_t splitk_bytes;
   int kc;           // set by gemm_launch for the split kernels: k values per slice

@@ -168,15 +168,21 @@ __device__ __forceinline__ int64_t epi_offset(const GemmArgs& g, int bt, int m, 
 // activation are applied to the rounded result on its way out, like the separate kernels of the callers would.  The
 // plain instantiations do not contain this code: it costs registers that the main loops need.
 template <typename T>
-__device__ __forceinline__ T ep_value(const GemmArgs& g, T r, int64_t in_row) {
+__device__ __forceinline__ T ep_value(const GemmArgs& g, T r, int64_t in_row, int row) {
   float v = TypeTraits<T>::to_f32(r);
   if (g.bias) v += TypeTraits<T>::to_f32(reinterpret_cast<const T*>(g.bias)[in_row]);
-  return TypeTraits<T>::from_f32(apply_act(v, g.act));
+  v = apply_act(v, g.act);
+  if (g.gate || g.resid) {
+    v = TypeTraits<T>::to_f32(TypeTraits<T>::from_f32(v));                    // what a separate gate / residual kernel would read
+    if (g.gate) v *= TypeTraits<T>::to_f32(reinterpret_cast<const T*>(g.gate)[(int64_t)(row / g.gate_rows) * g.ld_gate + in_row]);
+    if (g.resid) v += TypeTraits<T>::to_f32(reinterpret_cast<const T*>(g.resid)[(int64_t)row * g.ld_resid + in_row]);
+  }
+  return TypeTraits<T>::from_f32(v);
 }
 
 // eight consecutive outputs; their offset inside the row is a multiple of 8, so the bias comes as one 16-byte load
 template <typename T>
-__device__ __forceinline__ typename TypeTraits<T>::vec8 ep_vector(const GemmArgs& g, typename TypeTraits<T>::vec8 r, int64_t in_row) {
+__device__ __forceinline__ typename TypeTraits<T>::vec8 ep_vector(const GemmArgs& g, typename TypeTraits<T>::vec8 r, int64_t in_row, int row) {
   using V8 = typename TypeTraits<T>::vec8;
   V8 bv;
 #pragma unroll
@@ -184,6 +190,15 @@ __device__ __forceinline__ typename TypeTraits<T>::vec8 ep_vector(const GemmArgs
   if (g.bias) bv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(g.bias) + in_row);
 #pragma unroll
   for (int e = 0; e < 8; ++e) r[e] = TypeTraits<T>::from_f32(apply_act(TypeTraits<T>::to_f32(r[e]) + TypeTraits<T>::to_f32(bv[e]), g.act));
+  if (g.gate || g.resid) {                      // one row of gate per group of gate_rows rows of C
+    V8 gv, rv;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { gv[e] = (T)1.0f; rv[e] = (T)0.0f; }
+    if (g.gate) gv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(g.gate) + (int64_t)(row / g.gate_rows) * g.ld_gate + in_row);
+    if (g.resid) rv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(g.resid) + (int64_t)row * g.ld_resid + in_row);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = TypeTraits<T>::from_f32(TypeTraits<T>::to_f32(r[e]) * TypeTraits<T>::to_f32(gv[e]) + TypeTraits<T>::to_f32(rv[e]));
+  }
   return r;
 }
 
@@ -335,7 +350,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
       int gr = m0 + row, gc = n0 + cvec;
       if (gr < g.M && gc < g.N) {
         V8 v = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
-        if (EP) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc);
+        if (EP) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc, gr);
         *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = v;
       }
     }
@@ -352,7 +367,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m,
         if (row < g.M && col < g.N) {
           const int64_t off = epi_offset(g, bt, row, col);
           T v = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][e]) : acc[i][j][e]);
-          if (EP) v = ep_value<T>(g, v, off - (int64_t)row * g.ldc);
+          if (EP) v = ep_value<T>(g, v, off - (int64_t)row * g.ldc, row);
           C[off] = v;
         }
       }
@@ -646,7 +661,7 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
     const int gr = m0 + row, gc = n0 + cvec;
     if (gr < g.M && gc < g.N) {
       V8 v = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
-      if (EP) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc);
+      if (EP) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc, gr);
       *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = v;
     }
   }
@@ -705,7 +720,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) 
       if (row < g.M && col < g.N) {
         const int64_t off = epi_offset(g, bt, row, col);
         float v = g.sat8 ? sat8_rne(acc[i][j]) : acc[i][j];
-        if (g.bias || g.act) v = ep_value<float>(g, v, off - (int64_t)row * g.ldc);
+        if (g.bias || g.act || g.gate || g.resid) v = ep_value<float>(g, v, off - (int64_t)row * g.ldc, row);
         C[off] = v;
       }
     }
@@ -728,11 +743,11 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   int a_vec = aligned(g.A, 16) && g.lda % 8 == 0 && g.sA % 8 == 0;
   int b_vec = aligned(g.B, 16) && g.ldb % 8 == 0 && g.sB % 8 == 0;
   int c_vec = g.epi == EPI_PLAIN && g.cn == 1 && aligned(g.C, 16) && g.ldc % 8 == 0 && g.sC % 8 == 0 && g.N % 8 == 0 &&
-              (!g.bias || aligned(g.bias, 16));
+              (!g.bias || aligned(g.bias, 16)) && (!g.gate || (aligned(g.gate, 16) && g.ld_gate % 8 == 0)) && (!g.resid || (aligned(g.resid, 16) && g.ld_resid % 8 == 0));
   size_t lds = 2 * sizeof(GemmSmem<T, BM, BN>);
   // k-tiles of global loads kept in flight (tuning aid: BLR_GEMM_PD = 1, 2 or 3)
   static const int pd = [] { const char* e = getenv("BLR_GEMM_PD"); return e ? atoi(e) : 2; }();
-  const bool ep = g.bias != nullptr || g.act != 0;
+  const bool ep = g.bias != nullptr || g.act != 0 || g.gate != nullptr || g.resid != nullptr;
   void* fn = g.b_kn ? mfma_kernel_ptr<T, BM, BN, true>(pd, ep) : mfma_kernel_ptr<T, BM, BN, false>(pd, ep);
   static std::mutex mu;
   static std::set<void*> raised;
@@ -808,8 +823,8 @@ static bool ring_ok(const GemmArgs& g) {
   if (g.epi != EPI_PLAIN || g.cn < 1 || g.N < 8 || g.N % 8 || g.K % 8) return false;
   if (!aligned(g.A, 16) || !aligned(g.B, 16) || g.lda % 8 || g.sA % 8 || g.ldb % 8 || g.sB % 8) return false;
   if (g.cn == 1) {                                   // 16-byte stores, the fused output stage reads its vector the same way
-    if (!aligned(g.C, 16) || (g.bias && !aligned(g.bias, 16)) || g.ldc % 8 || g.sC % 8) return false;
-  } else if (g.bias || g.act) {
+    if (!aligned(g.C, 16) || (g.bias && !aligned(g.bias, 16)) || (g.gate && (!aligned(g.gate, 16) || g.ld_gate % 8)) || (g.resid && (!aligned(g.resid, 16) || g.ld_resid % 8)) || g.ldc % 8 || g.sC % 8) return false;
+  } else if (g.bias || g.act || g.gate || g.resid) {
     return false;                                    // interleaved columns are stored one by one, without an output stage
   }
   const int64_t lim = (int64_t)1 << 32;
@@ -822,7 +837,7 @@ template <typename T, int BM, int BN, bool SHALLOW = false, int NWV = 4, bool PA
 static int launch_ring(const GemmArgs& g, hipStream_t st) {
   int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
   const size_t lds = ring_lds_bytes<BM, BN, SHALLOW>();
-  const bool ep = g.bias != nullptr || g.act != 0;
+  const bool ep = g.bias != nullptr || g.act != 0 || g.gate != nullptr || g.resid != nullptr;
   void* fn;
   if constexpr (PARTIAL)
     fn = g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW, NWV, true> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW, NWV, true>;
@@ -867,7 +882,7 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   // BLR_GEMM_RING_WAVES = 4 or 8 the workgroup size of the two larger ones - options that tests switch with
   // blr_set_option).
   const int ring = option_value(OPT_GEMM_RING, 1);
-  if (ring > 0 && force == 0 && ring_ok(g) && g.splitk_ws && g.batch == 1 && g.cn == 1 && !g.sat8 && !g.bias && !g.act) {
+  if (ring > 0 && force == 0 && ring_ok(g) && g.splitk_ws && g.batch == 1 && g.cn == 1 && !g.sat8 && !g.bias && !g.act && !g.gate && !g.resid) {
     // few tiles, long reduction: slices of K as the batch of the partial-sum kernel, then one pass that adds them up
     int kc = 0;
     const int splits = option_value(OPT_GEMM_SPLITK, 1) == 0 ? 1 : splitk_plan(g.M, g.N, g.K, &kc);
@@ -925,7 +940,7 @@ int gemm_launch(const GemmArgs& g, int dtype, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0 || g.K <= 0 || g.batch <= 0) { set_error("gemm: empty problem"); return BLR_ERR_BAD_ARG; }
   // A handful of rows is a weight-streaming problem, not a tiling problem: plain products with (k, n)-ordered weights go to
   // the slab kernel of the decode path (it declines what it cannot take, e.g. a reduction deeper than one slab here).
-  if (g.M <= 16 && g.b_kn && g.cn == 1 && g.epi == EPI_PLAIN && !g.sat8 && !g.bias && g.act == 0 && (dtype == BLR_F16 || dtype == BLR_BF16)) {
+  if (g.M <= 16 && g.b_kn && g.cn == 1 && g.epi == EPI_PLAIN && !g.sat8 && !g.bias && g.act == 0 && !g.gate && !g.resid && (dtype == BLR_F16 || dtype == BLR_BF16)) {
     int rc = slab_gemm_launch(g.A, g.lda, g.sA, g.B, g.ldb, g.sB, g.C, g.ldc, g.sC, g.M, g.N, g.K, g.batch, dtype, nullptr, 1, st);
     if (rc != 1) return rc;
   }

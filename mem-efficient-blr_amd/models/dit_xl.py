@@ -21,6 +21,18 @@ def modulate(x, shift, scale):
     return torch.addcmul(shift.unsqueeze(1), x, (1 + scale).unsqueeze(1))
 
 
+def _gated(linear, h, gate, residual):
+    """residual + gate.unsqueeze(1) * linear(h) (reference DiT/models.py:120-121).  A structured linear that fuses its output stage
+    does the whole update while it writes its result; anything else gets one elementwise pass."""
+    if gate is None:
+        return linear(h)
+    if getattr(linear, "fuses", False):
+        from triton_funcs import _lib as L
+        with L.gate_residual(gate, h.shape[1], residual):
+            return linear(h).reshape(residual.shape)
+    return torch.addcmul(residual, gate.unsqueeze(1), linear(h))
+
+
 class TimestepEmbedder(nn.Module):
     def __init__(self, hidden, freq_dim=256):
         super().__init__()
@@ -42,11 +54,12 @@ class Attention(nn.Module):
         self.qkv = nn.Linear(dim, dim * 3, bias=True)
         self.proj = nn.Linear(dim, dim, bias=True)
 
-    def forward(self, x):
+    def forward(self, x, gate=None, residual=None):
+        """attention(x), or residual + gate * attention(x) with the update done by the last linear's output stage."""
         B, N, C = x.shape
         qkv = self.qkv(x).reshape(B, N, 3, self.heads, C // self.heads).permute(2, 0, 3, 1, 4)
         o = F.scaled_dot_product_attention(qkv[0], qkv[1], qkv[2])
-        return self.proj(o.transpose(1, 2).reshape(B, N, C))
+        return _gated(self.proj, o.transpose(1, 2).reshape(B, N, C), gate, residual)
 
 
 class Mlp(nn.Module):
@@ -56,11 +69,11 @@ class Mlp(nn.Module):
         self.act = nn.GELU(approximate="tanh")
         self.fc2 = nn.Linear(hidden, dim)
 
-    def forward(self, x):
+    def forward(self, x, gate=None, residual=None):
         h = self.fc1(x)
         if getattr(self.fc1, "fused_act", None) is None:     # a structured fc1 applies the GELU in its kernel's output stage
             h = self.act(h)
-        return self.fc2(h)
+        return _gated(self.fc2, h, gate, residual)
 
 
 class DiTBlock(nn.Module):
@@ -75,8 +88,8 @@ class DiTBlock(nn.Module):
     def forward(self, x, c):
         s1, c1, g1, s2, c2, g2 = self.adaLN_modulation(c).chunk(6, dim=1)
         # gate and residual (reference DiT/models.py:120-121) in one elementwise pass each
-        x = torch.addcmul(x, g1.unsqueeze(1), self.attn(modulate(self.norm1(x), s1, c1)))
-        x = torch.addcmul(x, g2.unsqueeze(1), self.mlp(modulate(self.norm2(x), s2, c2)))
+        x = self.attn(modulate(self.norm1(x), s1, c1), gate=g1, residual=x)
+        x = self.mlp(modulate(self.norm2(x), s2, c2), gate=g2, residual=x)
         return x
 
 

@@ -47,10 +47,12 @@ class _StructuredLinear(nn.Module):
 
     def _call(self, *args):
         """The forward function; library kernels take bias and activation into their output stage."""
-        if not self.fuses or (self.bias is None and self.fused_act is None):
+        if not self.fuses:
             return self.func(*args), False
         from triton_funcs import _lib as L
-        with L.fused_epilogue(self.bias, self.fused_act):
+        if self.bias is None and self.fused_act is None and getattr(L._ep_state, "outer", None) is None:
+            return self.func(*args), False
+        with L.fused_epilogue(self.bias, self.fused_act):          # (also picks up a gate / residual armed by the caller)
             return self.func(*args), True
 
     def _finish(self, out, fused=False):

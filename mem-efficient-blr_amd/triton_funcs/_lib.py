@@ -49,6 +49,10 @@ _SIGNATURES = {
     "blr_monarch_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 9 + [_vp, _sz, _vp, _vp, _i]),
     "blr_low_rank_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 6 + [_vp, _sz, _vp, _vp, _i]),
     "blr_dense_fwd_ep": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp, _vp, _i]),
+    "blr_blast_fwd_ep2": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64] + [_i] * 9 + [_vp, _sz, _vp, _vp, _i, _vp, _i, _i64, _vp, _i64]),
+    "blr_monarch_fwd_ep2": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 9 + [_vp, _sz, _vp, _vp, _i, _vp, _i, _i64, _vp, _i64]),
+    "blr_low_rank_fwd_ep2": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 6 + [_vp, _sz, _vp, _vp, _i, _vp, _i, _i64, _vp, _i64]),
+    "blr_dense_fwd_ep2": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp, _vp, _i, _vp, _i, _i64, _vp, _i64]),
     "blr_workspace_status": (_i, [_vp, _sz, _vp]),
     "blr_set_spin_limit": (None, [_c.c_uint]),
     "blr_set_option": (_i, [_c.c_char_p, _i, _i]),
@@ -204,15 +208,41 @@ def require_gpu(*tensors):
 _ep_state = threading.local()
 
 
+class gate_residual:
+    """with gate_residual(gate, gate_rows, residual): the next fused_epilogue context (i.e. the next wrapper-module call) on this
+    thread also multiplies by the gate and adds the residual."""
+
+    def __init__(self, gate, gate_rows, residual):
+        self.value = (gate, int(gate_rows), residual)
+
+    def __enter__(self):
+        _ep_state.outer = self.value
+        return self
+
+    def __exit__(self, *exc):
+        _ep_state.outer = None
+        return False
+
+
 class fused_epilogue:
-    def __init__(self, bias=None, act=None):
+    """with fused_epilogue(bias, act, gate=None, gate_rows=0, residual=None): the next structured-linear call returns
+    residual + gate[row // gate_rows] * act(op(x) + bias)   (gate (groups, out_f), residual (N, out_f); either may be None)."""
+
+    def __init__(self, bias=None, act=None, gate=None, gate_rows=0, residual=None):
         if act not in ACTS:
             raise BlrError(f"unknown activation {act!r}")
-        self.bias, self.act = bias, ACTS[act]
+        if gate is not None and gate_rows <= 0:
+            raise BlrError("a gate needs gate_rows > 0 (rows of the result that share one row of the gate)")
+        self.bias, self.act, self.gate, self.gate_rows, self.residual = bias, ACTS[act], gate, int(gate_rows), residual
 
     def __enter__(self):
         self.prev = getattr(_ep_state, "ep", None)
-        _ep_state.ep = (self.bias, self.act) if (self.bias is not None or self.act) else None
+        outer = getattr(_ep_state, "outer", None)
+        if outer is not None and self.gate is None and self.residual is None:
+            self.gate, self.gate_rows, self.residual = outer
+            _ep_state.outer = None
+        on = self.bias is not None or self.act or self.gate is not None or self.residual is not None
+        _ep_state.ep = (self.bias, self.act, self.gate, self.gate_rows, self.residual) if on else None
         return self
 
     def __exit__(self, *exc):
@@ -221,13 +251,23 @@ class fused_epilogue:
 
 
 def pending_epilogue(out_f, dtype, device):
-    """(bias pointer or None, activation code, keep-alive) of the active context, or None."""
+    """(bias pointer or None, activation code, keep-alive, (gate pointer, gate_rows, ld_gate, residual pointer, ld_residual)) of the
+    active context, or None."""
     ep = getattr(_ep_state, "ep", None)
     if ep is None:
         return None
-    bias, act = ep
+    bias, act, gate, gate_rows, resid = ep
     if bias is not None:
         if bias.numel() != out_f:
             raise BlrError(f"bias has {bias.numel()} values, the operator {out_f} outputs")
         bias = bias.detach().to(device=device, dtype=dtype).contiguous()
-    return (bias.data_ptr() if bias is not None else None), act, bias
+    extra = [None, 0, 0, None, 0]
+    if gate is not None:
+        gate = gate.detach().to(device=device, dtype=dtype).reshape(-1, out_f).contiguous()
+        extra[0:3] = [gate.data_ptr(), gate_rows, gate.stride(0)]
+    if resid is not None:
+        resid = resid.detach().to(device=device, dtype=dtype).reshape(-1, out_f)
+        if resid.stride(-1) != 1:
+            resid = resid.contiguous()
+        extra[3:5] = [resid.data_ptr(), resid.stride(0)]
+    return (bias.data_ptr() if bias is not None else None), act, (bias, gate, resid), tuple(extra)

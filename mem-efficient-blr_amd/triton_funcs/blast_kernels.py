@@ -73,9 +73,9 @@ def _blast(name, x, U, V, S, u_layout, s_layout, algo, want_intermediates):
     ws = L.workspace(x.device, need, algo, M, dt)
     ep = None if want_intermediates else L.pending_epilogue(out_f, x.dtype, x.device)
     if ep is not None:
-        rc = lib.blr_blast_fwd_ep(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
+        rc = lib.blr_blast_fwd_ep2(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
                                   out.data_ptr(), out.stride(0), M, in_f, out_f, b1, r, dt, u_layout, s_layout, algo,
-                                  ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1])
+                                  ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1], *ep[3])
     else:
         rc = lib.blr_blast_fwd(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
                                out.data_ptr(), out.stride(0),

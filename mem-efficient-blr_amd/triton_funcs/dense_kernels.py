@@ -29,8 +29,8 @@ def _dense(name, x, w, algo):
     ws = L.workspace(x.device, lib.blr_dense_workspace_bytes(M, in_f, out_f, dt, algo), algo, M, dt)
     ep = L.pending_epilogue(out_f, x.dtype, x.device)
     if ep is not None:
-        rc = lib.blr_dense_fwd_ep(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
-                                  M, in_f, out_f, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1])
+        rc = lib.blr_dense_fwd_ep2(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
+                                  M, in_f, out_f, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1], *ep[3])
     else:
         rc = lib.blr_dense_fwd(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
                                M, in_f, out_f, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))

@@ -31,8 +31,8 @@ def _low_rank(name, x, a, b, algo, want_z):
     ws = L.workspace(x.device, lib.blr_low_rank_workspace_bytes(M, in_f, out_f, r, dt, algo), algo, M, dt)
     ep = None if want_z else L.pending_epilogue(out_f, x.dtype, x.device)
     if ep is not None:
-        rc = lib.blr_low_rank_fwd_ep(x2.data_ptr(), x2.stride(0), a.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
-                                     M, in_f, out_f, r, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1])
+        rc = lib.blr_low_rank_fwd_ep2(x2.data_ptr(), x2.stride(0), a.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
+                                     M, in_f, out_f, r, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1], *ep[3])
     else:
         rc = lib.blr_low_rank_fwd(x2.data_ptr(), x2.stride(0), a.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
                                   z.data_ptr() if z is not None else None,

@@ -57,9 +57,9 @@ def _monarch(name, x, w1, w2, w2_layout, out_order, algo, want_out1):
     ws = L.workspace(x.device, lib.blr_monarch_workspace_bytes(M, in_f, out_f, k, q, dt, algo), algo, M, dt)
     ep = None if want_out1 else L.pending_epilogue(out_f, x.dtype, x.device)
     if ep is not None:
-        rc = lib.blr_monarch_fwd_ep(x2.data_ptr(), x2.stride(0), w1.data_ptr(), w2.data_ptr(), out.data_ptr(), out.stride(0),
+        rc = lib.blr_monarch_fwd_ep2(x2.data_ptr(), x2.stride(0), w1.data_ptr(), w2.data_ptr(), out.data_ptr(), out.stride(0),
                                     M, in_f, out_f, k, q, dt, w2_layout, out_order, algo,
-                                    ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1])
+                                    ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1], *ep[3])
     else:
         rc = lib.blr_monarch_fwd(x2.data_ptr(), x2.stride(0), w1.data_ptr(), w2.data_ptr(), out.data_ptr(), out.stride(0),
                                  out1.data_ptr() if out1 is not None else None,

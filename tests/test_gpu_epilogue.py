@@ -89,6 +89,35 @@ def test_dense_low_rank_monarch_bias_activation(M, dtype):
         assert_close(out, _ref_monarch(xm, w1_t, w2_t, dtype)[0] + rounded(mb, dtype), dtype, "monarch + bias", scale=2.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [6, 300])
+def test_gate_and_residual_in_the_output_stage(M, dtype):
+    """out = residual + gate[row // rows_per_gate] * act(op(x) + bias): the adaLN-Zero update of a DiT block, fused into the
+    write-out of the last GEMM above 16 rows and done by one elementwise launch at or below."""
+    from triton_funcs import blast_kernels as K, dense_kernels as D, low_rank_kernels as LR, _lib as L
+    rng = np.random.default_rng(40 + M)
+    b, p, q, r = 4, 32, 40, 64
+    in_f, out_f, rows = b * p, b * q, 3                      # three consecutive rows share a row of the gate
+    groups = -(-M // rows)
+    x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=M)
+    bias = rng.standard_normal(out_f); gate = rng.standard_normal((groups, out_f)); resid = rng.standard_normal((M, out_f))
+    grow = np.repeat(rounded(gate, dtype), rows, axis=0)[:M]
+    Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+    say(f"[case] gate + residual, blast / dense / low rank M={M} {dtype}")
+    with L.fused_epilogue(dev(bias, dtype), "gelu_tanh", gate=dev(gate, dtype), gate_rows=rows, residual=dev(resid, dtype)):
+        out = K.triton_blast_full_fp16(dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype))
+    h = _act(O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0] + rounded(bias, dtype), "gelu_tanh")
+    assert_close(out, rounded(resid, dtype) + grow * h, dtype, "blast gate/residual", scale=2.0)
+    w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)
+    with L.fused_epilogue(None, None, gate=dev(gate, dtype), gate_rows=rows):          # a gate alone
+        out = D.triton_dense_fp16(dev(x, dtype), dev(w, dtype))
+    assert_close(out, grow * (rounded(x, dtype) @ rounded(w, dtype)), dtype, "dense gate", scale=2.0)
+    a = rng.standard_normal((in_f, r)) / np.sqrt(in_f); bm = rng.standard_normal((r, out_f)) / np.sqrt(r)
+    with L.fused_epilogue(dev(bias, dtype), None, residual=dev(resid, dtype)):         # a residual alone
+        out = LR.triton_low_rank_fp16(dev(x, dtype), dev(a, dtype), dev(bm, dtype))
+    assert_close(out, rounded(resid, dtype) + (rounded(x, dtype) @ rounded(a, dtype)) @ rounded(bm, dtype) + rounded(bias, dtype), dtype, "low rank residual", scale=2.0)
+
+
 def test_wrapper_modules_fuse_bias_and_activation():
     """BlastLinear with a bias (and an activation requested by its owner) equals the unfused computation."""
     from models import wrappers as W
