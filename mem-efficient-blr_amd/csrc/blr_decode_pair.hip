@@ -420,9 +420,11 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     const int cus = device_cus() > 0 ? device_cus() : 256;
     const int ks_max = dp_ks_max(MT);
     int ks = 1;
-    while (ks < ks_max && cdiv(cdiv(P, ks), rpp) > DP_UNR1) ++ks;
-    // finer while that gives compute units without an item one (the bytes per compute unit bound the launch)
-    while (ks < ks_max && (int64_t)b * nch * ks < cus && cdiv(cdiv(P, ks + 1), rpp) >= 2) ++ks;
+    // Few, fat items: every k-slice is one more partial y that each slab has to fetch and add in its mix, which costs more
+    // than the idle compute units of this short kernel (measured: two slices 9.0 / 14.6 us, four / three slices 9.35 / 15.6 us
+    // on 4096 -> 4096 and 11008 -> 4096).  An item may take two batches of loads; slices are added only up to half the chip.
+    while (ks < ks_max && cdiv(cdiv(P, ks), rpp) > 2 * DP_UNR1) ++ks;
+    while (ks < ks_max && (int64_t)b * nch * ks < cus / 2 && cdiv(cdiv(P, ks + 1), rpp) >= 2) ++ks;
     if (e_ks > 0) ks = e_ks < ks_max ? e_ks : ks_max;
     int kc = (int)cdiv(P, ks);
     kc = (int)cdiv(kc, rpp) * rpp;
