@@ -14,6 +14,10 @@
 //     residency requirement.
 // The number of slab loads is a template parameter: the compiler then knows how many loads follow the mix operands
 // and waits for exactly those (loads under runtime branches make it wait for everything in flight).
+// The layouts of the bmm names are served at one row as well (measured 12.0 -> 9.6, 20.2 -> 16.6 and 17.1 -> 14.0 us on the
+// three Llama-7B layers against the single-launch kernel): U as (b, q, r) by a variant of the slab kernel whose slab is a
+// run of whole rows of U_i, and S as (r, i, j) by letting launch 1 rewrite it, eight ranks per workgroup, in the order the
+// mix reads.
 #include <map>
 #include <mutex>
 #include "blr_common.h"
@@ -53,11 +57,18 @@ struct PairParams {
   FastDiv nch2;
   int xcd_order;
   const void* bias; int act, ep;                 // fused output stage: bias of T (indexed like a row of out) or null, blr_act
+  const void* s_rij; int s_chunks;               // S given as (r, i, j): stage 1 rewrites it as (j, i, r) into S, eight ranks per workgroup
 };
 
 __device__ __forceinline__ void lds_barrier2() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rbuf2(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// v + the value of v in another lane of the same row of 16 lanes (DPP control word CTRL)
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
 }
 
 // Totals over the row groups of a workgroup (see decode3_kernel): red is [m][row group][column]; every lane of a column
@@ -86,15 +97,15 @@ __device__ __forceinline__ void pair_reduce(float (&acc)[MT][EPL], int lpr_log2,
 }
 
 // ---- launch 1: y[ks][j][m][n] = sum_k x[m, j P + k] V_j[k, n] over one k-slice -------------------------------------------
-template <typename T, int MT, int WB>
+template <typename T, int MT, int WB, bool ST>
 __global__ __launch_bounds__(DP_NT) void pair_stage1_kernel(PairParams p) {
   constexpr int TR4_BASE = 0; (void)TR4_BASE;
   constexpr int EPL = 128 / WB;
   __shared__ __attribute__((aligned(16))) float a_s[4096];
   __shared__ __attribute__((aligned(16))) float red[MT * DP_NT * EPL];
   const int tid = threadIdx.x;
-  const int M = p.M;
   TR4(0);
+  const int M = p.M;
   const int lpr1 = 1 << p.lpr1_log2, rpp1 = DP_NT >> p.lpr1_log2;
   const int cv1 = tid & (lpr1 - 1), rs1 = tid >> p.lpr1_log2;
   const int kpad1 = 1 << p.kpad1_log2;
@@ -107,7 +118,17 @@ __global__ __launch_bounds__(DP_NT) void pair_stage1_kernel(PairParams p) {
   const uint32_t ks = fd_div(t1, p.bdiv), j = t1 - ks * p.bdiv.d;
   const int n0 = (int)nc1 * lpr1 * EPL;
   const int k0 = (int)ks * p.kc1, kc = min(p.kc1, p.P - k0);
-  // the activations first (loads come back in order); outside the slice the offset is out of bounds and reads as zero
+  // S as (r, i, j): the first rank / 8 workgroups turn eight ranks each into 16-byte pieces of the (j, i, r) order the mix
+  // of launch 2 reads.  Thread = (i, j); its loads go out first and its store follows the loads of V, so nothing waits.
+  const __amdgpu_buffer_rsrc_t srbuf = rbuf2(p.s_rij ? p.s_rij : p.x, p.s_rij ? (uint32_t)p.b * p.bo * p.R * 2u : 2u);
+  const bool s_on = ST && it < (uint32_t)p.s_chunks && tid < p.b * p.bo;
+  uint32_t s16[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+  if (s_on) {                                              // (a load instruction costs its turn in the memory pipeline even when every lane is out of bounds)
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      s16[e] = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(srbuf, (uint32_t)(((int)it * 8 + e) * p.b * p.bo + tid) * 2u, 0, 0);
+  }
+  // the activations next (loads come back in order); outside the slice the offset is out of bounds and reads as zero
   u32x4 xq;
   if (p.x_vec) {
     if (tid * 8 < (MT << p.kpad1_log2)) {
@@ -138,6 +159,11 @@ __global__ __launch_bounds__(DP_NT) void pair_stage1_kernel(PairParams p) {
   };
   load_batch(0);
   TR4(1);
+  if (ST && s_on) {
+    const int si = tid / p.b, sj = tid - si * p.b;       // S[r][i][j] -> S_t[j][i][r]
+    const u32x4 pk = {s16[0] | (s16[1] << 16), s16[2] | (s16[3] << 16), s16[4] | (s16[5] << 16), s16[6] | (s16[7] << 16)};
+    *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(const_cast<void*>(p.S)) + ((int64_t)(sj * p.bo + si) * p.R + (int64_t)it * 8) * 2) = pk;
+  }
   if (p.x_vec) {
     if (tid * 8 < (MT << p.kpad1_log2)) {
       const typename TypeTraits<T>::vec8 v = __builtin_bit_cast(typename TypeTraits<T>::vec8, xq);
@@ -198,24 +224,32 @@ __global__ __launch_bounds__(DP_NT) void pair_stage1_kernel(PairParams p) {
 }
 
 // ---- launch 2: z_i = sum_j S_ij * y_j, then out_i = z_i U_i over a register-resident slab ---------------------------------
-template <typename T, int MT, int WB, int PFG>
+//
+// QR: U_i is (q, r) row-major (the bmm names).  A slab is then PF * rows-per-pass whole rows of U_i, one contiguous run of
+// memory read in linear order; a lane meets the same eight ranks in every load (its z sits in registers), keeps one
+// partial dot product per load and row, and the partials of a row are added up across its lanes: two DPP steps inside
+// the quad, one pass through LDS for the rest.  Needs rank = 8 * 2^n, 128 <= rank <= 4096.
+template <typename T, int MT, int WB, int PFG, bool QR>
 __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   constexpr int TR4_BASE = 512; (void)TR4_BASE;
   constexpr int EPL = 128 / WB;
   constexpr int PF = 8 * PFG;
+  static_assert(!QR || WB == 16, "rows of U along the rank: two-byte weights only");
   constexpr int KSM = dp_ks_max(MT);                 // k-slices of stage 1 this instantiation can add up
   using V8 = typename TypeTraits<T>::vec8;
   __shared__ __attribute__((aligned(16))) float a_s[DP_AS];
   __shared__ __attribute__((aligned(16))) float red[MT * DP_NT * EPL];
   const int tid = threadIdx.x;
-  const int M = p.M, R = p.R;
   TR4(0);
+  const int M = p.M, R = p.R;
   const uint32_t w = p.xcd_order ? xcd_item(blockIdx.x, gridDim.x) : blockIdx.x;
   const uint32_t i2 = fd_div(w, p.nch2), nc2 = w - i2 * p.nch2.d;
   const int lpr2 = 1 << p.lpr2_log2, rpp2 = DP_NT >> p.lpr2_log2;
   const int cv2 = tid & (lpr2 - 1), rs2 = tid >> p.lpr2_log2;
   const int n0_2 = (int)nc2 * lpr2 * EPL;
   const int n2 = n0_2 + cv2 * EPL;
+  const int rppq = DP_NT >> p.octs_log2;               // QR: rows of U a load of the workgroup covers
+  const int q0 = (int)nc2 * PF * rppq;                 // QR: first row of the slab
 
   // ---- mix operands of this thread: 8 ranks (one 16-byte piece) of y and S for up to DP_JJ input blocks ----
   const int oct = tid & ((1 << p.octs_log2) - 1), jg = tid >> p.octs_log2;
@@ -239,14 +273,16 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   }
   // ---- the whole slab of U right behind, in straight-line code: the compiler counts exactly these PF loads ----
   const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)((int64_t)p.bo * R * p.Q * WB / 8));
-  const uint32_t uoff = (uint32_t)((((int)i2 * R + rs2) * p.Q + (n2 < p.Q ? n2 : 0))) * (uint32_t)WB / 8u;
-  const uint32_t ustep = (uint32_t)rpp2 * (uint32_t)p.Q * (uint32_t)WB / 8u;
+  const uint32_t uoff = QR ? (uint32_t)(((int)i2 * p.Q + q0 + jg) * R + oct * 8) * 2u
+                            : (uint32_t)((((int)i2 * R + rs2) * p.Q + (n2 < p.Q ? n2 : 0))) * (uint32_t)WB / 8u;
+  const uint32_t ustep = QR ? (uint32_t)DP_NT * 16u : (uint32_t)rpp2 * (uint32_t)p.Q * (uint32_t)WB / 8u;
+  auto u_on = [&](int u) { return QR ? q0 + u * rppq + jg < p.Q : u < p.pfn; };   // QR: rows past the block are not read
   // A wave that asks for more than the memory path of its compute unit takes at once is held at the load until there
   // is room, so only the first eight loads go out before the mix; the rest follow group by group, each behind the
   // products of the group before (whose data has landed by then: loads come back in order).
   u32x4 pf[PF];
 #pragma unroll
-  for (int u = 0; u < 8; ++u) pf[u] = ldw16(ubuf, u < p.pfn ? uoff : DP_OOB, (uint32_t)u * ustep);
+  for (int u = 0; u < 8; ++u) pf[u] = ldw16(ubuf, u_on(u) ? uoff : DP_OOB, (uint32_t)u * ustep);
   TR4(1);
 
   // ---- mix: this thread's partial z over its input blocks, to LDS as [jg][m][r] (in `red`), then summed into a_s ----
@@ -296,6 +332,100 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   lds_barrier2();
   TR4(2);
 
+  auto store_out = [&](int m, int gn, float total) {       // one element of out: scale of the codes, fused bias / activation
+    float usc = 1.0f;
+    if constexpr (WB != 16) usc = (float)p.u_scales[(int64_t)i2 * p.Q + gn];
+    const int64_t oc = (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns;
+    T r = TypeTraits<T>::from_f32(total * usc);
+    if (p.ep) {                                            // on the rounded result, as a separate elementwise kernel would see it
+      float v = TypeTraits<T>::to_f32(r);
+      if (p.bias) v += TypeTraits<T>::to_f32(reinterpret_cast<const T*>(p.bias)[oc]);
+      r = TypeTraits<T>::from_f32(apply_act(v, p.act));
+    }
+    reinterpret_cast<T*>(p.out)[(int64_t)m * p.ldo + oc] = r;
+  };
+  if constexpr (QR) {
+    // ---- rows of U along the rank: one partial dot product per load and token row ----
+    float zr[MT][8];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(&a_s[(m << p.kld2_log2) + oct * 8]);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(&a_s[(m << p.kld2_log2) + oct * 8 + 4]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { zr[m][e] = lo[e]; zr[m][4 + e] = hi[e]; }
+    }
+    float part[MT][PF];
+#pragma unroll
+    for (int g = 0; g < PFG; ++g) {
+      if (g + 1 < PFG) {
+#pragma unroll
+        for (int v = 0; v < 8; ++v) { const int u = (g + 1) * 8 + v; pf[u] = ldw16(ubuf, u_on(u) ? uoff : DP_OOB, (uint32_t)u * ustep); }
+      }
+#pragma unroll
+      for (int v = 0; v < 8; ++v) {
+        const int u = g * 8 + v;
+        float wv[8];
+        cvtw<T, 16>(pf[u], wv);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          float s = 0.0f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) s = fmaf(zr[m][e], wv[e], s);
+          part[m][u] = s;
+        }
+      }
+    }
+    TR4(3);
+    // quad totals, then lane c of a quad keeps load 4 g + c: `red` holds [m][g][quad][c], written in thread order
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int g4 = 0; g4 < PF / 4; ++g4) {
+        float keep = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          float v = part[m][g4 * 4 + c];
+          v = dpp_add<0xB1>(v);                            // lanes 1 0 3 2
+          v = dpp_add<0x4E>(v);                            // lanes 2 3 0 1
+          keep = (tid & 3) == c ? v : keep;
+        }
+        red[(m * (PF / 4) + g4) * DP_NT + tid] = keep;
+      }
+    lds_barrier2();
+    // a group of threads adds the quads of four rows (loads 4 g .. 4 g + 3 of one row slot) as 16-byte pieces
+    const int nv_log2 = p.octs_log2 - 2;                   // quads per row of U
+    const int tpg_log2 = nv_log2 < 4 ? nv_log2 : 4, tpg = 1 << tpg_log2;
+    const int k = tid & (tpg - 1);
+    const int ngroups = (PF / 4) * rppq;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      if (m >= M) break;
+      for (int gi = tid >> tpg_log2; gi < ngroups; gi += DP_NT >> tpg_log2) {
+        const int g4 = gi >> (9 - p.octs_log2), rw = gi & (rppq - 1);
+        const float* src = &red[(m * (PF / 4) + g4) * DP_NT + ((rw << nv_log2) << 2)];
+        f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int qd = k; qd < (1 << nv_log2); qd += tpg) s += *reinterpret_cast<const f32x4*>(src + qd * 4);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          float v = s[c];
+          v = dpp_add<0xB1>(v);
+          v = dpp_add<0x4E>(v);
+          if (tpg_log2 >= 3) v = dpp_add<0x141>(v);        // the other quad of eight lanes (row_half_mirror)
+          if (tpg_log2 >= 4) v = dpp_add<0x140>(v);        // the other half of sixteen lanes (row_mirror)
+          s[c] = v;
+        }
+        if (k == 0) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int gn = q0 + (g4 * 4 + c) * rppq + rw;
+            if (gn < p.Q) store_out(m, gn, s[c]);
+          }
+        }
+      }
+    }
+    TR4(4);
+    return;
+  }
   // ---- products over the register-resident slab, eight loads at a time ----
   float acc[MT][EPL];
 #pragma unroll
@@ -307,7 +437,7 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   for (int g = 0; g < PFG; ++g) {
     if (g + 1 < PFG) {
 #pragma unroll
-      for (int v = 0; v < 8; ++v) { const int u = (g + 1) * 8 + v; pf[u] = ldw16(ubuf, u < p.pfn ? uoff : DP_OOB, (uint32_t)u * ustep); }
+      for (int v = 0; v < 8; ++v) { const int u = (g + 1) * 8 + v; pf[u] = ldw16(ubuf, u_on(u) ? uoff : DP_OOB, (uint32_t)u * ustep); }
     }
 #pragma unroll
     for (int h = 0; h < 8 / GV; ++h) {
@@ -334,21 +464,9 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   const int sub2_log2 = 9 - (p.lpr2_log2 + ilog2k(EPL));
   const int gn = n0_2 + (tid >> sub2_log2);
   if ((tid & ((1 << sub2_log2) - 1)) == 0 && gn < p.Q) {
-    float usc = 1.0f;                                    // per-output scale of the codes of U
-    if constexpr (WB != 16) usc = (float)p.u_scales[(int64_t)i2 * p.Q + gn];
-    T* outp = reinterpret_cast<T*>(p.out);
 #pragma unroll
     for (int m = 0; m < MT; ++m)
-      if (m < M) {
-        const int64_t oc = (int64_t)i2 * p.o_bs + (int64_t)gn * p.o_ns;
-        T r = TypeTraits<T>::from_f32(tot[m] * usc);
-        if (p.ep) {                                      // on the rounded result, as a separate elementwise kernel would see it
-          float v = TypeTraits<T>::to_f32(r);
-          if (p.bias) v += TypeTraits<T>::to_f32(reinterpret_cast<const T*>(p.bias)[oc]);
-          r = TypeTraits<T>::from_f32(apply_act(v, p.act));
-        }
-        outp[(int64_t)m * p.ldo + oc] = r;
-      }
+      if (m < M) store_out(m, gn, tot[m]);
   }
   TR4(4);
 }
@@ -356,28 +474,40 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
 // ---- host side --------------------------------------------------------------------------------------------------
 namespace {
 template <typename T, int MT, int WB>
-void* pair_slab_fn(int pfg) {
+void* pair_slab_fn(int pfg, bool qr) {
+  if constexpr (WB == 16) {
+    if (qr) {
+      switch (pfg) {
+        case 1: return (void*)pair_slab_kernel<T, MT, 16, 1, true>;
+        case 2: return (void*)pair_slab_kernel<T, MT, 16, 2, true>;
+        case 3: if constexpr (MT <= 2) return (void*)pair_slab_kernel<T, MT, 16, 3, true>; else return nullptr;
+        case 4: if constexpr (MT <= 2) return (void*)pair_slab_kernel<T, MT, 16, 4, true>; else return nullptr;
+        default: return nullptr;
+      }
+    }
+  }
+  if (qr) return nullptr;
   switch (pfg) {
-    case 1: return (void*)pair_slab_kernel<T, MT, WB, 1>;
-    case 2: return (void*)pair_slab_kernel<T, MT, WB, 2>;
-    case 3: if constexpr (WB == 16) return (void*)pair_slab_kernel<T, MT, WB, 3>; else return nullptr;
-    case 4: if constexpr (WB == 16) return (void*)pair_slab_kernel<T, MT, WB, 4>; else return nullptr;
+    case 1: return (void*)pair_slab_kernel<T, MT, WB, 1, false>;
+    case 2: return (void*)pair_slab_kernel<T, MT, WB, 2, false>;
+    case 3: if constexpr (WB == 16) return (void*)pair_slab_kernel<T, MT, WB, 3, false>; else return nullptr;
+    case 4: if constexpr (WB == 16) return (void*)pair_slab_kernel<T, MT, WB, 4, false>; else return nullptr;
     default: return nullptr;
   }
 }
 // two-byte weights at 1, 2 and 4 token rows, int8 codes at 1 and 2, int4 codes at 1 (as decode3_kernel)
 template <typename T>
-bool pair_fns(int MT, int wbits, int pfg, void** f1, void** f2) {
+bool pair_fns(int MT, int wbits, int pfg, bool qr, bool st, void** f1, void** f2) {
   *f1 = *f2 = nullptr;
   if (wbits == 16) {
-    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 16>; *f2 = pair_slab_fn<T, 1, 16>(pfg); }
-    else if (MT == 2) { *f1 = (void*)pair_stage1_kernel<T, 2, 16>; *f2 = pair_slab_fn<T, 2, 16>(pfg); }
-    else { *f1 = (void*)pair_stage1_kernel<T, 4, 16>; *f2 = pair_slab_fn<T, 4, 16>(pfg); }
+    if (MT == 1) { *f1 = st ? (void*)pair_stage1_kernel<T, 1, 16, true> : (void*)pair_stage1_kernel<T, 1, 16, false>; *f2 = pair_slab_fn<T, 1, 16>(pfg, qr); }
+    else if (MT == 2) { *f1 = st ? (void*)pair_stage1_kernel<T, 2, 16, true> : (void*)pair_stage1_kernel<T, 2, 16, false>; *f2 = pair_slab_fn<T, 2, 16>(pfg, qr); }
+    else { *f1 = st ? (void*)pair_stage1_kernel<T, 4, 16, true> : (void*)pair_stage1_kernel<T, 4, 16, false>; *f2 = pair_slab_fn<T, 4, 16>(pfg, qr); }
   } else if (wbits == 8) {
-    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 8>; *f2 = pair_slab_fn<T, 1, 8>(pfg); }
-    else if (MT == 2) { *f1 = (void*)pair_stage1_kernel<T, 2, 8>; *f2 = pair_slab_fn<T, 2, 8>(pfg); }
+    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 8, false>; *f2 = pair_slab_fn<T, 1, 8>(pfg, qr); }
+    else if (MT == 2) { *f1 = (void*)pair_stage1_kernel<T, 2, 8, false>; *f2 = pair_slab_fn<T, 2, 8>(pfg, qr); }
   } else if (wbits == 4) {
-    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 4>; *f2 = pair_slab_fn<T, 1, 4>(pfg); }
+    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 4, false>; *f2 = pair_slab_fn<T, 1, 4>(pfg, qr); }
   }
   return *f1 && *f2;
 }
@@ -392,7 +522,10 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   if (M < 1 || M > 4) return 1;
   if (a.wbits == 8 && M > 2) return 1;              // codes at more rows: the matrix-core kernel
   if (a.wbits == 4 && M > 1) return 1;
-  if (a.u_layout != BLR_U_RQ || a.perm_per > 0) return 1;      // U (b, q, r) and Monarch: the single-launch kernels
+  if (a.perm_per > 0) return 1;                     // Monarch: the single-launch kernels
+  const bool qr = a.u_layout == BLR_U_QR;           // U (b, q, r): two-byte weights with a power-of-two rank of at least 128
+  if (qr && (a.wbits != 16 || R < 128 || (R & (R - 1)))) return 1;
+  if (!qr && a.u_layout != BLR_U_RQ) return 1;
   if (b > 16 * DP_JJ || b >= 65536 || bo >= 65536 || R % 8 || R > 4096) return 1;
   if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return 1;
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
@@ -406,7 +539,14 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
-  if (a.S && (p.s_sr != 1 || !aligned(a.S, 16))) return 1;     // S in 16-byte pieces along the rank
+  // S as (r, i, j) with two-byte weights: rewritten by launch 1 into the scratch region as (j, i, r).  (Codes come with S in
+  // that order too; they stay on the single-launch kernel, which measured 0.3 - 0.5 us faster on them.)
+  const bool s_turn = a.S && a.s_layout == BLR_S_RIJ && a.wbits == 16;
+  if (s_turn) {
+    if (b * bo > DP_NT) return 1;
+    p.s_sj = (int64_t)bo * R; p.s_si = R; p.s_sr = 1;
+  }
+  if (a.S && !s_turn && (p.s_sr != 1 || !aligned(a.S, 16))) return 1;     // S in 16-byte pieces along the rank
   p.x_vec = aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0;
 
   // ---- stage 1: 128-rank chunks, k split so that an item is at most eight loads per lane; any number of workgroups ----
@@ -439,9 +579,15 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   }
   { static const int e_xcd = env_i("BLR_XCD_ORDER", 1); p.xcd_order = e_xcd; }
   { const void* eb = nullptr; int ea = 0; if (epilogue_pending(&eb, &ea)) { p.ep = 1; p.bias = eb; p.act = ea; } }
-  const size_t ybytes = (size_t)p.ks1 * b * M * R * 2;
-  if (ybytes > region_bytes) return d2_bail(__LINE__);
+  const size_t ybytes = ((size_t)p.ks1 * b * M * R * 2 + 255) / 256 * 256;
+  const size_t sbytes = s_turn ? (size_t)b * bo * R * 2 : 0;
+  if (ybytes + sbytes > region_bytes) return d2_bail(__LINE__);
   p.y = region;
+  if (s_turn) {
+    p.s_rij = a.S; p.s_chunks = R / 8;
+    p.S = reinterpret_cast<char*>(region) + ybytes;
+    if (b * (int)p.nch1.d * p.ks1 < p.s_chunks) return 1;       // one chunk of S per workgroup of launch 1
+  }
 
   // ---- mix + stage 2: a slab spans the whole rank; the narrowest column chunk that keeps it within the registers ----
   {
@@ -449,7 +595,15 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     const int cus = device_cus() > 0 ? device_cus() : 256;
     int best_lpr = 0, best_pfn = 0;
     double best = 1e30;
-    for (int lpr0 = 16; lpr0 >= 4; lpr0 >>= 1) {
+    if (qr) {                                          // whole rows of U_i: 8, 16, 24 or 32 loads per lane of 8 KiB per workgroup each
+      const int rppq = DP_NT / (R / 8);
+      for (int pfn = 8; pfn <= (MT <= 2 ? 32 : 16); pfn += 8) {
+        const int nch = (int)cdiv(Q, pfn * rppq);
+        const double est = (double)cdiv((int64_t)bo * nch, cus) * (0.6 + pfn * 8192.0 / 35e3);
+        if (est < best) { best = est; best_lpr = 16; best_pfn = pfn; p.nch2 = fd_make((uint32_t)nch); }
+      }
+    }
+    for (int lpr0 = 16; lpr0 >= 4 && !qr; lpr0 >>= 1) {
       if (e_lpr > 0 && lpr0 != e_lpr) continue;
       if (lpr0 == 4 && WBITS == 16 && e_lpr != 4) continue;        // 64-byte pieces of a row only for codes
       int lpr = lpr0;
@@ -485,11 +639,11 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     // runs stage 1 under that stream: 16.3 against 17.5 us at 4096 -> 22016, rank 1024; below that the two launches win
     // (9.5 against 10.6 us at 4096 -> 4096, rank 512).  BLR_DECODE_PAIR=2 takes every call this path can serve.
     const double slab_bytes = (double)p.pfn * (DP_NT >> p.lpr2_log2) * (1 << p.lpr2_log2) * 16.0;
-    if (enabled != 2 && slab_bytes > 192.0 * 1024.0 && a.S && a.perm_per == 0 && bo > 1) return 1;
+    if (enabled != 2 && !qr && slab_bytes > 192.0 * 1024.0 && a.S && a.perm_per == 0 && bo > 1) return 1;
   }
   const int pfg = (p.pfn + 7) / 8;
   void *f1 = nullptr, *f2 = nullptr;
-  const bool have = a.dtype == BLR_F16 ? pair_fns<f16>(MT, WBITS, pfg, &f1, &f2) : pair_fns<bf16>(MT, WBITS, pfg, &f1, &f2);
+  const bool have = a.dtype == BLR_F16 ? pair_fns<f16>(MT, WBITS, pfg, qr, s_turn, &f1, &f2) : pair_fns<bf16>(MT, WBITS, pfg, qr, s_turn, &f1, &f2);
   if (!have) return d2_bail(__LINE__);
   const int grid1 = b * (int)p.nch1.d * p.ks1, grid2 = bo * (int)p.nch2.d;
   static const int dbg = env_i("BLR_D2_DEBUG", 0);

@@ -133,6 +133,28 @@ def test_blast_llama7b_decode(name, layer, M):
         assert_close(out, _ref(x, U, Vt, S, torch.float16)[0], torch.float16, f"{layer}/{name}/{algo}/M{M}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(16, 64, 72, 128), (4, 32, 40, 256), (8, 64, 100, 512), (16, 48, 1376, 1024), (2, 40, 24, 2048)],
+                         ids=lambda s: "b%d-p%d-q%d-r%d" % s)
+def test_blast_bmm_single_row_power_of_two_rank(shape, dtype):
+    """One token row of the bmm names (U as (b, q, r), S as (r, i, j)) at ranks 8 * 2^n: two launches, the second reads whole
+    rows of U_i (the last slab of a block is ragged at these q) and the first rewrites S for it.  With and without a fused
+    bias + activation."""
+    from triton_funcs import blast_kernels as K, _lib as L
+    b, p, q, r = shape
+    say(f"[case] bmm single row b={b} p={p} q={q} r={r} {dtype}")
+    x, U, Vt, S = blast_inputs(b, p, q, r, (1,), seed=5)
+    ref = _ref(x, U, Vt, S, dtype)[0]
+    out = _run_blast("triton_blast_bmm_fp16", x, U, Vt, S, dtype, "auto")
+    assert_close(out, ref, dtype, "bmm M=1")
+    bias = np.random.default_rng(5).standard_normal(b * q)
+    Uk, Vk, Sk = O.blast_to_bmm_layout(U, Vt, S)
+    with L.fused_epilogue(dev(bias, dtype), "silu"):
+        out = K.triton_blast_bmm_fp16(dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype))
+    v = ref + rounded(bias, dtype)
+    assert_close(out, v / (1.0 + np.exp(-v)), dtype, "bmm M=1 + bias + silu")
+
+
 @pytest.mark.parametrize("layer", list(LLAMA))
 @pytest.mark.parametrize("name", ["triton_blast_full_fp16", "triton_blast_bmm_fp16"])
 def test_blast_llama7b_prefill_rows(name, layer):

@@ -131,7 +131,8 @@ def _spinning_cases(dtype):
     return {
         # a permutation period of 254 (not a multiple of 4) keeps this call on the single-launch kernels
         "monarch_m8": _monarch_case(4, 1024, 1016, 1024, 8, dtype, 60),
-        "blast_bmm_m1": _blast_case(16, 256, 256, 512, 1, "triton_blast_bmm_fp16", dtype, 61),
+        # U as (b, q, r) with a rank that is not a power of two: the single-launch kernel (its workgroups hand y and z over)
+        "blast_bmm_m1": _blast_case(16, 256, 256, 480, 1, "triton_blast_bmm_fp16", dtype, 61),
         # 4104 input features cannot be cut into equal blocks of whole 16-byte pieces: the phase engine serves the call
         # (one launch, a barrier of the whole grid between the two products)
         "low_rank_phases_m1": _low_rank_case(4104, 4096, 512, 1, dtype, 62),

@@ -24,23 +24,25 @@ def _operands(b, p, q, r, M, dtype, seed):
     return dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype), ref
 
 
-def _call_static(L, x, U, V, S, b, r):
+def _call_static(L, x, U, V, S, b, r, layouts=None):
     M, in_f = x.shape
-    out_f = b * U.shape[2]
+    ul, sl = layouts or (L.U_RQ, L.S_JIR)
+    out_f = b * (U.shape[2] if ul == L.U_RQ else U.shape[1])
     out = torch.full((M, out_f), float("nan"), device=x.device, dtype=x.dtype)
     rc = L.lib().blr_blast_fwd_static(x.data_ptr(), x.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(), out.data_ptr(), out.stride(0),
-                                      M, in_f, out_f, b, r, L.dtype_code(x.dtype), L.U_RQ, L.S_JIR, L.stream_ptr(x.device))
+                                      M, in_f, out_f, b, r, L.dtype_code(x.dtype), ul, sl, L.stream_ptr(x.device))
     return rc, out
 
 
-def _call_workspace(L, x, U, V, S, b, r, algo):
+def _call_workspace(L, x, U, V, S, b, r, algo, layouts=None):
     M, in_f = x.shape
-    out_f = b * U.shape[2]
+    ul, sl = layouts or (L.U_RQ, L.S_JIR)
+    out_f = b * (U.shape[2] if ul == L.U_RQ else U.shape[1])
     dt = L.dtype_code(x.dtype)
     out = torch.full((M, out_f), float("nan"), device=x.device, dtype=x.dtype)
     ws = torch.zeros(max(L.lib().blr_blast_workspace_bytes(M, in_f, out_f, b, r, dt, algo), 1 << 20), dtype=torch.uint8, device=x.device)
     rc = L.lib().blr_blast_fwd(x.data_ptr(), x.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(), out.data_ptr(), out.stride(0), None, None,
-                               M, in_f, out_f, b, r, dt, L.U_RQ, L.S_JIR, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
+                               M, in_f, out_f, b, r, dt, ul, sl, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
     torch.cuda.synchronize()
     return rc, out
 
@@ -64,6 +66,25 @@ def test_two_calls_in_a_row_the_second_smaller(dtype):
         assert_close(got, want.to(torch.float64).cpu().numpy(), dtype, f"static call {n} against blr_blast_fwd")
         if algo == L.ALGO_TILED:
             assert torch.equal(got, want), f"call {n}: same kernels, different bits"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_bmm_layouts_at_one_to_four_rows(dtype):
+    """U as (b, q, r) and S as (r, i, j) at 4, 2 and 1 rows: the first launch also leaves S, reordered, in the scratch behind
+    its own result; each call is smaller than the one before."""
+    from triton_funcs import _lib as L
+    for n, (b, p, q, r, M) in enumerate([(16, 64, 72, 256, 4), (8, 32, 100, 128, 2), (4, 32, 40, 128, 1)]):
+        say(f"[case] blast_fwd_static bmm layouts call {n}: b={b} p={p} q={q} r={r} M={M} {dtype}")
+        x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=90 + n)
+        ref = O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0].reshape(M, b * q)
+        Uk, Vk, Sk = (dev(a, dtype) for a in O.blast_to_bmm_layout(U, Vt, S))
+        rc, got = _call_static(L, dev(x, dtype), Uk, Vk, Sk, b, r, (L.U_QR, L.S_RIJ))
+        assert rc == 0, L.lib().blr_last_error().decode()
+        torch.cuda.synchronize()
+        rc2, want = _call_workspace(L, dev(x, dtype), Uk, Vk, Sk, b, r, L.ALGO_AUTO, (L.U_QR, L.S_RIJ))
+        assert rc2 == 0, L.lib().blr_last_error().decode()
+        assert_close(got, ref, dtype, f"static bmm call {n} against the oracle")
+        assert_close(got, want.to(torch.float64).cpu().numpy(), dtype, f"static bmm call {n} against blr_blast_fwd")
 
 
 def test_oversize_call_is_refused_without_a_launch():
