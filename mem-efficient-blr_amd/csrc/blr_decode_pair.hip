@@ -528,6 +528,9 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   if (!qr && a.u_layout != BLR_U_RQ) return 1;
   if (b > 16 * DP_JJ || b >= 65536 || bo >= 65536 || R % 8 || R > 4096) return 1;
   if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return 1;
+  // 32-bit offsets into every operand, and DP_OOB has to lie beyond each of them
+  if ((int64_t)a.in_f * R * 2 >= (int64_t)DP_OOB || (int64_t)a.out_f * R * 2 >= (int64_t)DP_OOB || (int64_t)b * bo * R * 2 >= (int64_t)DP_OOB ||
+      ((int64_t)(M - 1) * a.ldx + a.in_f) * 2 >= (int64_t)DP_OOB) return 1;
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int WBITS = a.wbits, EPL = 128 / WBITS;
 
