@@ -1312,7 +1312,14 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     if (rc != 1) return rc;
   }
   if (a.rows_only) { set_error("blast_q: code rows that are not whole 16-byte pieces need in_f / b, r and out_f / b to be multiples of 8 and at most 4096"); return BLR_ERR_UNSUPPORTED; }
-  {
+  if (a.perm_per > 0) {
+    // Monarch (few, wide blocks): the single-launch kernel where its stage 1 fits one batch of loads per item (11.3 against
+    // about 12 us at 4096 -> 4096), the two launches for deeper input blocks (11008 -> 4096: input blocks of 2752 rows)
+    int rc = decode3_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
+    if (rc != 1) return rc;
+    rc = decode_pair_launch(a, region, decode2_region_bytes(), st);
+    if (rc != 1) return rc;
+  } else {
     int rc = decode_pair_launch(a, region, decode2_region_bytes(), st);
     if (rc != 1) return rc;
     rc = decode3_blast_launch(a, region, epoch_word, arrive_word, err_word, st);

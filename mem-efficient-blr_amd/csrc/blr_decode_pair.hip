@@ -57,6 +57,7 @@ struct PairParams {
   FastDiv nch2;
   int xcd_order;
   const void* bias; int act, ep;                 // fused output stage: bias of T (indexed like a row of out) or null, blr_act
+  int perm_per;                                  // Monarch: z_i[r] = y[r / per][i per + r % per] (no S); 0 otherwise
   const void* s_rij; int s_chunks;               // S given as (r, i, j): stage 1 rewrites it as (j, i, r) into S, eight ranks per workgroup
 };
 
@@ -259,17 +260,21 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   const int ib = p.bo > 1 ? (int)i2 : 0;               // (a single output block: every slab uses S of block 0, or none)
   u32x4 yq[MT][KSM][DP_JJ];
   u32x4 sq[DP_JJ];
+  // Monarch: the "mix" is a gather - the eight ranks of this thread come from one input block (the period is a multiple
+  // of eight), so group 0 fetches that one piece of y and the other groups contribute nothing
+  const int pj = p.perm_per > 0 ? (oct * 8) / p.perm_per : 0;
+  const int pr = p.perm_per > 0 ? (int)i2 * p.perm_per + (oct * 8 - pj * p.perm_per) : oct * 8;
 #pragma unroll
   for (int jj = 0; jj < DP_JJ; ++jj) {
-    const int j = jg * p.jpg + jj;
-    const bool on = mix_on && jj < p.jpg && j < p.b;
+    const int j = p.perm_per > 0 ? pj : jg * p.jpg + jj;
+    const bool on = p.perm_per > 0 ? (mix_on && jj == 0 && jg == 0) : (mix_on && jj < p.jpg && j < p.b);
     sq[jj] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(sbuf, (on && p.S) ? (uint32_t)(ib * (int)p.s_si + j * (int)p.s_sj + oct * 8) * 2u : DP_OOB, 0, 0));
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int ks = 0; ks < KSM; ++ks)
         if (ks < p.ks1 && m < M)
-          yq[m][ks][jj] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ybuf, on ? (uint32_t)(((ks * p.b + j) * M + m) * R + oct * 8) * 2u : DP_OOB, 0, 0));
+          yq[m][ks][jj] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ybuf, on ? (uint32_t)(((ks * p.b + j) * M + m) * R + pr) * 2u : DP_OOB, 0, 0));
   }
   // ---- the whole slab of U right behind, in straight-line code: the compiler counts exactly these PF loads ----
   const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)((int64_t)p.bo * R * p.Q * WB / 8));
@@ -517,27 +522,29 @@ bool pair_fns(int MT, int wbits, int pfg, bool qr, bool st, void** f1, void** f2
 int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_bytes, hipStream_t st) {
   static const int enabled = env_i("BLR_DECODE_PAIR", 1);
   if (!enabled) return 1;
+  static const int dbg0 = env_i("BLR_D2_DEBUG", 0);
+  auto decline = [&](int line) { if (dbg0) fprintf(stderr, "decode pair: not for this call (line %d)\n", line); return 1; };
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
-  if (M < 1 || M > 4) return 1;
-  if (a.wbits == 8 && M > 2) return 1;              // codes at more rows: the matrix-core kernel
-  if (a.wbits == 4 && M > 1) return 1;
-  if (a.perm_per > 0) return 1;                     // Monarch: the single-launch kernels
+  if (M < 1 || M > 4) return decline(__LINE__);
+  if (a.wbits == 8 && M > 2) return decline(__LINE__);              // codes at more rows: the matrix-core kernel
+  if (a.wbits == 4 && M > 1) return decline(__LINE__);
+  if (a.perm_per > 0 && (a.S || a.perm_per % 8 || bo != b || a.perm_per * b != R)) return decline(__LINE__);   // Monarch: whole 16-byte pieces of one input block
   const bool qr = a.u_layout == BLR_U_QR;           // U (b, q, r): two-byte weights with a power-of-two rank of at least 128
-  if (qr && (a.wbits != 16 || R < 128 || (R & (R - 1)))) return 1;
-  if (!qr && a.u_layout != BLR_U_RQ) return 1;
-  if (b > 16 * DP_JJ || b >= 65536 || bo >= 65536 || R % 8 || R > 4096) return 1;
-  if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return 1;
+  if (qr && (a.wbits != 16 || R < 128 || (R & (R - 1)))) return decline(__LINE__);
+  if (!qr && a.u_layout != BLR_U_RQ) return decline(__LINE__);
+  if (b > 16 * DP_JJ || b >= 65536 || bo >= 65536 || R % 8 || R > 4096) return decline(__LINE__);
+  if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return decline(__LINE__);
   // 32-bit offsets into every operand, and DP_OOB has to lie beyond each of them
   if ((int64_t)a.in_f * R * 2 >= (int64_t)DP_OOB || (int64_t)a.out_f * R * 2 >= (int64_t)DP_OOB || (int64_t)b * bo * R * 2 >= (int64_t)DP_OOB ||
-      ((int64_t)(M - 1) * a.ldx + a.in_f) * 2 >= (int64_t)DP_OOB) return 1;
+      ((int64_t)(M - 1) * a.ldx + a.in_f) * 2 >= (int64_t)DP_OOB) return decline(__LINE__);
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int WBITS = a.wbits, EPL = 128 / WBITS;
 
   PairParams p = {};
   p.x = a.x; p.ldx = a.ldx; p.V = a.V; p.U = a.U; p.S = a.S; p.out = a.out; p.ldo = a.ldo;
   p.u_scales = (const f16*)a.u_scales; p.v_scales = (const f16*)a.v_scales;
-  p.M = M; p.b = b; p.bo = bo; p.P = P; p.R = R; p.Q = Q;
+  p.M = M; p.b = b; p.bo = bo; p.P = P; p.R = R; p.Q = Q; p.perm_per = a.perm_per;
   p.o_bs = a.out_ns ? a.out_bs : Q; p.o_ns = a.out_ns ? a.out_ns : 1;
   if (a.s_layout == BLR_S_JIR) { p.s_sj = (int64_t)b * R; p.s_si = R; p.s_sr = 1; }
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
@@ -546,10 +553,10 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   // that order too; they stay on the single-launch kernel, which measured 0.3 - 0.5 us faster on them.)
   const bool s_turn = a.S && a.s_layout == BLR_S_RIJ && a.wbits == 16;
   if (s_turn) {
-    if (b * bo > DP_NT) return 1;
+    if (b * bo > DP_NT) return decline(__LINE__);
     p.s_sj = (int64_t)bo * R; p.s_si = R; p.s_sr = 1;
   }
-  if (a.S && !s_turn && (p.s_sr != 1 || !aligned(a.S, 16))) return 1;     // S in 16-byte pieces along the rank
+  if (a.S && !s_turn && (p.s_sr != 1 || !aligned(a.S, 16))) return decline(__LINE__);     // S in 16-byte pieces along the rank
   p.x_vec = aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0;
 
   // ---- stage 1: 128-rank chunks, k split so that an item is at most eight loads per lane; any number of workgroups ----
@@ -589,7 +596,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   if (s_turn) {
     p.s_rij = a.S; p.s_chunks = R / 8;
     p.S = reinterpret_cast<char*>(region) + ybytes;
-    if (b * (int)p.nch1.d * p.ks1 < p.s_chunks) return 1;       // one chunk of S per workgroup of launch 1
+    if (b * (int)p.nch1.d * p.ks1 < p.s_chunks) return decline(__LINE__);       // one chunk of S per workgroup of launch 1
   }
 
   // ---- mix + stage 2: a slab spans the whole rank; the narrowest column chunk that keeps it within the registers ----
@@ -642,7 +649,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     // runs stage 1 under that stream: 16.3 against 17.5 us at 4096 -> 22016, rank 1024; below that the two launches win
     // (9.5 against 10.6 us at 4096 -> 4096, rank 512).  BLR_DECODE_PAIR=2 takes every call this path can serve.
     const double slab_bytes = (double)p.pfn * (DP_NT >> p.lpr2_log2) * (1 << p.lpr2_log2) * 16.0;
-    if (enabled != 2 && !qr && slab_bytes > 192.0 * 1024.0 && a.S && a.perm_per == 0 && bo > 1) return 1;
+    if (enabled != 2 && !qr && slab_bytes > 192.0 * 1024.0 && a.S && a.perm_per == 0 && bo > 1) return decline(__LINE__);
   }
   const int pfg = (p.pfn + 7) / 8;
   void *f1 = nullptr, *f2 = nullptr;

@@ -106,6 +106,24 @@ def test_monarch_llama7b(layer, M):
         assert_close(out[:, rows], ref, torch.float16, f"monarch {layer} {name} M{M}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 1104, 256, 40), (2, 2752, 128, 72)], ids=lambda s: "b%d-p%d-r%d-s%d" % s)
+def test_monarch_single_row_deep_input_blocks(shape, dtype):
+    """One token row with input blocks deeper than the single-launch kernel takes in one batch of loads: the two-launch
+    kernels, whose second launch gathers its z through the permutation.  Plain and with a fused bias."""
+    from triton_funcs import _lib as L
+    b, p, rank, s = shape
+    x, w1_t, w2_t = monarch_inputs(b, p, rank, s, (1,), seed=9)
+    ref = _ref_monarch(x, w1_t, w2_t, dtype)[0]
+    say(f"[case] monarch single row b={b} p={p} rank={rank} s={s} {dtype}")
+    out = _run_monarch("triton_monarch_right_left_fp16", x, w1_t, w2_t, dtype)
+    assert_close(out, ref, dtype, "monarch M=1, deep blocks", scale=2.0)
+    bias = np.random.default_rng(9).standard_normal(b * s)
+    with L.fused_epilogue(dev(bias, dtype), None):
+        out = _run_monarch("triton_monarch_right_left_fp16", x, w1_t, w2_t, dtype)
+    assert_close(out, ref + rounded(bias, dtype), dtype, "monarch M=1, deep blocks + bias", scale=2.0)
+
+
 def test_monarch_index_map_bit_exact_on_gpu():
     """Integer-valued inputs make every product exact in fp16/fp32: the permutation must then be bit-exact."""
     b, p, rank, s = 4, 4, 8, 4
