@@ -107,21 +107,23 @@ def test_monarch_llama7b(layer, M):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 5, 16])
 @pytest.mark.parametrize("shape", [(4, 1104, 256, 40), (2, 2752, 128, 72)], ids=lambda s: "b%d-p%d-r%d-s%d" % s)
-def test_monarch_single_row_deep_input_blocks(shape, dtype):
-    """One token row with input blocks deeper than the single-launch kernel takes in one batch of loads: the two-launch
-    kernels, whose second launch gathers its z through the permutation.  Plain and with a fused bias."""
+def test_monarch_few_rows_deep_input_blocks(shape, M, dtype):
+    """Input blocks deeper than the few-row kernels take in one piece.  One row: the two-launch kernels, whose second launch
+    gathers its z through the permutation.  2..16 rows: the blocks are cut into equal slices and a small kernel adds the
+    slices while it permutes.  Plain and with a fused bias."""
     from triton_funcs import _lib as L
     b, p, rank, s = shape
-    x, w1_t, w2_t = monarch_inputs(b, p, rank, s, (1,), seed=9)
+    x, w1_t, w2_t = monarch_inputs(b, p, rank, s, (M,), seed=9)
     ref = _ref_monarch(x, w1_t, w2_t, dtype)[0]
-    say(f"[case] monarch single row b={b} p={p} rank={rank} s={s} {dtype}")
+    say(f"[case] monarch M={M} b={b} p={p} rank={rank} s={s} {dtype}")
     out = _run_monarch("triton_monarch_right_left_fp16", x, w1_t, w2_t, dtype)
-    assert_close(out, ref, dtype, "monarch M=1, deep blocks", scale=2.0)
+    assert_close(out, ref, dtype, "monarch, deep blocks", scale=2.0)
     bias = np.random.default_rng(9).standard_normal(b * s)
     with L.fused_epilogue(dev(bias, dtype), None):
         out = _run_monarch("triton_monarch_right_left_fp16", x, w1_t, w2_t, dtype)
-    assert_close(out, ref + rounded(bias, dtype), dtype, "monarch M=1, deep blocks + bias", scale=2.0)
+    assert_close(out, ref + rounded(bias, dtype), dtype, "monarch, deep blocks + bias", scale=2.0)
 
 
 def test_monarch_index_map_bit_exact_on_gpu():
