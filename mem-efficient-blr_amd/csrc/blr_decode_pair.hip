@@ -12,6 +12,8 @@
 //     has fetched them), then for its slab of U, computes  z_i = sum_j S_ij * y_j  redundantly with the other slabs of
 //     block i while U streams, multiplies and stores.  No partial outputs, no tags, no epoch, no spinning, no
 //     residency requirement.
+// Where stage 1 has long items and U is small (deep input blocks: 11008 -> 4096), launch 1 carries extra workgroups that only
+// load the slabs of U, each on the XCD whose L2 its slab's workgroup of launch 2 will read from (see the launcher).
 // The number of slab loads is a template parameter: the compiler then knows how many loads follow the mix operands
 // and waits for exactly those (loads under runtime branches make it wait for everything in flight).
 // The layouts of the bmm names are served at one row as well (measured 12.0 -> 9.6, 20.2 -> 16.6 and 17.1 -> 14.0 us on the
@@ -57,6 +59,9 @@ struct PairParams {
   FastDiv nch2;
   int xcd_order;
   const void* bias; int act, ep;                 // fused output stage: bias of T (indexed like a row of out) or null, blr_act
+  int pre_split;                                 // workgroups that share the fetch of one slab (each takes pre_loads / pre_split loads)
+  int items1, grid2, pre_loads, qr;              // launch 1: workgroups of stage 1; behind them, one per slab of launch 2 that fetches the
+                                                 // slab's first pre_loads loads into the L2 of the XCD its slab workgroup will run on
   int perm_per;                                  // Monarch: z_i[r] = y[r / per][i per + r % per] (no S); 0 otherwise
   const void* s_rij; int s_chunks;               // S given as (r, i, j): stage 1 rewrites it as (j, i, r) into S, eight ranks per workgroup
 };
@@ -97,6 +102,31 @@ __device__ __forceinline__ void pair_reduce(float (&acc)[MT][EPL], int lpr_log2,
   }
 }
 
+// Where a slab workgroup's loads of U start: byte offset of this lane's first load, the uniform step between loads, and what
+// decides whether load u exists (rows of U along the rank: the row of the load lies inside the block; otherwise u < pfn).
+struct SlabLoads { uint32_t uoff, ustep; int qrow0, rppq; };
+template <int WB>
+__device__ __forceinline__ SlabLoads slab_loads(const PairParams& p, uint32_t w, int tid, bool qr) {
+  constexpr int EPL = 128 / WB;
+  const uint32_t i2 = fd_div(w, p.nch2), nc2 = w - i2 * p.nch2.d;
+  SlabLoads s;
+  if (qr) {
+    const int oct = tid & ((1 << p.octs_log2) - 1), jg = tid >> p.octs_log2;
+    s.rppq = DP_NT >> p.octs_log2;
+    s.qrow0 = (int)nc2 * p.pfn * s.rppq + jg;              // (pfn is the slab kernel's whole load count in this layout)
+    s.uoff = (uint32_t)(((int)i2 * p.Q + s.qrow0) * p.R + oct * 8) * 2u;
+    s.ustep = (uint32_t)DP_NT * 16u;
+  } else {
+    const int lpr2 = 1 << p.lpr2_log2, rpp2 = DP_NT >> p.lpr2_log2;
+    const int cv2 = tid & (lpr2 - 1), rs2 = tid >> p.lpr2_log2;
+    const int n2 = (int)nc2 * lpr2 * EPL + cv2 * EPL;
+    s.rppq = 0; s.qrow0 = 0;
+    s.uoff = (uint32_t)((((int)i2 * p.R + rs2) * p.Q + (n2 < p.Q ? n2 : 0))) * (uint32_t)WB / 8u;
+    s.ustep = (uint32_t)rpp2 * (uint32_t)p.Q * (uint32_t)WB / 8u;
+  }
+  return s;
+}
+
 // ---- launch 1: y[ks][j][m][n] = sum_k x[m, j P + k] V_j[k, n] over one k-slice -------------------------------------------
 template <typename T, int MT, int WB, bool ST>
 __global__ __launch_bounds__(DP_NT) void pair_stage1_kernel(PairParams p) {
@@ -106,6 +136,31 @@ __global__ __launch_bounds__(DP_NT) void pair_stage1_kernel(PairParams p) {
   __shared__ __attribute__((aligned(16))) float red[MT * DP_NT * EPL];
   const int tid = threadIdx.x;
   TR4(0);
+  if (blockIdx.x >= (uint32_t)p.items1) {
+    // Not a stage-1 item: this workgroup pulls the head of one slab of U into L2 while stage 1 leaves most of the memory system
+    // idle.  It picks the slab whose workgroup of launch 2 will run on the same XCD (workgroup w runs on XCD w % 8, and the L2 is
+    // per XCD): blocks of eight consecutive slab indices are permuted so that index and own index agree modulo 8.
+    const uint32_t g8 = ((uint32_t)p.grid2 + 7u) & ~7u;
+    const uint32_t q = blockIdx.x, tq = q - (uint32_t)p.items1;
+    const uint32_t part = tq / g8, t = tq - part * g8;
+    const uint32_t b2 = (t & ~7u) + (q & 7u);
+    if (b2 >= (uint32_t)p.grid2) return;
+    const int per_part = p.pre_loads / p.pre_split, u_lo = (int)part * per_part, u_hi = u_lo + per_part;
+    const uint32_t w2 = p.xcd_order ? xcd_item(b2, (uint32_t)p.grid2) : b2;
+    const SlabLoads sl = slab_loads<WB>(p, w2, tid, p.qr != 0);
+    const __amdgpu_buffer_rsrc_t ub = rbuf2(p.U, (uint32_t)((int64_t)p.bo * p.R * p.Q * WB / 8));   // plain cached loads: the lines should stay
+    for (int u0 = u_lo; u0 < u_hi; u0 += 8) {
+      u32x4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const bool on = u0 + u < u_hi && (p.qr ? sl.qrow0 + (u0 + u) * sl.rppq < p.Q : u0 + u < p.pfn);
+        v[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ub, on ? sl.uoff : DP_OOB, (uint32_t)(u0 + u) * sl.ustep, 0));
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) asm volatile("" ::"v"(v[u]));
+    }
+    return;
+  }
   const int M = p.M;
   const int lpr1 = 1 << p.lpr1_log2, rpp1 = DP_NT >> p.lpr1_log2;
   const int cv1 = tid & (lpr1 - 1), rs1 = tid >> p.lpr1_log2;
@@ -278,10 +333,9 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   }
   // ---- the whole slab of U right behind, in straight-line code: the compiler counts exactly these PF loads ----
   const __amdgpu_buffer_rsrc_t ubuf = wbuf(p.U, (uint32_t)((int64_t)p.bo * R * p.Q * WB / 8));
-  const uint32_t uoff = QR ? (uint32_t)(((int)i2 * p.Q + q0 + jg) * R + oct * 8) * 2u
-                            : (uint32_t)((((int)i2 * R + rs2) * p.Q + (n2 < p.Q ? n2 : 0))) * (uint32_t)WB / 8u;
-  const uint32_t ustep = QR ? (uint32_t)DP_NT * 16u : (uint32_t)rpp2 * (uint32_t)p.Q * (uint32_t)WB / 8u;
-  auto u_on = [&](int u) { return QR ? q0 + u * rppq + jg < p.Q : u < p.pfn; };   // QR: rows past the block are not read
+  const SlabLoads sl = slab_loads<WB>(p, w, tid, QR);
+  const uint32_t uoff = sl.uoff, ustep = sl.ustep;
+  auto u_on = [&](int u) { return QR ? sl.qrow0 + u * sl.rppq < p.Q : u < p.pfn; };   // QR: rows past the block are not read
   // A wave that asks for more than the memory path of its compute unit takes at once is held at the load until there
   // is room, so only the first eight loads go out before the mix; the rest follow group by group, each behind the
   // products of the group before (whose data has landed by then: loads come back in order).
@@ -656,11 +710,35 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   const bool have = a.dtype == BLR_F16 ? pair_fns<f16>(MT, WBITS, pfg, qr, s_turn, &f1, &f2) : pair_fns<bf16>(MT, WBITS, pfg, qr, s_turn, &f1, &f2);
   if (!have) return d2_bail(__LINE__);
   const int grid1 = b * (int)p.nch1.d * p.ks1, grid2 = bo * (int)p.nch2.d;
+  // Launch 1 also warms the L2 with U where its own items are long enough to hide that and all of U fits: extra workgroups,
+  // each on the XCD where its slab's workgroup of launch 2 will run, load whole slabs and drop the data.  A slab's loads are
+  // 8 KiB per workgroup each and a compute unit draws about 35 GB/s: a fetch that outlasts stage 1 only delays launch 2, one
+  // that shares compute units with a short stage 1 slows it down, and a fetch of part of a long stream of U gains nothing.
+  // Measured, without / with: 11008 -> 4096 (88 KiB items, 8 MB of U) 15.0 -> 13.9 us, low rank on that shape 15.1 -> 14.0,
+  // Monarch 15.8 -> 15.2, low rank 4096 -> 4096 (64 KiB items, four workgroups per slab) 12.4 -> 11.7 (one per slab: 12.8);
+  // 4096 -> 4096 (32 KiB items) 9.2 -> 9.4 - 9.6; 4096 -> 22016 (45 MB of U) 16.6 -> 17.1 - 18.3.  Hence: items of at least
+  // 60 KB, whole slabs of at most 16 loads, at most 12 MB of U and no more slabs than compute units; as many workgroups per
+  // slab (1, 2 or 4) as keep one's share within three quarters of an item.  BLR_DP_PRE / BLR_DP_PRE_SPLIT override (0: none).
+  static const int e_pre = env_i("BLR_DP_PRE", -1), e_split = env_i("BLR_DP_PRE_SPLIT", 0);
+  p.items1 = grid1; p.grid2 = grid2; p.qr = qr ? 1 : 0;
+  {
+    const double item_bytes = (double)p.kc1 * (1 << p.lpr1_log2) * 16.0;
+    const double u_bytes = (double)bo * R * Q * WBITS / 8.0;
+    const int cus = device_cus() > 0 ? device_cus() : 256;
+    const int pfn8 = (int)cdiv(p.pfn, 8) * 8;
+    int pre = (item_bytes >= 60e3 && pfn8 <= 16 && u_bytes <= 12e6 && grid2 <= cus) ? pfn8 : 0;
+    if (e_pre >= 0) { pre = (int)cdiv(e_pre, 8) * 8; if (pre > pfn8) pre = pfn8; }
+    int split = 1;
+    while (split < 4 && pre * 8192.0 / split > 0.75 * item_bytes && pre % (2 * split) == 0) split *= 2;
+    if ((e_split == 1 || e_split == 2 || e_split == 4) && pre % e_split == 0) split = e_split;
+    p.pre_loads = pre; p.pre_split = split;
+  }
+  const int grid1_all = grid1 + (p.pre_loads > 0 ? (int)cdiv(grid2, 8) * 8 * p.pre_split : 0);
   static const int dbg = env_i("BLR_D2_DEBUG", 0);
   if (dbg) fprintf(stderr, "decode pair: M=%d b=%d bo=%d P=%d R=%d Q=%d wb=%d | stage 1: %d items (ks %d, kc %d) | slabs %d (lpr %d, pfn %d, octs %d, jpg %d)\n",
                    M, b, bo, P, R, Q, WBITS, grid1, p.ks1, p.kc1, grid2, 1 << p.lpr2_log2, p.pfn, 1 << p.octs_log2, p.jpg);
   void* args[] = {&p};
-  hipError_t e = hipLaunchKernel(f1, dim3(grid1), dim3(DP_NT), args, 0, st);
+  hipError_t e = hipLaunchKernel(f1, dim3(grid1_all), dim3(DP_NT), args, 0, st);
   if (e == hipSuccess) e = hipLaunchKernel(f2, dim3(grid2), dim3(DP_NT), args, 0, st);
   if (e != hipSuccess) { set_error("decode pair: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   if (p.ep) epilogue_taken();
