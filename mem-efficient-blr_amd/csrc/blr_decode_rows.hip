@@ -288,12 +288,56 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   TR5(4);
 }
 
+// ---- warming the L2 for the second product ---------------------------------------------------------------------------------
+// A launch between the two products that only adds slices (low rank, sliced Monarch) leaves the memory system idle.  Extra
+// workgroups of that launch load the chunks of the second product's factor and drop the data: chunk of workgroup w2 of the next
+// launch by a workgroup that runs on the same XCD (workgroup w of a launch runs on XCD w % 8 and each XCD has its own L2), up
+// to a budget per workgroup that keeps an XCD's share within its L2.
+struct RowsPrefetch {
+  const char* W; int64_t w_bs_bytes;      // factor; bytes per batch entry
+  uint32_t chunk_step, row_stride;        // bytes from chunk to chunk and from row to row of a chunk
+  uint32_t piece16, last_piece16;         // 16-byte pieces per row of a chunk (of the last chunk of an entry)
+  uint32_t nrows;                         // rows of a chunk
+  uint32_t budget16;                      // at most this many pieces per workgroup
+  FastDiv nch; uint32_t xcd_span;         // as in RowsParams of the launch that will read the chunks
+  uint32_t nblocks2;                      // workgroups of that launch (0: nothing to fetch)
+};
+
+__device__ __forceinline__ void rows_prefetch(const RowsPrefetch& f, uint32_t first_block) {
+  const uint32_t q = blockIdx.x, t = q - first_block;
+  const uint32_t b2 = (t & ~7u) + (q & 7u);              // same XCD as workgroup b2 of the next launch
+  if (b2 >= f.nblocks2) return;
+  const uint32_t item = f.xcd_span ? (b2 & 7u) * f.xcd_span + (b2 >> 3) : b2;
+  const uint32_t bt = fd_div(item, f.nch), ch = item - bt * f.nch.d;
+  const uint32_t p16 = ch + 1 == f.nch.d ? f.last_piece16 : f.piece16;
+  const char* base = f.W + (int64_t)bt * f.w_bs_bytes + (int64_t)ch * f.chunk_step;
+  uint32_t units = f.nrows * p16;
+  if (units > f.budget16) units = f.budget16;
+  const uint32_t nt = blockDim.x;
+  for (uint32_t u0 = threadIdx.x; u0 < units; u0 += 8 * nt) {
+    u32x4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const uint32_t u = u0 + (uint32_t)k * nt;
+      if (u < units) {
+        const uint32_t row = u / p16, pc = u - row * p16;
+        v[k] = *reinterpret_cast<const u32x4*>(base + (int64_t)row * f.row_stride + (int64_t)pc * 16);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (u0 + (uint32_t)k * nt < units) asm volatile("" ::"v"(v[k]));
+  }
+}
+
 // ---- the mix between the two products: z[i][m][r] = sum_j S(i, j, r) y[j][m][r], rank contiguous in S ------------------------
 // One thread per four ranks of one (i, m): 2 b eight-byte loads, all in flight at once, neighbouring threads on neighbouring
 // ranks.  Y is re-read b times and S M times - from L2, both are a few hundred KiB.  fp32 sums in input-block order.
 template <typename T, int B>
 __global__ __launch_bounds__(256) void rows_mix_kernel(const T* __restrict__ Y, const T* __restrict__ S, T* __restrict__ Z,
-                                                        int M, int b, int R, int64_t s_si, int64_t s_sj, FastDiv r4div, FastDiv bdiv, uint32_t total) {
+                                                        int M, int b, int R, int64_t s_si, int64_t s_sj, FastDiv r4div, FastDiv bdiv, uint32_t total,
+                                                        RowsPrefetch pf, uint32_t nmix) {
+  if (blockIdx.x >= nmix) { rows_prefetch(pf, nmix); return; }
   const uint32_t item = blockIdx.x * 256u + threadIdx.x;
   if (item >= total) return;
   const uint32_t t = fd_div(item, r4div), r4 = item - t * r4div.d;
@@ -326,7 +370,8 @@ __global__ __launch_bounds__(256) void rows_mix_kernel(const T* __restrict__ Y, 
 
 // Low rank seen as BLAST with one output block and S = 1: z[m][r] = sum_j y[j][m][r] (the k-slices of x A), fp32 sums in slice order.
 template <typename T>
-__global__ __launch_bounds__(256) void rows_sum_kernel(const T* __restrict__ Y, T* __restrict__ Z, int b, int64_t MR4) {
+__global__ __launch_bounds__(256) void rows_sum_kernel(const T* __restrict__ Y, T* __restrict__ Z, int b, int64_t MR4, RowsPrefetch pf, uint32_t nmix) {
+  if (blockIdx.x >= nmix) { rows_prefetch(pf, nmix); return; }
   const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (item >= MR4) return;
   using V4 = typename TypeTraits<T>::vec4;
@@ -350,7 +395,9 @@ __global__ __launch_bounds__(256) void rows_sum_kernel(const T* __restrict__ Y, 
 // Monarch with its input blocks cut into ks slices (so that the first product spreads over the chip): the slices are added and
 // the permutation applied in one pass, z[l][m][r] = sum_s y[(r / per) ks + s][m][l per + r % per]; thread = four ranks.
 template <typename T>
-__global__ __launch_bounds__(256) void rows_perm_sum_kernel(const T* __restrict__ Y, T* __restrict__ Z, int ks, int M, int R, int per, int64_t items) {
+__global__ __launch_bounds__(256) void rows_perm_sum_kernel(const T* __restrict__ Y, T* __restrict__ Z, int ks, int M, int R, int per, int64_t items,
+                                                            RowsPrefetch pf, uint32_t nmix) {
+  if (blockIdx.x >= nmix) { rows_prefetch(pf, nmix); return; }
   const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (item >= items) return;
   using V4 = typename TypeTraits<T>::vec4;
@@ -375,8 +422,9 @@ __global__ __launch_bounds__(256) void rows_perm_sum_kernel(const T* __restrict_
 // entry points).  Neighbouring threads take neighbouring output blocks i, so that a wave reads whole (r, :, :) slices of S.
 template <typename T>
 __global__ __launch_bounds__(256) void rows_mix_rij_kernel(const T* __restrict__ Y, const T* __restrict__ S, T* __restrict__ Z,
-                                                            int M, int R, FastDiv r4div, uint32_t total) {
+                                                            int M, int R, FastDiv r4div, uint32_t total, RowsPrefetch pf, uint32_t nmix) {
   constexpr int B = 16;
+  if (blockIdx.x >= nmix) { rows_prefetch(pf, nmix); return; }
   const uint32_t item = blockIdx.x * 256u + threadIdx.x;
   if (item >= total) return;
   const uint32_t i = item & (B - 1), t = item >> 4;
@@ -407,22 +455,26 @@ __global__ __launch_bounds__(256) void rows_mix_rij_kernel(const T* __restrict__
 
 namespace {
 
+inline unsigned prefetch_blocks(const RowsPrefetch& pf) { return pf.nblocks2 ? (pf.nblocks2 + 7u) & ~7u : 0u; }
+
 template <typename T>
-int rows_mix_rij_t(const void* Y, const void* S, void* Z, int M, int R, hipStream_t st) {
+int rows_mix_rij_t(const void* Y, const void* S, void* Z, int M, int R, const RowsPrefetch& pf, hipStream_t st) {
   const uint32_t total = (uint32_t)((int64_t)M * 16 * (R / 4));
-  hipLaunchKernelGGL((rows_mix_rij_kernel<T>), dim3((unsigned)cdiv(total, 256)), dim3(256), 0, st, (const T*)Y, (const T*)S, (T*)Z, M, R,
-                     fd_make((uint32_t)(R / 4)), total);
+  const uint32_t nmix = (uint32_t)cdiv(total, 256);
+  hipLaunchKernelGGL((rows_mix_rij_kernel<T>), dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const T*)Y, (const T*)S, (T*)Z, M, R,
+                     fd_make((uint32_t)(R / 4)), total, pf, nmix);
   BLR_CHECK_LAUNCH("rows_mix_rij");
   return BLR_OK;
 }
 
 template <typename T>
-int rows_mix_t(const void* Y, const void* S, void* Z, int M, int b, int R, int64_t s_si, int64_t s_sj, hipStream_t st) {
+int rows_mix_t(const void* Y, const void* S, void* Z, int M, int b, int R, int64_t s_si, int64_t s_sj, const RowsPrefetch& pf, hipStream_t st) {
   const uint32_t total = (uint32_t)((int64_t)M * b * (R / 4));
-  const dim3 grid((unsigned)cdiv(total, 256)), block(256);
+  const uint32_t nmix = (uint32_t)cdiv(total, 256);
+  const dim3 grid(nmix + prefetch_blocks(pf)), block(256);
   const FastDiv r4div = fd_make((uint32_t)(R / 4)), bdiv = fd_make((uint32_t)b);
-  if (b == 16) hipLaunchKernelGGL((rows_mix_kernel<T, 16>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total);
-  else hipLaunchKernelGGL((rows_mix_kernel<T, 0>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total);
+  if (b == 16) hipLaunchKernelGGL((rows_mix_kernel<T, 16>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total, pf, nmix);
+  else hipLaunchKernelGGL((rows_mix_kernel<T, 0>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total, pf, nmix);
   BLR_CHECK_LAUNCH("rows_mix");
   return BLR_OK;
 }
@@ -458,8 +510,8 @@ int rows_launch_t(RowsParams& p, int batch, hipStream_t st) {
   return BLR_OK;
 }
 
-// One batch of skinny products; returns 1 when the operands do not fit the kernel.
-int rows_product(RowsParams p, int batch, int dtype, int wbits, bool nk, hipStream_t st) {
+// Plans one batch of skinny products (chunk width, rounds, item order); returns 1 when the operands do not fit the kernel.
+int rows_plan(RowsParams& p, int batch, int dtype, int wbits, bool nk) {
   if (nk && wbits != 16) return 1;
   if (p.K % 8 || p.N % 8 || p.N > 65536 || p.K > 4 * DR_WAVES * DR_MAX_STEPS * 32) return 1;
   if (!aligned(p.A, 16) || !aligned(p.W, 16) || p.lda % 8 || p.a_bs % 8 || p.w_bs % 32) return 1;
@@ -485,10 +537,48 @@ int rows_product(RowsParams p, int batch, int dtype, int wbits, bool nk, hipStre
   if ((int64_t)batch * p.nch.d >= 65536) return 1;
   static const int e_xcd = env_i("BLR_DR_XCD", 1);
   p.xcd_span = (e_xcd && (batch * p.nch.d) % 8 == 0) ? (uint32_t)(batch * p.nch.d / 8) : 0u;
+  return BLR_OK;
+}
+
+int rows_launch(RowsParams p, int batch, int dtype, int wbits, bool nk, hipStream_t st) {
   if (nk) return dtype == BLR_F16 ? rows_launch_t<f16, 16, true>(p, batch, st) : rows_launch_t<bf16, 16, true>(p, batch, st);
   if (wbits == 16) return dtype == BLR_F16 ? rows_launch_t<f16, 16>(p, batch, st) : rows_launch_t<bf16, 16>(p, batch, st);
   if (wbits == 8) return dtype == BLR_F16 ? rows_launch_t<f16, 8>(p, batch, st) : rows_launch_t<bf16, 8>(p, batch, st);
   return dtype == BLR_F16 ? rows_launch_t<f16, 4>(p, batch, st) : rows_launch_t<bf16, 4>(p, batch, st);
+}
+
+// What the launch before a planned product can fetch ahead for it; nblocks2 = 0 when the chunks are not whole 16-byte pieces
+// or the factor is too small to matter.
+RowsPrefetch rows_prefetch_plan(const RowsParams& p, int batch, int wbits, bool nk) {
+  RowsPrefetch f = {};
+  static const int enabled = env_i("BLR_DR_PREFETCH", 1);
+  static const int e_kb = env_i("BLR_DR_PREFETCH_KB", 96);
+  if (!enabled) return f;
+  const int64_t w_bytes = (int64_t)batch * p.K * p.N * wbits / 8;
+  if (w_bytes < (1 << 20)) return f;
+  f.W = reinterpret_cast<const char*>(p.W); f.w_bs_bytes = p.w_bs * wbits / 8;
+  if (nk) {                                              // chunk = 16 npc whole rows of K elements: one contiguous run
+    const int cw = p.npc * 16;
+    f.chunk_step = (uint32_t)((int64_t)cw * p.K * 2); f.row_stride = 0; f.nrows = 1;
+    f.piece16 = f.chunk_step / 16;
+    f.last_piece16 = (uint32_t)((int64_t)(p.N - (int)(p.nch.d - 1) * cw) * p.K * 2 / 16);
+  } else {                                               // chunk = K rows of 8 npc columns
+    const int cw = p.npc * 8;
+    const int64_t piece = (int64_t)cw * wbits / 8, row = (int64_t)p.N * wbits / 8;
+    if (piece % 16 || row % 16 || f.w_bs_bytes % 16) return f;
+    f.chunk_step = (uint32_t)piece; f.row_stride = (uint32_t)row; f.nrows = (uint32_t)p.K;
+    f.piece16 = (uint32_t)(piece / 16);
+    f.last_piece16 = (uint32_t)((row - (int64_t)(p.nch.d - 1) * piece) / 16);
+  }
+  f.nch = p.nch; f.xcd_span = p.xcd_span;
+  f.nblocks2 = (uint32_t)batch * p.nch.d;
+  // per workgroup: what a compute unit draws during the launch (about 35 GB/s for 2 - 3 us), and an XCD's share within 3 MB of its L2
+  int64_t budget = (int64_t)e_kb * 1024;
+  const int64_t per_xcd = (int64_t)3 << 20;
+  if (budget * ((f.nblocks2 + 7) / 8) > per_xcd) budget = per_xcd / ((f.nblocks2 + 7) / 8);
+  f.budget16 = (uint32_t)(budget / 16);
+  if (f.budget16 == 0) f.nblocks2 = 0;
+  return f;
 }
 
 }  // namespace
@@ -539,7 +629,16 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
 
   const void* ep_bias = nullptr; int ep_act = 0;
   if (epilogue_pending(&ep_bias, &ep_act)) { s2.ep = 1; s2.bias = ep_bias; s2.act = ep_act; }
-  int rc = rows_product(s1, b * mks, a.dtype, a.wbits, false, st);
+  int rc = rows_plan(s1, b * mks, a.dtype, a.wbits, false);
+  if (rc) return rc;
+  rc = rows_plan(s2, bo, a.dtype, a.wbits, u_nk);
+  if (rc) return rc;
+  // Fetching ahead pays where the launch in between is trivial (the sum of slices of low rank and of sliced Monarch) and the
+  // factor small: 11008 -> 4096 at 16 rows, low rank 18.8 -> 17.6 us, Monarch 18.6 -> 17.6 us.  Next to the BLAST mix, which is
+  // itself waiting on memory, it costs more than it gives (4096 -> 22016: 20.0 -> 21.9 us; 11008 -> 4096: 17.8 -> 18.3 us).
+  const bool ahead = (lowrank || (monarch && mks > 1)) && (int64_t)bo * R * Q * a.wbits / 8 <= (int64_t)12 << 20;
+  const RowsPrefetch pf = ahead ? rows_prefetch_plan(s2, bo, a.wbits, u_nk) : RowsPrefetch{};
+  rc = rows_launch(s1, b * mks, a.dtype, a.wbits, false, st);
   if (rc) return rc;
   int64_t si, sj, sr;
   if (a.s_layout == BLR_S_JIR) { sj = (int64_t)b * R; si = R; sr = 1; }
@@ -547,24 +646,26 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   else { si = (int64_t)b * R; sj = R; sr = 1; }
   if (monarch && mks > 1) {
     const int64_t items = (int64_t)bo * M * R / 4;
-    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_perm_sum_kernel<f16>, dim3((unsigned)cdiv(items, 256)), dim3(256), 0, st, (const f16*)Y, (f16*)Z, mks, M, R, a.perm_per, items);
-    else hipLaunchKernelGGL(rows_perm_sum_kernel<bf16>, dim3((unsigned)cdiv(items, 256)), dim3(256), 0, st, (const bf16*)Y, (bf16*)Z, mks, M, R, a.perm_per, items);
+    const uint32_t nmix = (uint32_t)cdiv(items, 256);
+    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_perm_sum_kernel<f16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const f16*)Y, (f16*)Z, mks, M, R, a.perm_per, items, pf, nmix);
+    else hipLaunchKernelGGL(rows_perm_sum_kernel<bf16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const bf16*)Y, (bf16*)Z, mks, M, R, a.perm_per, items, pf, nmix);
     BLR_CHECK_LAUNCH("rows_perm_sum");
   } else if (monarch)
     rc = BLR_OK;
   else if (lowrank) {
     const int64_t mr4 = (int64_t)M * R / 4;
-    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_sum_kernel<f16>, dim3((unsigned)cdiv(mr4, 256)), dim3(256), 0, st, (const f16*)Y, (f16*)Z, b, mr4);
-    else hipLaunchKernelGGL(rows_sum_kernel<bf16>, dim3((unsigned)cdiv(mr4, 256)), dim3(256), 0, st, (const bf16*)Y, (bf16*)Z, b, mr4);
+    const uint32_t nmix = (uint32_t)cdiv(mr4, 256);
+    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_sum_kernel<f16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const f16*)Y, (f16*)Z, b, mr4, pf, nmix);
+    else hipLaunchKernelGGL(rows_sum_kernel<bf16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const bf16*)Y, (bf16*)Z, b, mr4, pf, nmix);
     BLR_CHECK_LAUNCH("rows_sum");
   } else if (sr == 1 && si % 4 == 0 && sj % 4 == 0 && R % 4 == 0 && aligned(a.S, 8) && (int64_t)M * b * (R / 4) * (R / 4) < ((int64_t)1 << 32) && b < 65536)   // the multiply-high division is exact below 2^32 / divisor
-    rc = a.dtype == BLR_F16 ? rows_mix_t<f16>(Y, a.S, Z, M, b, R, si, sj, st) : rows_mix_t<bf16>(Y, a.S, Z, M, b, R, si, sj, st);
+    rc = a.dtype == BLR_F16 ? rows_mix_t<f16>(Y, a.S, Z, M, b, R, si, sj, pf, st) : rows_mix_t<bf16>(Y, a.S, Z, M, b, R, si, sj, pf, st);
   else if (a.s_layout == BLR_S_RIJ && b == 16 && R % 4 == 0 && aligned(a.S, 16) && (int64_t)M * (R / 4) * (R / 4) < ((int64_t)1 << 32))
-    rc = a.dtype == BLR_F16 ? rows_mix_rij_t<f16>(Y, a.S, Z, M, R, st) : rows_mix_rij_t<bf16>(Y, a.S, Z, M, R, st);
+    rc = a.dtype == BLR_F16 ? rows_mix_rij_t<f16>(Y, a.S, Z, M, R, pf, st) : rows_mix_rij_t<bf16>(Y, a.S, Z, M, R, pf, st);
   else
     rc = blast_mix_launch(Y, a.S, Z, M, b, R, si, sj, sr, a.dtype, st, 0);
   if (rc) return rc;
-  rc = rows_product(s2, bo, a.dtype, a.wbits, u_nk, st);
+  rc = rows_launch(s2, bo, a.dtype, a.wbits, u_nk, st);
   if (rc == BLR_OK && s2.ep) epilogue_taken();
   return rc == 1 ? BLR_ERR_UNSUPPORTED : rc;
 }
