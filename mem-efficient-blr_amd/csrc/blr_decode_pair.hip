@@ -285,7 +285,10 @@ __global__ __launch_bounds__(DP_NT) void pair_stage1_kernel(PairParams p) {
 // memory read in linear order; a lane meets the same eight ranks in every load (its z sits in registers), keeps one
 // partial dot product per load and row, and the partials of a row are added up across its lanes: two DPP steps inside
 // the quad, one pass through LDS for the rest.  Needs rank = 8 * 2^n, 128 <= rank <= 4096.
-template <typename T, int MT, int WB, int PFG, bool QR>
+// JJ: input blocks a mix thread combines at most, 2 or 4 - a load costs its turn in the memory pipeline even with every lane
+// out of bounds, so calls whose threads combine one or two blocks (rank 512 with 16 blocks) get a kernel without the other two
+// (4096 -> 4096 at one row: 9.8 -> 9.7 us, with U as (b, q, r) 9.9 -> 9.4 us).
+template <typename T, int MT, int WB, int PFG, bool QR, int JJ>
 __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   constexpr int TR4_BASE = 512; (void)TR4_BASE;
   constexpr int EPL = 128 / WB;
@@ -313,14 +316,14 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   const __amdgpu_buffer_rsrc_t ybuf = rbuf2(p.y, (uint32_t)p.ks1 * p.b * M * R * 2u);
   const __amdgpu_buffer_rsrc_t sbuf = rbuf2(p.S ? p.S : p.x, p.S ? (uint32_t)p.b * p.bo * R * 2u : 2u);
   const int ib = p.bo > 1 ? (int)i2 : 0;               // (a single output block: every slab uses S of block 0, or none)
-  u32x4 yq[MT][KSM][DP_JJ];
-  u32x4 sq[DP_JJ];
+  u32x4 yq[MT][KSM][JJ];
+  u32x4 sq[JJ];
   // Monarch: the "mix" is a gather - the eight ranks of this thread come from one input block (the period is a multiple
   // of eight), so group 0 fetches that one piece of y and the other groups contribute nothing
   const int pj = p.perm_per > 0 ? (oct * 8) / p.perm_per : 0;
   const int pr = p.perm_per > 0 ? (int)i2 * p.perm_per + (oct * 8 - pj * p.perm_per) : oct * 8;
 #pragma unroll
-  for (int jj = 0; jj < DP_JJ; ++jj) {
+  for (int jj = 0; jj < JJ; ++jj) {
     const int j = p.perm_per > 0 ? pj : jg * p.jpg + jj;
     const bool on = p.perm_per > 0 ? (mix_on && jj == 0 && jg == 0) : (mix_on && jj < p.jpg && j < p.b);
     sq[jj] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(sbuf, (on && p.S) ? (uint32_t)(ib * (int)p.s_si + j * (int)p.s_sj + oct * 8) * 2u : DP_OOB, 0, 0));
@@ -354,7 +357,7 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) z8[e] = 0.0f;
 #pragma unroll
-      for (int jj = 0; jj < DP_JJ; ++jj) {
+      for (int jj = 0; jj < JJ; ++jj) {
         if (jj < p.jpg) {
           float y8[8];
 #pragma unroll
@@ -532,41 +535,45 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
 
 // ---- host side --------------------------------------------------------------------------------------------------
 namespace {
-template <typename T, int MT, int WB>
-void* pair_slab_fn(int pfg, bool qr) {
+template <typename T, int MT, int WB, int JJ>
+void* pair_slab_fn_jj(int pfg, bool qr) {
   if constexpr (WB == 16) {
     if (qr) {
       switch (pfg) {
-        case 1: return (void*)pair_slab_kernel<T, MT, 16, 1, true>;
-        case 2: return (void*)pair_slab_kernel<T, MT, 16, 2, true>;
-        case 3: if constexpr (MT <= 2) return (void*)pair_slab_kernel<T, MT, 16, 3, true>; else return nullptr;
-        case 4: if constexpr (MT <= 2) return (void*)pair_slab_kernel<T, MT, 16, 4, true>; else return nullptr;
+        case 1: return (void*)pair_slab_kernel<T, MT, 16, 1, true, JJ>;
+        case 2: return (void*)pair_slab_kernel<T, MT, 16, 2, true, JJ>;
+        case 3: if constexpr (MT <= 2) return (void*)pair_slab_kernel<T, MT, 16, 3, true, JJ>; else return nullptr;
+        case 4: if constexpr (MT <= 2) return (void*)pair_slab_kernel<T, MT, 16, 4, true, JJ>; else return nullptr;
         default: return nullptr;
       }
     }
   }
   if (qr) return nullptr;
   switch (pfg) {
-    case 1: return (void*)pair_slab_kernel<T, MT, WB, 1, false>;
-    case 2: return (void*)pair_slab_kernel<T, MT, WB, 2, false>;
-    case 3: if constexpr (WB == 16) return (void*)pair_slab_kernel<T, MT, WB, 3, false>; else return nullptr;
-    case 4: if constexpr (WB == 16) return (void*)pair_slab_kernel<T, MT, WB, 4, false>; else return nullptr;
+    case 1: return (void*)pair_slab_kernel<T, MT, WB, 1, false, JJ>;
+    case 2: return (void*)pair_slab_kernel<T, MT, WB, 2, false, JJ>;
+    case 3: if constexpr (WB == 16) return (void*)pair_slab_kernel<T, MT, WB, 3, false, JJ>; else return nullptr;
+    case 4: if constexpr (WB == 16) return (void*)pair_slab_kernel<T, MT, WB, 4, false, JJ>; else return nullptr;
     default: return nullptr;
   }
 }
+template <typename T, int MT, int WB>
+void* pair_slab_fn(int pfg, bool qr, int jpg) {
+  return jpg <= 2 ? pair_slab_fn_jj<T, MT, WB, 2>(pfg, qr) : pair_slab_fn_jj<T, MT, WB, DP_JJ>(pfg, qr);
+}
 // two-byte weights at 1, 2 and 4 token rows, int8 codes at 1 and 2, int4 codes at 1 (as decode3_kernel)
 template <typename T>
-bool pair_fns(int MT, int wbits, int pfg, bool qr, bool st, void** f1, void** f2) {
+bool pair_fns(int MT, int wbits, int pfg, bool qr, bool st, int jpg, void** f1, void** f2) {
   *f1 = *f2 = nullptr;
   if (wbits == 16) {
-    if (MT == 1) { *f1 = st ? (void*)pair_stage1_kernel<T, 1, 16, true> : (void*)pair_stage1_kernel<T, 1, 16, false>; *f2 = pair_slab_fn<T, 1, 16>(pfg, qr); }
-    else if (MT == 2) { *f1 = st ? (void*)pair_stage1_kernel<T, 2, 16, true> : (void*)pair_stage1_kernel<T, 2, 16, false>; *f2 = pair_slab_fn<T, 2, 16>(pfg, qr); }
-    else { *f1 = st ? (void*)pair_stage1_kernel<T, 4, 16, true> : (void*)pair_stage1_kernel<T, 4, 16, false>; *f2 = pair_slab_fn<T, 4, 16>(pfg, qr); }
+    if (MT == 1) { *f1 = st ? (void*)pair_stage1_kernel<T, 1, 16, true> : (void*)pair_stage1_kernel<T, 1, 16, false>; *f2 = pair_slab_fn<T, 1, 16>(pfg, qr, jpg); }
+    else if (MT == 2) { *f1 = st ? (void*)pair_stage1_kernel<T, 2, 16, true> : (void*)pair_stage1_kernel<T, 2, 16, false>; *f2 = pair_slab_fn<T, 2, 16>(pfg, qr, jpg); }
+    else { *f1 = st ? (void*)pair_stage1_kernel<T, 4, 16, true> : (void*)pair_stage1_kernel<T, 4, 16, false>; *f2 = pair_slab_fn<T, 4, 16>(pfg, qr, jpg); }
   } else if (wbits == 8) {
-    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 8, false>; *f2 = pair_slab_fn<T, 1, 8>(pfg, qr); }
-    else if (MT == 2) { *f1 = (void*)pair_stage1_kernel<T, 2, 8, false>; *f2 = pair_slab_fn<T, 2, 8>(pfg, qr); }
+    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 8, false>; *f2 = pair_slab_fn<T, 1, 8>(pfg, qr, jpg); }
+    else if (MT == 2) { *f1 = (void*)pair_stage1_kernel<T, 2, 8, false>; *f2 = pair_slab_fn<T, 2, 8>(pfg, qr, jpg); }
   } else if (wbits == 4) {
-    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 4, false>; *f2 = pair_slab_fn<T, 1, 4>(pfg, qr); }
+    if (MT == 1) { *f1 = (void*)pair_stage1_kernel<T, 1, 4, false>; *f2 = pair_slab_fn<T, 1, 4>(pfg, qr, jpg); }
   }
   return *f1 && *f2;
 }
@@ -707,7 +714,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   }
   const int pfg = (p.pfn + 7) / 8;
   void *f1 = nullptr, *f2 = nullptr;
-  const bool have = a.dtype == BLR_F16 ? pair_fns<f16>(MT, WBITS, pfg, qr, s_turn, &f1, &f2) : pair_fns<bf16>(MT, WBITS, pfg, qr, s_turn, &f1, &f2);
+  const bool have = a.dtype == BLR_F16 ? pair_fns<f16>(MT, WBITS, pfg, qr, s_turn, p.jpg, &f1, &f2) : pair_fns<bf16>(MT, WBITS, pfg, qr, s_turn, p.jpg, &f1, &f2);
   if (!have) return d2_bail(__LINE__);
   const int grid1 = b * (int)p.nch1.d * p.ks1, grid2 = bo * (int)p.nch2.d;
   // Launch 1 also warms the L2 with U where its own items are long enough to hide that and all of U fits: extra workgroups,
