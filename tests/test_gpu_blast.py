@@ -171,6 +171,46 @@ def test_blast_llama7b_prefill_rows(name, layer):
     assert torch.isfinite(out).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_blast_tiled_intermediates_element_by_element(dtype):
+    """Y and Z of the tiled path (M > 16) checked per element, with S eight times larger than in the other tests so that the
+    partial sums of the mix are large against single terms.  fp16 adds the up to b terms of z in packed fp16 (bf16: in fp32),
+    Y and Z are rounded to the 16-bit type as in the reference (triton_funcs/blast_kernels.py:543,548), so an element of z may
+    be off by a few roundings of the magnitude sum_j |S_ij y_j|: bound (b + 4) * eps * sum_j |S_ij| |y_j| per element, eps =
+    2^-11 (fp16) or 2^-8 (bf16)."""
+    from triton_funcs import _lib as L
+    b, p, q, r, M = 16, 64, 72, 128, 96
+    x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=21)
+    S = S * 8.0
+    Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+    xd, Ud, Vd, Sd = dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype)
+    out = torch.empty((M, b * q), device="cuda", dtype=dtype)
+    z = torch.full((b, M, r), float("nan"), device="cuda", dtype=dtype)
+    y = torch.full((b, M, r), float("nan"), device="cuda", dtype=dtype)
+    dt = L.dtype_code(dtype)
+    ws = torch.zeros(max(L.lib().blr_blast_workspace_bytes(M, b * p, b * q, b, r, dt, L.ALGO_TILED), 1 << 20), dtype=torch.uint8, device="cuda")
+    say(f"[case] tiled BLAST, Y and Z per element, {dtype}")
+    rc = L.lib().blr_blast_fwd(xd.data_ptr(), xd.stride(0), Ud.data_ptr(), Vd.data_ptr(), Sd.data_ptr(), out.data_ptr(), out.stride(0),
+                               z.data_ptr(), y.data_ptr(), M, b * p, b * q, b, r, dt, L.U_RQ, L.S_JIR, L.ALGO_TILED, ws.data_ptr(), ws.numel(),
+                               L.stream_ptr(xd.device))
+    assert rc == 0, L.lib().blr_last_error().decode()
+    torch.cuda.synchronize()
+    eps = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    xr, Vr, Sr = rounded(x, dtype), rounded(Vt, dtype), rounded(S, dtype)
+    _, z_ref, y_ref = O.blast_forward(xr, rounded(U, dtype), Vr, Sr)
+    y_mag = np.einsum("njp,jrp->jnr", np.abs(xr.reshape(M, b, p)), np.abs(Vr))
+    y_got = y.double().cpu().numpy()
+    assert np.all(np.abs(y_got - y_ref) <= 2 * eps * y_mag + 1e-30), "an element of Y is off by more than its rounding"
+    # z from the Y the kernel actually stored (so the bound is about the mix alone)
+    z_from_y = np.einsum("ijr,jnr->inr", Sr, y_got)
+    z_mag = np.einsum("ijr,jnr->inr", np.abs(Sr), np.abs(y_got))
+    err = np.abs(z.double().cpu().numpy() - z_from_y)
+    worst = float(np.max(err / (z_mag + 1e-30)))
+    say(f"  worst |z - z_ref| / sum_j |S y| = {worst:.3e} (bound {(b + 4) * eps:.3e})")
+    assert np.all(err <= (b + 4) * eps * z_mag + 1e-30)
+    assert_close(out, O.blast_forward(xr, rounded(U, dtype), Vr, Sr)[0], dtype, "out with large S", scale=2.0)
+
+
 def test_blast_linearity_full_size():
     """Size-independent property at full gate_up shape: f(2a - 3b) == 2 f(a) - 3 f(b) within rounding."""
     from triton_funcs import blast_kernels as K
