@@ -1,4 +1,8 @@
-// BLAST at 5 to 16 token rows as three launches: y = x V on the matrix cores, the rank-space mix, out = z U on the matrix cores.
+// BLAST at 2 to 16 token rows as three launches: y = x V on the matrix cores, the rank-space mix, out = z U on the matrix cores.
+// Low rank runs as BLAST with one output block and S = 1 (its middle launch adds the k-slices of x A), Monarch as two launches
+// (its permutation is the store pattern of the first product) or, with input blocks deeper than 1024 rows, as three (the
+// blocks are cut into slices; the middle launch adds them while it permutes).  A middle launch that only adds slices also
+// carries workgroups that load the second product's factor into L2 (rows_prefetch).
 //
 // rows_product_kernel computes a batch of skinny products  out[bt] (M x N) = A[bt] (M x K) W[bt] (K x N),  M <= 16, with W
 // row-major (the column index contiguous) - the layout of V (b, p, r) and of U (b, r, q).  A workgroup of eight waves owns
