@@ -1013,7 +1013,11 @@ static void mix_dispatch(dim3 grid, size_t lds, hipStream_t st, const void* Y, c
     hipLaunchKernelGGL((blast_mix_kernel<T, 0>), grid, dim3(256), lds, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, sat8);
 }
 
-// S slab of a workgroup of the mix kernels: s_t[(j * b + i) * 64 + r] = S(i, j, r0 + r) for 64 ranks, zero past R.
+// S slab of a workgroup of the mix kernels: s_t[(j * b + i) * MIX_LDR + r] = S(i, j, r0 + r) for 64 ranks, zero past R.  Rows
+// of 72 elements, not 64: staging S stored (r, i, j) writes one (j, i) row per lane, and with rows of 128 bytes every lane of a
+// wave would hit the same bank (the mix of a 4608 -> 1152, rank 576 layer at 4096 rows took 54 us with S in that order and
+// 40 us with S (j, i, r); 16-byte reads of a row stay aligned with 144-byte rows).
+constexpr int MIX_LDR = 72;
 // 16-byte pieces along whichever of r or j is contiguous in memory; element-wise otherwise.
 template <typename T>
 __device__ __forceinline__ void mix_stage_s(const T* __restrict__ S, T* s_t, int b, int R, int r0,
@@ -1028,7 +1032,7 @@ __device__ __forceinline__ void mix_stage_s(const T* __restrict__ S, T* s_t, int
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = (T)0.0f;
       if (r0 + r8 < R) v = *reinterpret_cast<const V8*>(&S[(int64_t)i * s_si + (int64_t)j * s_sj + r0 + r8]);
-      *reinterpret_cast<V8*>(&s_t[ji * 64 + r8]) = v;
+      *reinterpret_cast<V8*>(&s_t[ji * MIX_LDR + r8]) = v;
     }
   } else if (vec_ok && s_sj == 1 && (b & 7) == 0) {            // (r, i, j): j contiguous
     const int jv = b >> 3;
@@ -1040,7 +1044,7 @@ __device__ __forceinline__ void mix_stage_s(const T* __restrict__ S, T* s_t, int
       for (int e = 0; e < 8; ++e) v[e] = (T)0.0f;
       if (r0 + r < R) v = *reinterpret_cast<const V8*>(&S[(int64_t)(r0 + r) * s_sr + (int64_t)i * s_si + j8]);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s_t[((j8 + e) * b + i) * 64 + r] = v[e];
+      for (int e = 0; e < 8; ++e) s_t[((j8 + e) * b + i) * MIX_LDR + r] = v[e];
     }
   } else {
     for (int idx = tid; idx < b * b * 64; idx += 256) {
@@ -1048,7 +1052,7 @@ __device__ __forceinline__ void mix_stage_s(const T* __restrict__ S, T* s_t, int
       const int j = ji / b, i = ji - j * b;
       T v = (T)0.0f;
       if (r0 + r < R) v = S[(int64_t)i * s_si + (int64_t)j * s_sj + (int64_t)(r0 + r) * s_sr];
-      s_t[idx] = v;
+      s_t[ji * MIX_LDR + r] = v;
     }
   }
 }
@@ -1084,7 +1088,7 @@ __global__ __launch_bounds__(256) void blast_mix_vec_kernel(const T* __restrict_
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         if (j < b) {
-          V8 sv = *reinterpret_cast<const V8*>(&s_t[(j * b + i) * 64 + rl * 8]);
+          V8 sv = *reinterpret_cast<const V8*>(&s_t[(j * b + i) * MIX_LDR + rl * 8]);
 #pragma unroll
           for (int e = 0; e < 8; ++e) acc[e] = fmaf(TypeTraits<T>::to_f32(sv[e]), TypeTraits<T>::to_f32(yv[j][e]), acc[e]);
         }
@@ -1136,7 +1140,7 @@ __global__ __launch_bounds__(256) void blast_mix_h2_kernel(const f16* __restrict
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         if (FULL16 || j < b) {
-          const H8 sv = *reinterpret_cast<const H8*>(&s_t[(j * b + i) * 64 + rl * 8]);
+          const H8 sv = *reinterpret_cast<const H8*>(&s_t[(j * b + i) * MIX_LDR + rl * 8]);
 #pragma unroll
           for (int u = 0; u < MB; ++u)
 #pragma unroll
@@ -1189,7 +1193,7 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
   }
   int r_chunks = (int)cdiv(R, 64);
   if (dtype != BLR_F32 && b <= 16 && R % 8 == 0 && aligned(Y, 16) && aligned(Z, 16)) {
-    size_t lds = (size_t)b * b * 64 * 2;
+    size_t lds = (size_t)b * b * MIX_LDR * 2;
     static const int mpw_env = [] { const char* e = getenv("BLR_MIX_MPW"); return e ? atoi(e) : 0; }();
     // S may be fetched in 16-byte pieces if every piece starts on a 16-byte boundary
     const int s_vec = aligned(S, 16) && ((s_sr == 1 && s_si % 8 == 0 && s_sj % 8 == 0) ||
