@@ -193,14 +193,19 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
     for (int s = 0; s < STEPS; ++s) av[s] = u32x4{0u, 0u, 0u, 0u};
   }
   if constexpr (NK) {
-    // column groups past the chunk or the factor, and k past K, read as zero (offset out of the buffer's bounds)
+    // columns past the factor and k past K read as zero (offset out of the buffer's bounds); column groups past the chunk are
+    // not asked for at all (a load costs its turn in the memory pipeline even with every lane out of bounds; their registers
+    // stay undefined and only reach columns that are never stored)
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s)
+    for (int t = 0; t < 8; ++t) {
+      if (t < p.npc) {
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const int c = colp + 16 * t, k = kb + 32 * s;
-        wr[s][t] = Piece::load(wb, (t < p.npc && c < N && k < K) ? (uint32_t)(c * K + k) * 2u : DR_OOB);
+        for (int s = 0; s < STEPS; ++s) {
+          const int c = colp + 16 * t, k = kb + 32 * s;
+          wr[s][t] = Piece::load(wb, (c < N && k < K) ? (uint32_t)(c * K + k) * 2u : DR_OOB);
+        }
       }
+    }
   } else if (live) {
     const uint32_t wbase = (uint32_t)(kb * N + colp) * (uint32_t)WB / 8u;
     const uint32_t rowb = (uint32_t)N * (uint32_t)WB / 8u;
