@@ -662,7 +662,12 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
     if (gr < g.M && gc < g.N) {
       V8 v = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
       if (EP) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc, gr);
-      *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = v;
+      if (g.epi == EPI_MONARCH_SCATTER) {            // column c of entry bt -> block c / per, column bt * per + c % per
+        const int d = gc / g.per;
+        *reinterpret_cast<V8*>(&C[(int64_t)d * g.sL + (int64_t)gr * g.ldc + (int64_t)bt * g.per + (gc - d * g.per)]) = v;
+      } else {
+        *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = v;
+      }
     }
   }
 }
@@ -820,7 +825,10 @@ size_t gemm_splitk_bytes(int M, int N, int K, int dtype) {
 }
 
 static bool ring_ok(const GemmArgs& g) {
-  if (g.epi != EPI_PLAIN || g.cn < 1 || g.N < 8 || g.N % 8 || g.K % 8) return false;
+  if (g.cn < 1 || g.N < 8 || g.N % 8 || g.K % 8) return false;
+  // Monarch's scatter of the first product: an 8-column vector stays inside one destination block when the period is a multiple of 8
+  if (g.epi == EPI_MONARCH_SCATTER && (g.per % 8 || g.sL % 8 || g.cn != 1 || g.sat8 || g.bias || g.act || g.gate || g.resid)) return false;
+  if (g.epi != EPI_PLAIN && g.epi != EPI_MONARCH_SCATTER) return false;
   if (!aligned(g.A, 16) || !aligned(g.B, 16) || g.lda % 8 || g.sA % 8 || g.ldb % 8 || g.sB % 8) return false;
   if (g.cn == 1) {                                   // 16-byte stores, the fused output stage reads its vector the same way
     if (!aligned(g.C, 16) || (g.bias && !aligned(g.bias, 16)) || (g.gate && (!aligned(g.gate, 16) || g.ld_gate % 8)) || (g.resid && (!aligned(g.resid, 16) || g.ld_resid % 8)) || g.ldc % 8 || g.sC % 8) return false;
@@ -882,7 +890,7 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   // BLR_GEMM_RING_WAVES = 4 or 8 the workgroup size of the two larger ones - options that tests switch with
   // blr_set_option).
   const int ring = option_value(OPT_GEMM_RING, 1);
-  if (ring > 0 && force == 0 && ring_ok(g) && g.splitk_ws && g.batch == 1 && g.cn == 1 && !g.sat8 && !g.bias && !g.act && !g.gate && !g.resid) {
+  if (ring > 0 && force == 0 && ring_ok(g) && g.epi == EPI_PLAIN && g.splitk_ws && g.batch == 1 && g.cn == 1 && !g.sat8 && !g.bias && !g.act && !g.gate && !g.resid) {
     // few tiles, long reduction: slices of K as the batch of the partial-sum kernel, then one pass that adds them up
     int kc = 0;
     const int splits = option_value(OPT_GEMM_SPLITK, 1) == 0 ? 1 : splitk_plan(g.M, g.N, g.K, &kc);
