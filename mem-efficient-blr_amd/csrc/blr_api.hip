@@ -339,6 +339,19 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   else if (s_layout == BLR_S_RIJ) { sr = (int64_t)b * b; si = b; sj = 1; }
   else { si = (int64_t)b * r; sj = r; sr = 1; }
   int rc = 1;
+  // A few dozen rows are still a weight-streaming problem: 256-row tiles would leave most compute units without one and the
+  // others with a long stream each (4096 -> 4096 at 17 rows: 36 us through the tiles, 12 us at 16 rows through the few-row
+  // kernels).  Up to 128 rows the three launches of the few-row path run over tiles of 16 rows with the weights held in registers
+  // (at 128 rows 32 / 44 / 43 us against 39 / 48 / 56 us through the tiles on the three Llama-7B layers).
+  static const int rows_max_m = getenv("BLR_TILED_ROWS_MAX_M") ? atoi(getenv("BLR_TILED_ROWS_MAX_M")) : 128;
+  if (M <= rows_max_m && !y_out && !z_out && !sat8 && fused <= 0 && dtype != BLR_F32) {
+    StreamBlastArgs s = {};
+    s.x = x; s.ldx = ldx; s.U = U; s.V = V; s.S = S; s.out = out; s.ldo = ldo;
+    s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
+    s.dtype = dtype; s.u_layout = u_layout; s.s_layout = s_layout; s.wbits = 16;
+    rc = decode_rows_launch(s, ws, ws_bytes, st);
+    if (rc != 1) return rc;
+  }
   // Nobody asked for Y: x V and the mix can run as one launch with Y kept inside the compute units (BLR_ALGO_FUSED).  Chosen
   // by itself only for narrow input blocks: the fused kernel re-reads V once per 32 rows, and from about 128 columns per
   // block on that costs more than the round trip of Y it saves (measured at 4096 rows: 1152 -> 1152, r = 288: 64 against
@@ -458,6 +471,14 @@ int blr_blast_q_fwd(const void* x, int64_t ldx, const void* u_codes, const void*
   if (M > 16) {
     size_t need = blr_blast_q_workspace_bytes(M, in_f, out_f, b, r, bits);
     if (!ws || ws_bytes < need) { set_error("blast_q: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
+    if (M <= 128) {                                  // and up to 128 rows too, in tiles of 16 rows: no dequantized copy of the weights
+      StreamBlastArgs s = {};
+      s.x = x; s.ldx = ldx; s.U = u_codes; s.V = v_codes; s.S = S; s.u_scales = u_scales; s.v_scales = v_scales;
+      s.out = out; s.ldo = ldo; s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
+      s.dtype = dtype; s.u_layout = BLR_U_RQ; s.s_layout = BLR_S_RIJ; s.wbits = bits;
+      rc = decode_rows_launch(s, ws, ws_bytes, st);
+      if (rc != 1) return rc;
+    }
     const size_t sub = align_up(M <= 16 ? stream_blast_workspace(M, in_f, out_f, b, r, bits) : 2 * align_up((size_t)b * M * r * 2, 256), 256);
     char* wp = reinterpret_cast<char*>(ws) + sub;
     void* Ud = wp; wp += align_up((size_t)r * out_f * 2, 256);
@@ -496,6 +517,18 @@ int blr_quantize_sym(const void* w, int dtype, int64_t outer, int64_t reduce, in
 }
 
 // ---- Monarch --------------------------------------------------------------------------------------
+// Monarch at 17..128 rows through the few-row kernels: bytes of their intermediates - the first product's output (in slices
+// of the input blocks when those are deeper than 1024 rows, as decode_rows_launch cuts them) and the permuted z.
+static size_t monarch_rows_bytes(int M, int in_f, int b, int rank, int dtype) {
+  if (M <= 16 || M > 128 || dtype == BLR_F32 || b < 2 || in_f % b || rank % b) return 0;
+  const int P = in_f / b;
+  int mks = 1;
+  if (P > 1024)
+    for (int ks = (P + 1023) / 1024; ks <= 8; ++ks)
+      if (P % ks == 0 && (P / ks) % 8 == 0) { mks = ks; break; }
+  return align_up((size_t)b * mks * M * rank * 2, 256) + align_up((size_t)b * M * rank * 2, 256);
+}
+
 size_t blr_monarch_workspace_bytes(int M, int in_f, int out_f, int b, int rank, int dtype, int algo) {
   if (M <= 0 || b <= 0 || rank <= 0) return 0;
   int a = resolve_algo(algo, M, dtype, false);
@@ -504,7 +537,8 @@ size_t blr_monarch_workspace_bytes(int M, int in_f, int out_f, int b, int rank, 
     size_t s = stream_generic_workspace(2, M, in_f, out_f, b, rank);
     return s > tiled ? s : tiled;
   }
-  return tiled;
+  const size_t rows = monarch_rows_bytes(M, in_f, b, rank, dtype);
+  return rows > tiled ? rows : tiled;
 }
 
 int blr_monarch_fwd(const void* x, int64_t ldx, const void* w1, const void* w2,
@@ -529,6 +563,17 @@ int blr_monarch_fwd(const void* x, int64_t ldx, const void* w1, const void* w2,
     return stream_generic_launch(s, st);
   }
   if (a != BLR_ALGO_TILED) { set_error("monarch: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
+  if (!out1 && ws && monarch_rows_bytes(M, in_f, b, rank, dtype) && ws_bytes >= monarch_rows_bytes(M, in_f, b, rank, dtype)) {
+    StreamBlastArgs bl = {};
+    bl.x = x; bl.ldx = ldx; bl.U = w2; bl.V = w1; bl.S = nullptr; bl.out = out; bl.ldo = ldo;
+    bl.M = M; bl.in_f = in_f; bl.out_f = out_f; bl.b = b; bl.bo = b; bl.r = rank;
+    bl.dtype = dtype; bl.u_layout = w2_layout == BLR_W2_SR ? BLR_U_QR : BLR_U_RQ; bl.s_layout = BLR_S_IJR; bl.wbits = 16;
+    bl.perm_per = per;
+    if (out_order == BLR_OUT_INTERLEAVED) { bl.out_bs = 1; bl.out_ns = b; }
+    else { bl.out_bs = S; bl.out_ns = 1; }
+    const int rc = decode_rows_launch(bl, ws, ws_bytes, st);
+    if (rc != 1) return rc;
+  }
   const size_t need = out1 ? 0 : align_up((size_t)b * M * rank * elt_size(dtype), 256);
   if (need && (!ws || ws_bytes < need)) { set_error("monarch: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
   void* O1 = out1 ? out1 : ws;
@@ -556,6 +601,19 @@ int blr_monarch_fwd(const void* x, int64_t ldx, const void* w1, const void* w2,
 }
 
 // ---- low rank -------------------------------------------------------------------------------------
+// Low rank at 17..128 rows through the few-row kernels: BLAST with the input cut into 16 (or 8, 4, 2) slices, one output block
+// and S = 1.  Bytes of its intermediates (0 when the shape is not for it); the launch returns 1 when it does not apply.
+static int low_rank_slices(int in_f) {
+  for (int c = 16; c >= 2; c >>= 1)
+    if (in_f % c == 0 && (in_f / c) % 8 == 0) return c;
+  return 0;
+}
+static size_t low_rank_rows_bytes(int M, int in_f, int r, int dtype) {
+  const int bi = low_rank_slices(in_f);
+  if (M <= 16 || M > 128 || dtype == BLR_F32 || !bi) return 0;
+  return align_up((size_t)bi * M * r * 2, 256) + align_up((size_t)M * r * 2, 256);
+}
+
 size_t blr_low_rank_workspace_bytes(int M, int in_f, int out_f, int r, int dtype, int algo) {
   if (M <= 0 || r <= 0) return 0;
   int a = resolve_algo(algo, M, dtype, false);
@@ -564,7 +622,9 @@ size_t blr_low_rank_workspace_bytes(int M, int in_f, int out_f, int r, int dtype
     size_t s = stream_generic_workspace(1, M, in_f, out_f, 1, r);
     return s > tiled ? s : tiled;
   }
-  return tiled + gemm_splitk_bytes(M, r, in_f, dtype);       // x.A has few output tiles and a long reduction: room to cut it along K
+  size_t need = tiled + gemm_splitk_bytes(M, r, in_f, dtype);   // x.A has few output tiles and a long reduction: room to cut it along K
+  const size_t rows = low_rank_rows_bytes(M, in_f, r, dtype);   // 17..128 rows: the few-row path (x A in up to 16 slices of the input)
+  return rows > need ? rows : need;
 }
 
 int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
@@ -586,6 +646,14 @@ int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
     return stream_generic_launch(s, st);
   }
   if (a != BLR_ALGO_TILED) { set_error("low_rank: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
+  if (!z_out && ws && low_rank_rows_bytes(M, in_f, r, dtype) && ws_bytes >= low_rank_rows_bytes(M, in_f, r, dtype)) {
+    StreamBlastArgs bl = {};
+    bl.x = x; bl.ldx = ldx; bl.U = B; bl.V = A; bl.S = nullptr; bl.out = out; bl.ldo = ldo;
+    bl.M = M; bl.in_f = in_f; bl.out_f = out_f; bl.b = low_rank_slices(in_f); bl.bo = 1; bl.r = r;
+    bl.dtype = dtype; bl.u_layout = BLR_U_RQ; bl.s_layout = BLR_S_IJR; bl.wbits = 16;
+    const int rc = decode_rows_launch(bl, ws, ws_bytes, st);
+    if (rc != 1) return rc;
+  }
   const size_t need = z_out ? 0 : align_up((size_t)M * r * elt_size(dtype), 256);
   if (need && (!ws || ws_bytes < need)) { set_error("low_rank: workspace %zu < %zu", ws_bytes, need); return BLR_ERR_WORKSPACE; }
   void* Z = z_out ? z_out : ws;

@@ -29,6 +29,7 @@ namespace {
 constexpr int DR_NT = 512;
 constexpr int DR_WAVES = 8;
 constexpr int DR_MAX_STEPS = 4;           // 32-row steps of a wave: 8 loads per lane each
+constexpr int DR_MAX_M = 128;             // token rows: tiles of 16 over the same registers of weights
 constexpr uint32_t DR_OOB = 0x80000000u;
 }  // namespace
 
@@ -51,6 +52,8 @@ struct RowsParams {
   int M, K, N;
   int kw;                                 // rows of a wave's share per round (a multiple of 32)
   int rounds;                             // passes of the eight waves over the rows
+  int mtiles;                             // 16-row tiles of A and out (M <= 16: one); more than one only with rounds == 1: the
+                                          // weights then stay in registers and every further tile costs products and a reduction
   int per; int64_t o_ls; FastDiv perdiv;  // per > 0: Monarch scatter - column c of entry bt goes to out[(c / per) * o_ls + m * o_ms + bt * per + c % per]
   int npc;                                // 16-byte column pieces of a chunk (1..16)
   FastDiv nch;                            // chunks per batch entry
@@ -166,6 +169,29 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
   // More than 8 waves x STEPS x 32 rows: the workgroup passes over the rows in rounds (the loads of a round are issued when
   // the products of the one before are done - one more trip to memory per extra round).
+  u32x4 av[STEPS];
+  typename Piece::raw_t wr[STEPS][8];
+  auto products = [&]() {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      if constexpr (NK) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = RowsMfma<T>::run(av[s], Piece::expand(wr[s][e]), acc[e]);
+      } else {
+        u32x4 wx[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) wx[t] = Piece::expand(wr[s][t]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+          u32x4 bv;
+#pragma unroll
+          for (int h = 0; h < 4; ++h) bv[h] = __builtin_amdgcn_perm(wx[2 * h + 1][e >> 1], wx[2 * h][e >> 1], sel);
+          acc[e] = RowsMfma<T>::run(av[s], bv, acc[e]);
+        }
+      }
+    }
+  };
   for (int ro = 0; ro < p.rounds; ++ro) {
   const int kb = (ro * DR_WAVES + wv) * p.kw + 8 * g;    // first of this lane's eight k of step 0
 
@@ -173,8 +199,6 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   // 16-byte piece of each.  Lanes without a row / without a column piece issue nothing (their registers stay undefined:
   // they only reach rows and columns of the product that are never stored), so a narrow chunk costs the load path
   // only what its live lanes fetch.
-  u32x4 av[STEPS];
-  typename Piece::raw_t wr[STEPS][8];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     asm volatile("" : "=v"(av[s]));
@@ -216,27 +240,24 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   }
 
   TR5(1);
-#pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    if constexpr (NK) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = RowsMfma<T>::run(av[s], Piece::expand(wr[s][e]), acc[e]);
-    } else {
-      u32x4 wx[8];
-#pragma unroll
-      for (int t = 0; t < 8; ++t) wx[t] = Piece::expand(wr[s][t]);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
-        u32x4 bv;
-#pragma unroll
-        for (int h = 0; h < 4; ++h) bv[h] = __builtin_amdgcn_perm(wx[2 * h + 1][e >> 1], wx[2 * h][e >> 1], sel);
-        acc[e] = RowsMfma<T>::run(av[s], bv, acc[e]);
-      }
-    }
-  }
+  products();
   }  // rounds
   TR5(2);
+  // More than 16 rows (one round only): the weights stay in the registers; per further tile of 16 rows the activations are
+  // fetched (asked for before the reduction of the tile before, so that they arrive under it), multiplied and reduced.
+  for (int mt = 0;; ++mt) {
+  const int mrow0 = mt * 16;
+  const bool more = mt + 1 < p.mtiles;
+  u32x4 avn[STEPS];
+  if (more) {
+    const int row = mrow0 + 16 + n, kb = wv * p.kw + 8 * g;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int k = kb + 32 * s;
+      const uint32_t off = (row < p.M && k < K) ? (uint32_t)((int64_t)row * p.lda + (int64_t)bt * p.a_bs + k) * 2u : DR_OOB;
+      avn[s] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(abuf, off, 0, 0));
+    }
+  }
   if constexpr (NK) {
     // acc[e][t] is row 4 g + t, column col0 + 16 e + n
 #pragma unroll
@@ -259,13 +280,13 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
 #pragma unroll
   for (int w = 1; w < DR_WAVES; ++w) tot += *reinterpret_cast<const f32x4*>(&red[(w * 16 + m) * 128 + c4]);
   const int col = col0 + c4;
-  if (p.scales && m < p.M && c4 < cw && col < N) {
+  if (p.scales && mrow0 + m < p.M && c4 < cw && col < N) {
     const f16* sc = p.scales + (int64_t)bt * N + col;
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       if (col + e < N) tot[e] *= (float)sc[e];
   }
-  if (p.ep && m < p.M && c4 < cw && col < N) {
+  if (p.ep && mrow0 + m < p.M && c4 < cw && col < N) {
     const T* bias = reinterpret_cast<const T*>(p.bias);
 #pragma unroll
     for (int e = 0; e < 4; ++e)
@@ -275,12 +296,12 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
         tot[e] = apply_act(v, p.act);
       }
   }
-  if (m < p.M && c4 < cw && col < N) {
-    T* o = reinterpret_cast<T*>(p.out) + (int64_t)m * p.o_ms + (int64_t)bt * p.o_bs;
+  if (mrow0 + m < p.M && c4 < cw && col < N) {
+    T* o = reinterpret_cast<T*>(p.out) + (int64_t)(mrow0 + m) * p.o_ms + (int64_t)bt * p.o_bs;
     int ocol = col;
     if (p.per > 0) {                                     // (per is a multiple of 4: the four columns stay together)
       const uint32_t l = fd_div((uint32_t)col, p.perdiv);
-      o = reinterpret_cast<T*>(p.out) + (int64_t)l * p.o_ls + (int64_t)m * p.o_ms + (int64_t)bt * p.per;
+      o = reinterpret_cast<T*>(p.out) + (int64_t)l * p.o_ls + (int64_t)(mrow0 + m) * p.o_ms + (int64_t)bt * p.per;
       ocol = col - (int)l * p.per;
     }
     if (p.o_ns == 1 && col + 3 < N && ((reinterpret_cast<uintptr_t>(o + ocol) & 7) == 0)) {
@@ -294,6 +315,14 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
         if (col + e < N) o[(int64_t)(ocol + e) * p.o_ns] = TypeTraits<T>::from_f32(tot[e]);
     }
   }
+  if (!more) break;
+  __syncthreads();                                       // red is free again
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) av[s] = avn[s];
+  products();
+  }  // tiles of 16 rows
   TR5(4);
 }
 
@@ -527,6 +556,8 @@ int rows_plan(RowsParams& p, int batch, int dtype, int wbits, bool nk) {
   if ((int64_t)p.K * p.N * 2 >= (int64_t)DR_OOB) return 1;
   if (wbits != 16 && dtype != BLR_F16 && dtype != BLR_BF16) return 1;
   p.rounds = (int)cdiv(p.K, DR_WAVES * DR_MAX_STEPS * 32);
+  p.mtiles = (int)cdiv(p.M, 16);
+  if (p.mtiles > 1 && p.rounds > 1) return 1;          // more rows than one tile only with the whole factor slice in registers
   p.kw = (int)cdiv(cdiv(p.K, DR_WAVES * p.rounds), 32) * 32;
   const int cus = device_cus() > 0 ? device_cus() : 256;
   static const int e_npc = env_i("BLR_DR_NPC", 0);
@@ -600,7 +631,7 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   const bool u_nk = a.u_layout == BLR_U_QR;
   const bool monarch = a.perm_per > 0;                  // the mix is a permutation, folded into the store of the first product
   const bool lowrank = !monarch && !a.S && bo == 1;     // one output block, S = 1: the mix is the sum over the input slices
-  if (M < 1 || M > 16 || (!monarch && !lowrank && !a.S) || (bo != b && !lowrank) || (u_nk && a.wbits != 16)) return 1;
+  if (M < 1 || M > DR_MAX_M || (!monarch && !lowrank && !a.S) || (bo != b && !lowrank) || (u_nk && a.wbits != 16)) return 1;
   if (lowrank && a.wbits != 16) return 1;
   if (monarch && (a.wbits != 16 || a.perm_per % 4 || R % a.perm_per || R / a.perm_per != b || a.perm_per >= 65536)) return 1;
   if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return 1;

@@ -1,0 +1,88 @@
+"""GPU parity at 17 to 128 token rows, where every operator runs the few-row kernels over tiles of 16 rows (weights held in
+registers, one more set of products and one more reduction per tile) instead of 256-row GEMM tiles.
+
+Tolerance: the bound of the other parity tests, max|y - y_ref| <= 1e-2 * max|y_ref| for fp16 (2e-2 for bf16) against the fp64
+oracle on the same rounded inputs; twice that where a second rounded intermediate is involved (low rank, Monarch).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import blr_oracle as O
+from gpu_util import assert_close, blast_inputs, dev, rounded, say
+
+pytestmark = pytest.mark.gpu
+
+ROWS = [17, 40, 64, 100, 128]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", ROWS)
+@pytest.mark.parametrize("name", ["triton_blast_full_fp16", "triton_blast_bmm_fp16"])
+def test_blast(name, M, dtype):
+    from test_gpu_blast import _ref, _run_blast
+    b, p, q, r = 16, 64, 72, 128
+    x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=M)
+    say(f"[case] mid rows {name} M={M} {dtype}")
+    out = _run_blast(name, x, U, Vt, S, dtype, "auto")
+    assert tuple(out.shape) == (M, b * q)
+    assert_close(out, _ref(x, U, Vt, S, dtype)[0], dtype, f"{name} M={M}")
+
+
+@pytest.mark.parametrize("layer", ["qkvo", "gate_up", "down"])
+def test_blast_llama7b_64_rows_with_bias_and_activation(layer):
+    from triton_funcs import blast_kernels as K, _lib as L
+    p, q, r = {"qkvo": (256, 256, 512), "gate_up": (256, 1376, 1024), "down": (688, 256, 1024)}[layer]
+    b, M, dtype = 16, 64, torch.float16
+    x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=3)
+    bias = np.random.default_rng(3).standard_normal(b * q)
+    Uk, Vk, Sk = O.blast_to_partial_layout(U, Vt, S)
+    say(f"[case] mid rows llama7b {layer} M={M} + bias + silu")
+    with L.fused_epilogue(dev(bias, dtype), "silu"):
+        out = K.triton_blast_full_fp16(dev(x, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype))
+    v = O.blast_forward(rounded(x, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0] + rounded(bias, dtype)
+    assert_close(out, v / (1.0 + np.exp(-v)), dtype, f"{layer} M=64")
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("M", [17, 100, 128])
+def test_blast_codes(M, bits):
+    from triton_funcs import blast_sym_quant_kernels as Q
+    b, p, q, r = 16, 32, 40, 96
+    dtype = torch.float16
+    rng = np.random.default_rng(30 + M)
+    x = rng.standard_normal((1, M, b * p))
+    U = (rng.standard_normal((b, q, r)) / np.sqrt(r)).astype(np.float32)
+    V = (rng.standard_normal((b, p, r)) / np.sqrt(r)).astype(np.float32)
+    S = rng.standard_normal((r, b, b))
+    say(f"[case] mid rows blast_q bits={bits} M={M}")
+    Uq, Vq = Q.quantize_blast_factors(torch.from_numpy(U).cuda(), torch.from_numpy(V).cuda(), bits)
+    uc, us = O.quantize_sym(U, 2, bits); vc, vs = O.quantize_sym(V, 1, bits)
+    fn = Q.triton_blast_bmm_int8_fp16 if bits == 8 else Q.triton_blast_bmm_int4_fp16
+    out = fn(dev(x, dtype), Uq, Vq, dev(S, dtype))
+    assert_close(out, O.blast_q_forward(rounded(x, dtype), uc, us, vc, vs, rounded(S, dtype)), dtype, f"blast_q bits={bits} M={M}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [17, 100])
+def test_low_rank(M, dtype):
+    from triton_funcs import low_rank_kernels as K
+    rng = np.random.default_rng(50 + M)
+    in_f, r, out_f = 512, 64, 200
+    x = rng.standard_normal((M, in_f)); a = rng.standard_normal((in_f, r)) / np.sqrt(in_f); bm = rng.standard_normal((r, out_f)) / np.sqrt(r)
+    say(f"[case] mid rows low rank M={M} {dtype}")
+    out = K.triton_low_rank_fp16(dev(x, dtype), dev(a, dtype), dev(bm, dtype))
+    assert_close(out, (rounded(x, dtype) @ rounded(a, dtype)) @ rounded(bm, dtype), dtype, f"low rank M={M}", scale=2.0)
+
+
+@pytest.mark.parametrize("shape", [(4, 64, 64, 40), (4, 1104, 256, 40)], ids=["shallow", "deep-blocks"])
+@pytest.mark.parametrize("M", [17, 100])
+@pytest.mark.parametrize("name", ["triton_monarch_right_fp16", "triton_monarch_right_left_fp16"])
+def test_monarch(name, M, shape):
+    from test_gpu_monarch_lowrank_dense import _ref_monarch, _run_monarch, monarch_inputs
+    b, p, rank, s = shape
+    dtype = torch.float16
+    x, w1_t, w2_t = monarch_inputs(b, p, rank, s, (M,), seed=60 + M)
+    say(f"[case] mid rows {name} M={M} b={b} p={p} rank={rank} s={s}")
+    out = _run_monarch(name, x, w1_t, w2_t, dtype)
+    assert_close(out, _ref_monarch(x, w1_t, w2_t, dtype)[0], dtype, f"{name} M={M}", scale=2.0)
