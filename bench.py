@@ -11,7 +11,7 @@ graph, rotating through enough weight copies that the 256 MB Infinity Cache cann
 The one JSON line printed last carries `value` = microseconds per layer-step (lower is better),
 `roofline` for the dominant kernel (the gate_up streaming kernel), `cpu_baseline` (the CPU oracle's
 torch port of the same step on the host cores), and `layers`: per-layer microseconds with the
-fraction of HBM (M <= 16) or fp16-MFMA (M = 2048) peak for BLAST, quantized BLAST, Monarch,
+fraction of HBM (M = 1, 16, 64) or fp16-MFMA (M = 2048) peak for BLAST, quantized BLAST, Monarch,
 low-rank and dense.
 """
 from __future__ import annotations
@@ -308,9 +308,9 @@ def main():
             hbm = by / (us * 1e-6) / HBM_PEAK
             mf = fl / (us * 1e-6) / MFMA_PEAK
             table[name] = {"us": round(us, 2), "pct_hbm": round(100 * hbm, 1), "pct_mfma": round(100 * mf, 1),
-                           "bound": "hbm" if m <= 16 else "mfma"}
+                           "bound": "hbm" if m <= 128 else "mfma"}
         for lname, (i_f, o_f, r) in LAYERS.items():
-            for m in (1, 16, 2048):
+            for m in (1, 16, 64, 2048):
                 by, fl = blast_bytes_flops(m, i_f, r, o_f)
                 wbytes = 2 * r * (i_f + o_f + B * B)
                 row(f"blast_full/{lname}/M{m}", measure(lambda: mk_blast(m, i_f, o_f, r, L.U_RQ, L.S_JIR), wbytes), by, fl, m)
@@ -323,7 +323,7 @@ def main():
         for lname in ("gate_up", "down"):
             i_f, o_f, r = LAYERS[lname]
             for bits in (8, 4):
-                for m in (1, 4, 16):
+                for m in (1, 4, 16, 64):
                     by = r * (i_f + o_f) * bits // 8 + 2 * B * B * r + 2 * (o_f + B * r) + 2 * m * (i_f + o_f)
                     fl = 2 * m * r * (i_f + o_f + B * B)
                     row(f"blast_int{bits}/{lname}/M{m}", measure(lambda: mk_blast_q(m, i_f, o_f, r, bits), by), by, fl, m)

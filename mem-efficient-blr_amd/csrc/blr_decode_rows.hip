@@ -146,7 +146,8 @@ template <typename T> struct RowsPiece<T, 4> {
 // NK: the factor is stored transposed, W[bt][n][k] with k contiguous (U of the bmm names, (b, q, r)).  A 16-byte load then is
 // a lane's matrix-core operand as it stands: the lane of slot n and k-group g loads k .. k + 7 of column 16 cg + n for each of
 // the chunk's column groups cg (p.npc of them, 16 columns each).
-template <typename T, int STEPS, int WB, bool NK>
+// MULTI: more than one tile of 16 token rows (a separate instantiation: the single-tile kernel carries none of the loop).
+template <typename T, int STEPS, int WB, bool NK, bool MULTI>
 __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   using Piece = RowsPiece<T, WB>;
   static_assert(!NK || WB == 16, "codes are stored (k, n)");
@@ -247,9 +248,9 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
   // fetched (asked for before the reduction of the tile before, so that they arrive under it), multiplied and reduced.
   for (int mt = 0;; ++mt) {
   const int mrow0 = mt * 16;
-  const bool more = mt + 1 < p.mtiles;
+  const bool more = MULTI && mt + 1 < p.mtiles;
   u32x4 avn[STEPS];
-  if (more) {
+  if (MULTI && more) {
     const int row = mrow0 + 16 + n, kb = wv * p.kw + 8 * g;
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
@@ -315,13 +316,14 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
         if (col + e < N) o[(int64_t)(ocol + e) * p.o_ns] = TypeTraits<T>::from_f32(tot[e]);
     }
   }
-  if (!more) break;
+  if (!MULTI || !more) break;
   __syncthreads();                                       // red is free again
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) av[s] = avn[s];
-  products();
+  products();                                            // (what does not depend on the tile - widening of codes, byte permutes - is
+                                                         // moved in front of the loop by the compiler and done once)
   }  // tiles of 16 rows
   TR5(4);
 }
@@ -534,18 +536,22 @@ int plan_pieces(int batch, int K, int N, int wbits, int cus) {
   return best;
 }
 
-template <typename T, int WB, bool NK = false>
-int rows_launch_t(RowsParams& p, int batch, hipStream_t st) {
+template <typename T, int WB, bool NK, bool MULTI>
+int rows_launch_m(RowsParams& p, int batch, hipStream_t st) {
   const int steps = p.kw / 32;
   const dim3 grid((unsigned)(batch * p.nch.d)), block(DR_NT);
   switch (steps) {
-    case 1: hipLaunchKernelGGL((rows_product_kernel<T, 1, WB, NK>), grid, block, 0, st, p); break;
-    case 2: hipLaunchKernelGGL((rows_product_kernel<T, 2, WB, NK>), grid, block, 0, st, p); break;
-    case 3: hipLaunchKernelGGL((rows_product_kernel<T, 3, WB, NK>), grid, block, 0, st, p); break;
-    default: hipLaunchKernelGGL((rows_product_kernel<T, 4, WB, NK>), grid, block, 0, st, p); break;
+    case 1: hipLaunchKernelGGL((rows_product_kernel<T, 1, WB, NK, MULTI>), grid, block, 0, st, p); break;
+    case 2: hipLaunchKernelGGL((rows_product_kernel<T, 2, WB, NK, MULTI>), grid, block, 0, st, p); break;
+    case 3: hipLaunchKernelGGL((rows_product_kernel<T, 3, WB, NK, MULTI>), grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL((rows_product_kernel<T, 4, WB, NK, MULTI>), grid, block, 0, st, p); break;
   }
   BLR_CHECK_LAUNCH("rows_product");
   return BLR_OK;
+}
+template <typename T, int WB, bool NK = false>
+int rows_launch_t(RowsParams& p, int batch, hipStream_t st) {
+  return p.mtiles > 1 ? rows_launch_m<T, WB, NK, true>(p, batch, st) : rows_launch_m<T, WB, NK, false>(p, batch, st);
 }
 
 // Plans one batch of skinny products (chunk width, rounds, item order); returns 1 when the operands do not fit the kernel.
