@@ -676,7 +676,7 @@ size_t blr_dense_workspace_bytes(int M, int in_f, int out_f, int dtype, int algo
   if (M <= 0) return 0;
   int a = resolve_algo(algo, M, dtype, false);
   if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) return stream_generic_workspace(0, M, in_f, out_f, 1, 0);
-  return 0;
+  return dense_rows_bytes(M, in_f, out_f, dtype);            // 17..128 rows: partial products of the slices of the reduction
 }
 
 int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
@@ -697,6 +697,12 @@ int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t 
     return stream_generic_launch(s, st);
   }
   if (a != BLR_ALGO_TILED) { set_error("dense: algorithm %d not available", a); return BLR_ERR_UNSUPPORTED; }
+  {
+    // 17..128 rows: 256-row tiles would leave most compute units idle and give the others a long stream each (11008 -> 4096
+    // at 64 rows: 124 us); the few-row product kernel over tiles of 16 rows instead
+    const int rc = dense_rows_launch(x, ldx, W, out, ldo, M, in_f, out_f, dtype, ws, ws_bytes, st);
+    if (rc != 1) return rc;
+  }
   GemmArgs g = {};
   g.A = x; g.lda = ldx; g.B = W; g.ldb = out_f; g.b_kn = 1;
   g.C = out; g.ldc = ldo; g.cn = 1; g.M = M; g.N = out_f; g.K = in_f; g.batch = 1;

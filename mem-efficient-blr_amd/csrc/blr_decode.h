@@ -23,8 +23,17 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
 int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_bytes, hipStream_t st);
 
 // The same call as three launches - y = x V and out = z U on the matrix cores with the rank-space mix between them
-// (blr_decode_rows.hip; up to 16 token rows, U (b, r, q), two-byte weights).  region: scratch for y and z as T.  Same return convention.
+// (blr_decode_rows.hip; up to 128 token rows in tiles of 16, two-byte weights or codes).  region: scratch for y and z as T.  Same
+// return convention.
 int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_bytes, hipStream_t st);
+
+// Dense layer out = x W (W (in_f, out_f) row-major) at 17..128 token rows with the same product kernel: the reduction is cut
+// into equal slices of at most 1024 rows of W (so that the weights of a chunk stay in registers over the tiles of 16 token
+// rows), every slice leaves its partial product as T in `ws`, and one more launch adds the slices in fp32.  dense_rows_bytes:
+// bytes of the partial products, 0 when the shape is not for this path; the launch returns 1 then.
+size_t dense_rows_bytes(int M, int in_f, int out_f, int dtype);
+int dense_rows_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int in_f, int out_f, int dtype,
+                      void* ws, size_t ws_bytes, hipStream_t st);
 
 // Dense layer out = x W (W (K, N)) at up to 16 rows: slabs of W on the matrix cores, fp32 partial sums of the k-slices in `part`
 // (room for max_slices * M * N floats) added by a second launch.  Returns BLR_OK, a negative blr_status, or 1 when the

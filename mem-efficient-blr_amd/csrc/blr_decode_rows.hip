@@ -716,6 +716,55 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   return rc == 1 ? BLR_ERR_UNSUPPORTED : rc;
 }
 
+// ---- dense at 17..128 rows ----------------------------------------------------------------------------------------------
+namespace {
+int dense_slices(int in_f) {
+  for (int c = 1; c <= 16; ++c)
+    if (in_f % c == 0 && (in_f / c) % 8 == 0 && in_f / c <= 1024) return c;
+  return 0;
+}
+}  // namespace
+
+// Measured against the 256-row tiles (us at 17 / 64 / 128 rows): 4096 -> 4096 13 / 17 / 23 against 47 / 49 / 56, 11008 -> 4096
+// 26 / 33 / 44 against 116 / 124 / 144, 4096 -> 22016 46 / 58 / 77 against 54 / 56 / 63 - a wide output has enough tiles of its own
+// and pays for the slices' partial products, so it comes here only up to 48 rows.
+static bool dense_rows_wanted(int M, int out_f) { return M > 16 && M <= DR_MAX_M && (out_f <= 8192 || M <= 48); }
+
+size_t dense_rows_bytes(int M, int in_f, int out_f, int dtype) {
+  const int bi = dense_slices(in_f);
+  if (!dense_rows_wanted(M, out_f) || (dtype != BLR_F16 && dtype != BLR_BF16) || !bi || out_f % 8) return 0;
+  return bi > 1 ? align_up((size_t)bi * M * out_f * 2, 256) : 0;
+}
+
+int dense_rows_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int in_f, int out_f, int dtype,
+                      void* ws, size_t ws_bytes, hipStream_t st) {
+  static const int enabled = env_i("BLR_DENSE_ROWS", 1);
+  const int bi = dense_slices(in_f);
+  if (!enabled || !dense_rows_wanted(M, out_f) || (dtype != BLR_F16 && dtype != BLR_BF16) || !bi || out_f % 8) return 1;
+  if (bi > 1 && (ldo != out_f || !ws || ws_bytes < dense_rows_bytes(M, in_f, out_f, dtype) || !aligned(out, 8))) return 1;
+  const int64_t x_elems = (int64_t)(M - 1) * ldx + in_f;
+  if (x_elems * 2 >= (int64_t)DR_OOB || ldx % 8 || !aligned(x, 16) || !aligned(W, 16)) return 1;
+  RowsParams s = {};
+  s.A = x; s.lda = ldx; s.a_bs = in_f / bi; s.a_bytes = (uint32_t)(x_elems * 2);
+  s.W = W; s.w_bs = (int64_t)(in_f / bi) * out_f;
+  s.out = bi > 1 ? ws : out; s.o_ms = bi > 1 ? out_f : ldo; s.o_bs = (int64_t)M * out_f; s.o_ns = 1;
+  s.M = M; s.K = in_f / bi; s.N = out_f;
+  const void* ep_bias = nullptr; int ep_act = 0;
+  if (bi == 1 && epilogue_pending(&ep_bias, &ep_act)) { s.ep = 1; s.bias = ep_bias; s.act = ep_act; }
+  int rc = rows_plan(s, bi, dtype, 16, false);
+  if (rc) return rc;
+  rc = rows_launch(s, bi, dtype, 16, false, st);
+  if (rc) return rc == 1 ? BLR_ERR_UNSUPPORTED : rc;
+  if (bi == 1) { if (s.ep) epilogue_taken(); return BLR_OK; }
+  const int64_t mn4 = (int64_t)M * out_f / 4;
+  const uint32_t nsum = (uint32_t)cdiv(mn4, 256);
+  const RowsPrefetch none = {};
+  if (dtype == BLR_F16) hipLaunchKernelGGL(rows_sum_kernel<f16>, dim3(nsum), dim3(256), 0, st, (const f16*)ws, (f16*)out, bi, mn4, none, nsum);
+  else hipLaunchKernelGGL(rows_sum_kernel<bf16>, dim3(nsum), dim3(256), 0, st, (const bf16*)ws, (bf16*)out, bi, mn4, none, nsum);
+  BLR_CHECK_LAUNCH("rows_sum");
+  return BLR_OK;
+}
+
 }  // namespace blr
 
 #ifdef BLR_TRACE

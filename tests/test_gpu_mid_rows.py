@@ -86,3 +86,24 @@ def test_monarch(name, M, shape):
     say(f"[case] mid rows {name} M={M} b={b} p={p} rank={rank} s={s}")
     out = _run_monarch(name, x, w1_t, w2_t, dtype)
     assert_close(out, _ref_monarch(x, w1_t, w2_t, dtype)[0], dtype, f"{name} M={M}", scale=2.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [17, 64, 128])
+@pytest.mark.parametrize("shape", [(512, 200), (4096, 1024), (2752, 264)], ids=lambda s: "in%d-out%d" % s)
+def test_dense(shape, M, dtype):
+    """One slice (in_f <= 1024), four slices of 1024 and four of 688: the slices' partial products are rounded to the 16-bit
+    type before they are added, hence twice the tolerance."""
+    from triton_funcs import dense_kernels as D, _lib as L
+    in_f, out_f = shape
+    rng = np.random.default_rng(70 + M)
+    x = rng.standard_normal((M, in_f)); w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)
+    say(f"[case] mid rows dense M={M} in={in_f} out={out_f} {dtype}")
+    out = D.triton_dense_fp16(dev(x, dtype), dev(w, dtype))
+    ref = rounded(x, dtype) @ rounded(w, dtype)
+    assert_close(out, ref, dtype, f"dense M={M}", scale=2.0)
+    bias = rng.standard_normal(out_f)
+    with L.fused_epilogue(dev(bias, dtype), "gelu_tanh"):
+        out = D.triton_dense_fp16(dev(x, dtype), dev(w, dtype))
+    v = ref + rounded(bias, dtype)
+    assert_close(out, 0.5 * v * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (v + 0.044715 * v ** 3))), dtype, f"dense M={M} + bias + gelu", scale=2.0)
