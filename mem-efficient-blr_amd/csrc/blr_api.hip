@@ -676,7 +676,9 @@ size_t blr_dense_workspace_bytes(int M, int in_f, int out_f, int dtype, int algo
   if (M <= 0) return 0;
   int a = resolve_algo(algo, M, dtype, false);
   if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) return stream_generic_workspace(0, M, in_f, out_f, 1, 0);
-  return dense_rows_bytes(M, in_f, out_f, dtype);            // 17..128 rows: partial products of the slices of the reduction
+  const size_t rows = dense_rows_bytes(M, in_f, out_f, dtype);      // 17..128 rows: partial products of the slices of the reduction
+  const size_t splitk = gemm_splitk_bytes(M, out_f, in_f, dtype);    // more rows, few tiles: fp32 partial sums of the slices of K
+  return rows > splitk ? rows : splitk;
 }
 
 int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
@@ -706,6 +708,8 @@ int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t 
   GemmArgs g = {};
   g.A = x; g.lda = ldx; g.B = W; g.ldb = out_f; g.b_kn = 1;
   g.C = out; g.ldc = ldo; g.cn = 1; g.M = M; g.N = out_f; g.K = in_f; g.batch = 1;
+  // few output tiles and a long reduction (11008 -> 4096 at 256 rows: 32 tiles): room to cut it along K
+  if (ws && gemm_splitk_bytes(M, out_f, in_f, dtype) && ws_bytes >= gemm_splitk_bytes(M, out_f, in_f, dtype)) { g.splitk_ws = ws; g.splitk_bytes = ws_bytes; }
   attach_epilogue(g);
   return gemm_launch(g, dtype, st);
 }
