@@ -18,6 +18,7 @@
 //            Z per (i, m).  Z leaves as T.
 // What follows is an ordinary batched GEMM out_i = Z_i U_i.
 #include <hip/hip_runtime.h>
+#include <cmath>
 #include "blr_common.h"
 #include "blr_decode_dev.h"
 
@@ -257,8 +258,20 @@ int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, 
   YmixParams p = {};
   p.x = x; p.ldx = ldx; p.x_bytes = (uint32_t)(x_elems * 2); p.V = V; p.S = S; p.Z = Z;
   p.M = M; p.b = b; p.P = P; p.R = R;
-  const int pieces = R / 8, tiles = (int)cdiv(pieces, 16);
-  p.npc = (int)cdiv(pieces, tiles);
+  // Rank pieces per tile.  One workgroup per compute unit at a time; a workgroup takes about 10 + 0.85 npc us at 72-column input
+  // blocks, i.e. 12 + npc units, and a last round that is not full costs about half of what it leaves empty.  Measured at 4096
+  // rows, r = 576: 15 pieces = 640 workgroups (2.5 rounds) 68 us, 12 = 768 (3 rounds) 60 us, 9 = 1024 (4 rounds) 72 us; r = 288:
+  // 12 pieces = 384 (1.5 rounds) 34.8 us, 9 = 512 (2 rounds) 36.2 us.
+  const int pieces = R / 8;
+  const int cus = device_cus() > 0 ? device_cus() : 256;
+  static const int e_npc = env_i("BLR_YM_NPC", 0);
+  int best_npc = 16; double best_cost = -1.0;
+  for (int npc = 16; npc >= 4; --npc) {
+    const double x = (double)(cdiv(pieces, npc) * cdiv(M, YM_BM)) / cus;
+    const double cost = 0.5 * (std::ceil(x) + x) * (12 + npc);
+    if (best_cost < 0 || cost < best_cost - 1e-9) { best_cost = cost; best_npc = npc; }
+  }
+  p.npc = e_npc > 0 && e_npc <= 16 ? e_npc : best_npc;
   const int nrt = (int)cdiv(pieces, p.npc), nmt = (int)cdiv(M, YM_BM);
   if ((int64_t)nrt * nmt >= 65536 || nmt >= 65536) return 1;
   p.nmt = fd_make((uint32_t)nmt);
