@@ -87,20 +87,23 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
   const uint32_t rt = fd_div(item, p.nmt), mt = item - rt * p.nmt.d;
   const int m0 = (int)mt * YM_BM, r0 = (int)rt * BR;
   TR6(0);
-  // the mix's S operands depend on nothing: asked for first, used after phase 1.  Lane (n, g) of wave wv: S_r(i = n,
-  // j = 4 g .. 4 g + 3) for the wave's 16 ranks r0 + 16 wv ..
+  // the mix's S operands depend on nothing and are used after phase 1: asked for behind the first loads of phase 1 (the
+  // memory pipeline takes an instruction every 16 cycles, and the products can only start on those first loads).  Lane (n, g)
+  // of wave wv: S_r(i = n, j = 4 g .. 4 g + 3) for the wave's 16 ranks r0 + 16 wv ..; waves without ranks in the tile ask nothing
   const __amdgpu_buffer_rsrc_t sbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.St), 0, (uint32_t)((int64_t)b * b * R * 2), 0x00020000);
   const int rw = wv * 16;
   u32x2 sa[16];
-  {
+  auto load_sa = [&]() {
     const bool a_ok = n < b && 4 * g < b;
+    if (rw < BR) {
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      const int r = r0 + rw + q;
-      const uint32_t off = (a_ok && rw + q < BR && r < R) ? (uint32_t)(((int64_t)r * b + n) * b + 4 * g) * 2u : YM_OOB;
-      sa[q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(sbuf, off, 0, 0));
+      for (int q = 0; q < 16; ++q) {
+        const int r = r0 + rw + q;
+        const uint32_t off = (a_ok && rw + q < BR && r < R) ? (uint32_t)(((int64_t)r * b + n) * b + 4 * g) * 2u : YM_OOB;
+        sa[q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(sbuf, off, 0, 0));
+      }
     }
-  }
+  };
 
   // ---------------------------------------------- phase 1: Y pairs into LDS ----------------------------------------------
   // One pipeline over the k-steps of the wave's two input blocks (no drain between them): step q < KS belongs to block
@@ -159,6 +162,7 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
         for (int e = 0; e < 8; ++e) acc[mg][e] = f32x4{0.f, 0.f, 0.f, 0.f};
     };
     load_ab(a0, b0, 0);
+    load_sa();
     TR6(1);
     for (int q = 0; q < 2 * KS; q += 2) {                    // two steps per trip (the two register sets take turns)
       if (q == KS) next_block();
@@ -187,6 +191,8 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
           *reinterpret_cast<u32x4*>(dst + 4) = u32x4{pr[4], pr[5], pr[6], pr[7]};
         }
     }
+  } else {
+    load_sa();
   }
   TR6(3);
   __syncthreads();
