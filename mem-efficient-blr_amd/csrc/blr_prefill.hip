@@ -164,7 +164,8 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
     load_ab(a0, b0, 0);
     load_sa();
     TR6(1);
-    for (int q = 0; q < 2 * KS; q += 2) {                    // two steps per trip (the two register sets take turns)
+    int q = 0;
+    for (; q + 2 < 2 * KS; q += 2) {                         // two steps per trip (the two register sets take turns)
       if (q == KS) next_block();
       load_ab(a1, b1, q + 1);
       step(a0, b0);
@@ -172,6 +173,13 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
       load_ab(a0, b0, q + 2);
       step(a1, b1);
     }
+    // the last trip on its own: nothing is left to ask for behind it (ten loads that would all be out of bounds still cost
+    // their turns in the memory pipeline)
+    if (q == KS) next_block();
+    load_ab(a1, b1, q + 1);
+    step(a0, b0);
+    if (q + 1 == KS) next_block();
+    step(a1, b1);
     TR6(2);
     // acc[mg][e][t] is Y of block 2 wv + 1 at [m0 + 16 mg + 4 g + t][r0 + 8 n + e]; h0 holds block 2 wv
     if (n < p.npc) {
