@@ -357,7 +357,15 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   // block on that costs more than the round trip of Y it saves (measured at 4096 rows: 1152 -> 1152, r = 288: 64 against
   // 68 us; 4608 -> 1152, r = 576: 154 against 122 us; Llama-7B gate_up at 2048 rows: 201 against 186 us).
   static const int fuse_max_p = getenv("BLR_BLAST_FUSE_MAX_P") ? atoi(getenv("BLR_BLAST_FUSE_MAX_P")) : 128;
-  if (!y_out && !sat8 && fused >= 0 && (fused == 1 || P <= fuse_max_p))
+  // Narrow output blocks with the rank contiguous in U: the mix and the product with U run as one launch that reads Y once and
+  // never writes Z (blast_mixu_kernel); the first half is then the plain GEMM, which leaves Y.  Measured at 4096 rows against the
+  // mix kernel + batched GEMM: 4608 -> 1152, r = 576: 90 against 122 us; against the fused first half + batched GEMM: 1152 -> 1152,
+  // r = 288: 47 against 51 us.  BLR_BLAST_MIXU: 0 never, 1 only where the first half would not be fused anyway, 2 (default)
+  // wherever the kernel takes the shape.
+  static const int mixu_mode = getenv("BLR_BLAST_MIXU") ? atoi(getenv("BLR_BLAST_MIXU")) : 2;
+  const bool mixu_shape = !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && b == 16 && u_layout == BLR_U_QR && Q % 8 == 0 && Q <= 80 && r % 32 == 0;
+  const bool mixu = mixu_shape && (mixu_mode >= 2 || (mixu_mode == 1 && (P > fuse_max_p || fused < 0)));
+  if (!mixu && !y_out && !sat8 && fused >= 0 && (fused == 1 || P <= fuse_max_p))
     rc = blast_ymix_launch(x, ldx, V, S, Z, M, in_f, b, r, si, sj, sr, s_layout, dtype, Y, ybytes, st);   // (the unused room of Y holds S transposed)
   if (rc < 0) return rc;
   if (rc == 1 && fused == 1) { set_error("blast: the fused kernel does not take this shape (b even and <= 16, block width and rank multiples of 8, f16/bf16)"); return BLR_ERR_UNSUPPORTED; }
@@ -370,8 +378,10 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
     g1.sat8 = sat8;
     rc = gemm_launch(g1, dtype, st);
     if (rc) return rc;
-    rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st, sat8);
-    if (rc) return rc;
+    if (!mixu) {
+      rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st, sat8);
+      if (rc) return rc;
+    }
   }
 
   GemmArgs g2 = {};
@@ -382,6 +392,12 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   g2.C = out; g2.ldc = ldo; g2.sC = Q; g2.cn = 1;
   g2.M = M; g2.N = Q; g2.K = r; g2.batch = b;
   if (!sat8) attach_epilogue(g2);
+  if (mixu) {                                       // (Y is in memory: the branch above ran the GEMM and skipped the mix)
+    rc = blast_mixu_launch(Y, S, U, out, ldo, g2, M, b, r, Q, si, sj, sr, s_layout, dtype, Z, ybytes, st);
+    if (rc != 1) return rc;
+    rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st, sat8);
+    if (rc) return rc;
+  }
   return gemm_launch(g2, dtype, st);
 }
 

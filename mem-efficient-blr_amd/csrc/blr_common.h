@@ -139,6 +139,11 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
 int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, void* Z, int M, int in_f, int b, int R,
                       int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
                       hipStream_t st);
+// Second half for output blocks of at most 80 columns: out_i = mix(S, Y)_i U_i with U (b, Q, R), in one launch and without Z;
+// the fused output stage (bias, act, gate, resid) is taken from `ep`.  Same return convention; scratch as above.
+int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
+                      int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
+                      hipStream_t st);
 
 // ---- streaming (decode) engine (blr_stream.hip) -------------------------------------------
 struct StreamBlastArgs {

@@ -19,6 +19,7 @@
 // What follows is an ordinary batched GEMM out_i = Z_i U_i.
 #include <hip/hip_runtime.h>
 #include <cmath>
+#include <type_traits>
 #include "blr_common.h"
 #include "blr_decode_dev.h"
 
@@ -313,6 +314,290 @@ int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, 
   if (dtype == BLR_F16) hipLaunchKernelGGL(blast_ymix_kernel<f16>, grid, block, lds, st, p);
   else hipLaunchKernelGGL(blast_ymix_kernel<bf16>, grid, block, lds, st, p);
   BLR_CHECK_LAUNCH("blast_ymix");
+  return BLR_OK;
+}
+
+
+// ---- second half for narrow output blocks: out_i = mix(S, Y)_i U_i in one launch, Z never written -------------------------
+//
+// When an output block is at most 80 columns wide, the results of ALL output blocks for a tile of 16 rows fit the registers of one
+// workgroup (16 blocks x 16 rows x 80 columns of fp32 = 80 KB).  The workgroup then walks the rank in blocks of 64: it reads the
+// block of Y for all input blocks once (the only pass over the intermediate), forms the block of every Z_i on the matrix cores
+// (one 16 x 16 x 16 product per rank, as in the kernel above), hands it through LDS as T and multiplies it with the block of U_i.
+// U (b, Q, R) has the rank contiguous, so 16 bytes of it are an operand as they stand - but the lanes of a matrix-core operand
+// are its rows, and a load whose neighbouring lanes read different rows of U occupies the compute unit's memory pipeline for 64
+// cycles instead of 16 (measured: 3 us per step with such loads, 0.5 us without any).  A small kernel therefore first re-lays U
+// (1.3 MB at 4608 -> 1152, rank 576) and S in the order the lanes read them: U as (i, rank / 8, q, 8) - neighbouring lanes, i.e.
+// neighbouring columns q, then read neighbouring 16-byte pieces - and S as (r / 2, j / 4, i, r % 2, 4), 16 bytes per lane and pair of ranks.
+// A block of 64 ranks is two matrix-core steps of 32; step s takes the ranks 16 g + 8 s + e (g = 0..3 the lane group, e = 0..7 the
+// element of the lane's 16 bytes).
+//   wave w: four of the 32 load instructions that bring a block of Y (8 rows of 128 bytes each) into LDS; the mix of slots
+//   4 w .. 4 w + 3 of a step (ranks 16 (w / 2) + 8 s + 4 (w % 2) + 0..3 of the block); output blocks 2 w, 2 w + 1.
+// S and U of step c + 2 are asked for right after step c has used its registers, Y of the next block at the start of a block.
+namespace {
+constexpr int MU_NT = 512;
+constexpr int MU_BM = 16;
+constexpr int MU_RB = 64;       // ranks per block
+constexpr int MU_LDY = 72;      // two-byte elements per LDS row of Y (64 ranks): 144 bytes keep 16-byte accesses aligned and rows apart
+constexpr int MU_LDZ = 40;      // per LDS row of Z (the 32 slots of a step)
+__device__ __forceinline__ void mu_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+}  // namespace
+
+struct MixuParams {
+  const void* Y; const void* Sp; const void* Ut; void* out; int64_t ldo;     // Sp (r / 2, j / 4, i, r % 2, 4), Ut (i, rank / 8, q, 8)
+  int M, R, Q;
+  uint32_t y_bytes;
+  const void* bias; int act;
+  const void* gate; int gate_rows; int64_t ld_gate;
+  const void* resid; int64_t ld_resid;
+};
+
+template <typename T, int NTQ>
+__global__ __launch_bounds__(MU_NT) void blast_mixu_kernel(MixuParams p) {
+  __shared__ __attribute__((aligned(16))) uint16_t mu_lds[256 * MU_LDY + 2 * 256 * MU_LDZ];
+  uint16_t* const y_s = mu_lds;                              // [input block j][row m][rank of the block]
+  uint16_t (*const z_s)[256 * MU_LDZ] = reinterpret_cast<uint16_t (*)[256 * MU_LDZ]>(mu_lds + 256 * MU_LDY);   // per step: [output block i][row m][slot]
+  const int tid = threadIdx.x, wv = tid >> 6, l = tid & 63, n = l & 15, g = l >> 4;
+  const int M = p.M, R = p.R, Q = p.Q;
+  const int m0 = (int)blockIdx.x * MU_BM;
+  const int NB = (R + MU_RB - 1) / MU_RB;             // the last block may hold 32 ranks: what lies past them is not asked for
+  const bool half_u = (R % MU_RB) != 0 && g >= 2, half_y = (R % MU_RB) != 0 && (l & 7) >= 4;
+  TR6(0);
+  const __amdgpu_buffer_rsrc_t ybuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.Y), 0, p.y_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t sbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.Sp), 0, (uint32_t)(256 * R * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t ubuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.Ut), 0, (uint32_t)((int64_t)16 * Q * R * 2), 0x00020000);
+  // Y: eight lanes fetch the 128 bytes of one (j, m); a load instruction covers eight rows m of one input block; the wave's four
+  // loads are rows 0..7 and 8..15 of the input blocks 2 wv and 2 wv + 1.  Per-lane offsets are few (registers are short):
+  // whatever is the same for all lanes goes into the scalar offset of the load.
+  const int piece = l & 7, yrow = l >> 3;
+  uint32_t yoff[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    yoff[h] = m0 + 8 * h + yrow < M ? (uint32_t)(((int64_t)(2 * wv) * M + m0 + 8 * h + yrow) * R + piece * 8) * 2u : YM_OOB;
+  const uint32_t yjs = (uint32_t)((int64_t)M * R * 2);           // from one input block to the next
+  const int ypos = ((2 * wv) * 16 + yrow) * MU_LDY + piece * 8;
+  // S_r(i = n, j = 4 g .. 4 g + 3) of the wave's four ranks of a step
+  const int rk = 16 * (wv >> 1) + 4 * (wv & 1);                  // + 8 s + 64 k
+  const uint32_t soff = (uint32_t)((rk >> 1) * 64 + l) * 16u;      // Sp: 16 bytes per lane and pair of ranks
+  // U_i(q = 16 nt + n, ranks 16 g + 8 s .. + 7 of the block), i = 2 wv + ii: piece (i, 8 k + 2 g + s, q) of Ut
+  const uint32_t uoff = (uint32_t)(((int64_t)(2 * wv) * (R / 8) + 2 * g) * Q + n) * 16u;
+  const uint32_t uoff_last = 16 * (NTQ - 1) + n < Q ? uoff : YM_OOB;      // the last column tile of a block may be partly empty
+  const uint32_t uis = (uint32_t)((R / 8) * Q) * 16u;            // from one output block to the next
+  struct Regs { u32x4 s[2]; u32x4 u[2][NTQ]; };
+  auto load_y = [&](u32x4 (&yr)[4], int k) {
+    const bool cut = half_y && k == NB - 1;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      yr[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ybuf, cut ? YM_OOB : yoff[u & 1], (uint32_t)k * (MU_RB * 2u) + (uint32_t)(u >> 1) * yjs, 0));
+  };
+  auto store_y = [&](const u32x4 (&yr)[4]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x4*>(&y_s[ypos + ((u >> 1) * 16 + (u & 1) * 8) * MU_LDY]) = yr[u];
+  };
+  auto load_s = [&](Regs& r, int k, int s) {                 // rank 64 k + 8 s + rk + q
+#pragma unroll
+    for (int q = 0; q < 2; ++q) r.s[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(sbuf, soff + (uint32_t)q * 1024u, (uint32_t)(k * MU_RB + 8 * s) * 512u, 0));
+  };
+  auto load_u = [&](Regs& r, int k, int s) {
+    const bool cut = half_u && k == NB - 1;
+    const uint32_t v0 = cut ? YM_OOB : uoff, vl = cut ? YM_OOB : uoff_last;
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+      for (int nt = 0; nt < NTQ; ++nt)
+        r.u[ii][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ubuf, (nt == NTQ - 1 ? vl : v0) + (uint32_t)nt * 256u,
+                                                                                        (uint32_t)((8 * k + s) * Q) * 16u + (uint32_t)ii * uis, 0));
+  };
+  f32x4 acc[2][NTQ];
+#pragma unroll
+  for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+    for (int nt = 0; nt < NTQ; ++nt) acc[ii][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // step s of block k on the register set `cur`.  No load sits under a condition (the compiler would then wait for everything in
+  // flight where the paths meet): the last blocks ask again for the last block, which costs their turns in the memory pipeline
+  // and nothing else.
+  auto step = [&](int k, auto SS, Regs& cur) {
+    constexpr int s = decltype(SS)::value;
+    const int kn = min(k + 1, NB - 1);
+    // the mix of this wave's four ranks: operand B = Y_r(j = 4 g .. 4 g + 3, m = n), gathered from the four rows of its lane
+    u32x2 yv[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) yv[t] = *reinterpret_cast<const u32x2*>(&y_s[((4 * g + t) * 16 + n) * MU_LDY + rk + 8 * s]);
+    f32x4 d[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+      const u32x2 yb = {__builtin_amdgcn_perm(yv[1][q >> 1], yv[0][q >> 1], sel), __builtin_amdgcn_perm(yv[3][q >> 1], yv[2][q >> 1], sel)};
+      d[q] = YmDot<T>::mfma16(u32x2{cur.s[q >> 1][2 * (q & 1)], cur.s[q >> 1][2 * (q & 1) + 1]}, yb, f32x4{0.f, 0.f, 0.f, 0.f});
+    }
+    load_s(cur, kn, s);
+    // d[q][t] = Z_r(i = 4 g + t, m = n) of slot 4 wv + q
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      *reinterpret_cast<u32x2*>(&z_s[s][((4 * g + t) * 16 + n) * MU_LDZ + 4 * wv]) = u32x2{ym_pack<T>(d[0][t], d[1][t]), ym_pack<T>(d[2][t], d[3][t])};
+    mu_barrier();                                   // Z of the step is whole (the other step's buffer was last read a barrier ago)
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+      const u32x4 zv = *reinterpret_cast<const u32x4*>(&z_s[s][((2 * wv + ii) * 16 + n) * MU_LDZ + 8 * g]);
+#pragma unroll
+      for (int nt = 0; nt < NTQ; ++nt) acc[ii][nt] = YmDot<T>::mfma(cur.u[ii][nt], zv, acc[ii][nt]);
+    }
+    load_u(cur, kn, s);
+  };
+  using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>;
+  Regs ra, rb;
+  // Y is the operand that comes from memory rather than from L2: two blocks of it are in flight per workgroup (one asked for
+  // 32 KB per block time, 12 GB/s per compute unit, and the block time was the latency of that request).  Block k asks for
+  // block k + 2 into the registers `yl` that block k gave to LDS, and puts block k + 1 from `ys` into LDS at its end.
+  auto block = [&](int k, u32x4 (&yl)[4], const u32x4 (&ys)[4]) {
+    load_y(yl, min(k + 2, NB - 1));
+    step(k, S0{}, ra);
+    step(k, S1{}, rb);
+    store_y(ys);                                    // every wave is past the barrier of the step: nobody reads this block of Y any more
+    mu_barrier();                                   // Y of the next block is whole
+  };
+
+  u32x4 y0[4], y1[4];
+  load_y(y0, 0); load_s(ra, 0, 0); load_u(ra, 0, 0); load_s(rb, 0, 1); load_u(rb, 0, 1);
+  load_y(y1, min(1, NB - 1));
+  store_y(y0);
+  mu_barrier();
+  TR6(1);
+  int k = 0;
+  for (; k + 1 < NB; k += 2) {
+    block(k, y0, y1);
+    block(k + 1, y1, y0);
+    TR6(2 + ((k >> 1) & 7));
+  }
+  if (k < NB) block(k, y0, y1);
+  TR6(14);
+
+  // acc[ii][nt][t] = out(m = m0 + n, column (2 wv + ii) Q + 16 nt + 4 g + t).  The tile (16 rows x 16 Q columns) goes through LDS
+  // (over Y and the first Z buffer, which nobody reads any more: every wave is past the last step's barrier) so that it leaves
+  // in whole rows: 16 bytes per lane, neighbouring lanes on neighbouring columns.
+  using V4 = typename TypeTraits<T>::vec4;
+  using V8 = typename TypeTraits<T>::vec8;
+  const int OLD = 16 * Q + 8;
+  uint16_t* const o_s = mu_lds;
+#pragma unroll
+  for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+    for (int nt = 0; nt < NTQ; ++nt) {
+      const int q = 16 * nt + 4 * g;
+      if (q < Q) {
+        V4 o;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) o[t] = TypeTraits<T>::from_f32(acc[ii][nt][t]);
+        *reinterpret_cast<V4*>(&o_s[n * OLD + (2 * wv + ii) * Q + q]) = o;
+      }
+    }
+  mu_barrier();
+  const int ppr = 2 * Q;                                   // 16-byte pieces per row
+  for (int pi = tid; pi < 16 * ppr; pi += MU_NT) {
+    const int mr = pi / ppr, col = (pi - mr * ppr) * 8, m = m0 + mr;
+    if (m >= M) break;
+    const V8 rv8 = *reinterpret_cast<const V8*>(&o_s[mr * OLD + col]);
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = TypeTraits<T>::to_f32(rv8[e]);
+    if (p.bias) {
+      const V8 bv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(p.bias) + col);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += TypeTraits<T>::to_f32(bv[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = apply_act(v[e], p.act);
+    if (p.gate || p.resid) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = TypeTraits<T>::to_f32(TypeTraits<T>::from_f32(v[e]));
+      if (p.gate) {
+        const V8 gv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(p.gate) + (int64_t)(m / p.gate_rows) * p.ld_gate + col);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= TypeTraits<T>::to_f32(gv[e]);
+      }
+      if (p.resid) {
+        const V8 rv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(p.resid) + (int64_t)m * p.ld_resid + col);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += TypeTraits<T>::to_f32(rv[e]);
+      }
+    }
+    V8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = TypeTraits<T>::from_f32(v[e]);
+    *reinterpret_cast<V8*>(reinterpret_cast<T*>(p.out) + (int64_t)m * p.ldo + col) = o;
+  }
+  TR6(15);
+}
+
+// U (16, Q, R) -> Ut (i, rank / 8, q, 8) and S(i, j, r) with any strides -> Sp (r / 2, j / 4, i, r % 2, 4): one thread per 16-byte
+// piece of Ut, then one per 8-byte piece of Sp.
+template <typename T>
+__global__ __launch_bounds__(256) void mixu_prep_kernel(const T* __restrict__ U, const T* __restrict__ S, T* __restrict__ Ut, T* __restrict__ Sp,
+                                                         int Q, int R, int64_t s_si, int64_t s_sj, int64_t s_sr) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int R8 = R / 8;
+  const int64_t nu = (int64_t)16 * R8 * Q;
+  if (idx < nu) {
+    const int q = (int)(idx % Q), o = (int)((idx / Q) % R8), i = (int)(idx / ((int64_t)Q * R8));
+    *reinterpret_cast<u32x4*>(Ut + idx * 8) = *reinterpret_cast<const u32x4*>(U + ((int64_t)i * Q + q) * R + 8 * o);
+  } else if (idx - nu < (int64_t)R * 64) {
+    const int64_t k = idx - nu;
+    const int l = (int)(k & 63), r = (int)(k >> 6), n = l & 15, g = l >> 4;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) Sp[(((int64_t)(r >> 1) * 64 + l) * 2 + (r & 1)) * 4 + t] = S[(int64_t)n * s_si + (int64_t)(4 * g + t) * s_sj + (int64_t)r * s_sr];
+  }
+}
+
+namespace {
+template <typename T>
+void* mixu_fn(int ntq) {
+  switch (ntq) {
+    case 1: return (void*)blast_mixu_kernel<T, 1>;
+    case 2: return (void*)blast_mixu_kernel<T, 2>;
+    case 3: return (void*)blast_mixu_kernel<T, 3>;
+    case 4: return (void*)blast_mixu_kernel<T, 4>;
+    case 5: return (void*)blast_mixu_kernel<T, 5>;
+    default: return nullptr;
+  }
+}
+}  // namespace
+
+// out (M, b Q) = [mix(S, Y)_i U_i]_i with the fused output stage of `ep` (bias, act, gate, resid; its other members are not
+// read).  Y (b, M, R), U (b, Q, R) of dtype.  scratch: room for U and S re-laid (b Q R + b b R elements, rounded up to 256
+// bytes each).  Returns BLR_OK, a negative blr_status, or 1 when the shape is not for this kernel (b other than 16, blocks wider than
+// 80 columns or not a multiple of 8, rank not a multiple of 32, unaligned operands, fp32).
+int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
+                      int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
+                      hipStream_t st) {
+  if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
+  if (b != 16 || Q % 8 || Q > 80 || Q < 8 || R % 32 || M < 1) return 1;
+  if (!aligned(Y, 16) || !aligned(U, 16) || !aligned(out, 16) || ldo % 8) return 1;
+  if ((ep.bias && !aligned(ep.bias, 16)) || (ep.gate && (!aligned(ep.gate, 16) || ep.ld_gate % 8 || ep.gate_rows < 1)) ||
+      (ep.resid && (!aligned(ep.resid, 16) || ep.ld_resid % 8))) return 1;
+  const int64_t y_bytes = (int64_t)b * M * R * 2;
+  if (y_bytes >= (int64_t)YM_OOB || (int64_t)b * Q * R * 2 >= (int64_t)YM_OOB || (int64_t)b * b * R * 2 >= (int64_t)YM_OOB) return 1;
+  if (cdiv(M, MU_BM) >= 2147483647LL) return 1;
+  MixuParams p = {};
+  p.Y = Y; p.out = out; p.ldo = ldo; p.M = M; p.R = R; p.Q = Q; p.y_bytes = (uint32_t)y_bytes;
+  p.bias = ep.bias; p.act = ep.act; p.gate = ep.gate; p.gate_rows = ep.gate ? ep.gate_rows : 1; p.ld_gate = ep.ld_gate;
+  p.resid = ep.resid; p.ld_resid = ep.ld_resid;
+  const size_t ut_bytes = align_up((size_t)b * Q * R * 2, 256), sp_bytes = (size_t)b * b * R * 2;
+  if (!scratch || scratch_bytes < ut_bytes + sp_bytes || !aligned(scratch, 16)) return 1;
+  void* Ut = scratch;
+  void* Sp = reinterpret_cast<char*>(scratch) + ut_bytes;
+  {
+    const unsigned tg = (unsigned)cdiv((int64_t)b * (R / 8) * Q + (int64_t)R * 64, 256);
+    if (dtype == BLR_F16) hipLaunchKernelGGL(mixu_prep_kernel<f16>, dim3(tg), dim3(256), 0, st, (const f16*)U, (const f16*)S, (f16*)Ut, (f16*)Sp, Q, R, s_si, s_sj, s_sr);
+    else hipLaunchKernelGGL(mixu_prep_kernel<bf16>, dim3(tg), dim3(256), 0, st, (const bf16*)U, (const bf16*)S, (bf16*)Ut, (bf16*)Sp, Q, R, s_si, s_sj, s_sr);
+    BLR_CHECK_LAUNCH("mixu_prep");
+  }
+  p.Ut = Ut; p.Sp = Sp;
+  void* fn = dtype == BLR_F16 ? mixu_fn<f16>((int)cdiv(Q, 16)) : mixu_fn<bf16>((int)cdiv(Q, 16));
+  if (!fn) return 1;
+  void* args[] = {&p};
+  hipError_t e = hipLaunchKernel(fn, dim3((unsigned)cdiv(M, MU_BM)), dim3(MU_NT), args, 0, st);
+  if (e != hipSuccess) { set_error("blast_mixu: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
 }
 

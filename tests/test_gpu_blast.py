@@ -113,6 +113,45 @@ def test_blast_fused_algorithm(name, shape, dtype):
     assert_close(out, back(tiled), dtype, f"fused against tiled {name}")
 
 
+NARROW_OUT = [(16, 288, 72, 576, (300,)), (16, 136, 40, 64, (129,)), (16, 200, 80, 96, (4, 50)), (16, 256, 8, 32, (131,)),
+              (16, 144, 24, 160, (1000,))]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", NARROW_OUT)
+def test_blast_bmm_narrow_output_blocks(shape, dtype):
+    """Output blocks of at most 80 columns with the bmm layouts above 128 rows: the mix and the product with U are one launch
+    that keeps the results of all 16 output blocks of a 16-row tile in registers (Z is never written).  Row counts that are
+    not multiples of 16, 1 to 5 column tiles per block, one to eighteen 32-rank chunks; then the same call with S handed over
+    as (j, i, r) through the C ABI, which the kernel transposes first, and with bias, activation, gate and residual."""
+    from triton_funcs import _lib as L
+    b, p, q, r, lead = shape
+    say(f"[case] narrow output blocks b={b} p={p} q={q} r={r} lead={lead} {dtype}")
+    x, U, Vt, S = blast_inputs(b, p, q, r, lead, seed=23)
+    ref = _ref(x, U, Vt, S, dtype)[0]
+    out = _run_blast("triton_blast_bmm_fp16", x, U, Vt, S, dtype, "tiled")
+    assert_close(out, ref.reshape(tuple(out.shape)), dtype, "narrow output blocks")
+    M, in_f, out_f = int(np.prod(lead)), b * p, b * q
+    Ub, Vb, _ = O.blast_to_bmm_layout(U, Vt, S)
+    _, _, Sp = O.blast_to_partial_layout(U, Vt, S)
+    lib = L.lib()
+    dt = L.F16 if dtype == torch.float16 else L.BF16
+    xd, Ud, Vd, Sd = dev(x.reshape(M, in_f), dtype), dev(Ub, dtype), dev(Vb, dtype), dev(Sp, dtype)
+    o2 = torch.empty((M, out_f), device="cuda", dtype=dtype)
+    ws = torch.empty(lib.blr_blast_workspace_bytes(M, in_f, out_f, b, r, dt, 2), device="cuda", dtype=torch.uint8)
+    L.check(lib.blr_blast_fwd(xd.data_ptr(), in_f, Ud.data_ptr(), Vd.data_ptr(), Sd.data_ptr(), o2.data_ptr(), out_f, None, None,
+                              M, in_f, out_f, b, r, dt, L.U_QR, L.S_JIR, 2, ws.data_ptr(), ws.numel(), L.stream_ptr(xd.device)), "blr_blast_fwd")
+    assert_close(o2, ref.reshape(M, out_f), dtype, "narrow output blocks, S as (j, i, r)")
+    rng = np.random.default_rng(24)
+    rows = 7
+    bias = rng.standard_normal(out_f); gate = rng.standard_normal((-(-M // rows), out_f)); resid = rng.standard_normal((M, out_f))
+    with L.fused_epilogue(dev(bias, dtype), "gelu_tanh", gate=dev(gate, dtype), gate_rows=rows, residual=dev(resid, dtype)):
+        out = _run_blast("triton_blast_bmm_fp16", x.reshape(M, in_f), U, Vt, S, dtype, "tiled")
+    v = ref.reshape(M, out_f) + rounded(bias, dtype)
+    h = 0.5 * v * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (v + 0.044715 * v ** 3)))
+    assert_close(out, rounded(resid, dtype) + np.repeat(rounded(gate, dtype), rows, axis=0)[:M] * h, dtype, "narrow output blocks + output stage", scale=2.0)
+
+
 def test_blast_fused_refuses_what_it_cannot_tile():
     from triton_funcs import _lib as L
     x, U, Vt, S = blast_inputs(2, 40, 24, 72, (5,), seed=22)              # two blocks: not a multiple of four
