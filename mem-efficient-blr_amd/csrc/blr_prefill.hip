@@ -538,9 +538,9 @@ __global__ __launch_bounds__(256) void mixu_prep_kernel(const T* __restrict__ U,
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int R8 = R / 8;
   const int64_t nu = (int64_t)16 * R8 * Q;
-  if (idx < nu) {
-    const int q = (int)(idx % Q), o = (int)((idx / Q) % R8), i = (int)(idx / ((int64_t)Q * R8));
-    *reinterpret_cast<u32x4*>(Ut + idx * 8) = *reinterpret_cast<const u32x4*>(U + ((int64_t)i * Q + q) * R + 8 * o);
+  if (idx < nu) {                                   // neighbouring threads read neighbouring pieces of a row of U
+    const int o = (int)(idx % R8), q = (int)((idx / R8) % Q), i = (int)(idx / ((int64_t)Q * R8));
+    *reinterpret_cast<u32x4*>(Ut + (((int64_t)i * R8 + o) * Q + q) * 8) = *reinterpret_cast<const u32x4*>(U + idx * 8);
   } else if (idx - nu < (int64_t)R * 64) {
     const int64_t k = idx - nu;
     const int l = (int)(k & 63), r = (int)(k >> 6), n = l & 15, g = l >> 4;
