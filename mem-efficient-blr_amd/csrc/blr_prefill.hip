@@ -74,7 +74,7 @@ __device__ __forceinline__ uint32_t ym_pack(float lo, float hi) {
   return __builtin_bit_cast(u32x2, v)[0];
 }
 
-template <typename T>
+template <typename T, bool STAGE>
 __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
   extern __shared__ __attribute__((aligned(16))) uint32_t ym_lds[];
   const int tid = threadIdx.x, wv = tid >> 6, l = tid & 63, n = l & 15, g = l >> 4;
@@ -210,10 +210,17 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
   // ---------------------------------------------- phase 2: the mix ----------------------------------------------------------
   // lane (n, g): operand A = S_r(i = n, j = 4 g .. 4 g + 3), operand B = Y_r(j = 4 g .. 4 g + 3, m = 16 mg + n); the
   // product's lane holds Z_r(i = 4 g + t, m = 16 mg + n), t = 0..3
-  if (rw < BR) {
-    const bool b_ok = 2 * g < JP;
+  // A lane's 16 bytes of Z belong to a row (i, m) of their own: stored from here, an instruction touches 64 cache lines and
+  // holds the memory pipeline eight times as long as one that writes whole rows (5.3 of a workgroup's 15 us were these
+  // stores).  STAGE: the 16 rows of a product group go through LDS behind Y ([i][m][rank], 16 lanes per row) and leave as
+  // runs of BR ranks; without (the tile's Y leaves no room for that) the lanes store their pieces themselves.
+  const bool b_ok = 2 * g < JP;
+  const int ZRS = BR / 2 + 4;                                // dwords per staged row
+  uint32_t* const z_st = ym_lds + JP * JS;
 #pragma unroll
-    for (int mg = 0; mg < 2; ++mg) {
+  for (int mg = 0; mg < 2; ++mg) {
+    if (STAGE && mg == 1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // the first group's rows have been read
+    if (rw < BR) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {                          // eight ranks at a time
         if (rw + 8 * h < BR) {
@@ -229,18 +236,34 @@ __global__ __launch_bounds__(YM_NT) void blast_ymix_kernel(YmixParams p) {
             d[q] = YmDot<T>::mfma16(sa[8 * h + q], yb, f32x4{0.f, 0.f, 0.f, 0.f});
           }
           const int m = m0 + 16 * mg + n, r = r0 + rw + 8 * h;
-          if (m < M && r < R) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              const int i = 4 * g + t;
-              if (i < b) {
-                u32x4 o;
+          for (int t = 0; t < 4; ++t) {
+            const int i = 4 * g + t;
+            u32x4 o;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) o[q] = ym_pack<T>(d[2 * q][t], d[2 * q + 1][t]);
-                *reinterpret_cast<u32x4*>(reinterpret_cast<T*>(p.Z) + ((int64_t)i * M + m) * R + r) = o;
-              }
+            for (int q = 0; q < 4; ++q) o[q] = ym_pack<T>(d[2 * q][t], d[2 * q + 1][t]);
+            if (STAGE) {
+              if (i < b) *reinterpret_cast<u32x4*>(&z_st[(i * 16 + n) * ZRS + (rw + 8 * h) / 2]) = o;
+            } else if (m < M && r < R && i < b) {
+              *reinterpret_cast<u32x4*>(reinterpret_cast<T*>(p.Z) + ((int64_t)i * M + m) * R + r) = o;
             }
           }
+        }
+      }
+    }
+    if (STAGE) {
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      const int pc = tid & 15, r = r0 + pc * 8;
+      if (pc < p.npc && r < R) {                           // 32 rows per pass: output blocks 2 it, 2 it + 1
+        const int rr = tid >> 4, m = m0 + 16 * mg + (rr & 15);
+        u32x4 v[8];
+#pragma unroll
+        for (int it = 0; it < 8; ++it)
+          if (2 * it < b) v[it] = *reinterpret_cast<const u32x4*>(&z_st[(rr + 32 * it) * ZRS + pc * 4]);
+        if (m < M) {
+#pragma unroll
+          for (int it = 0; it < 8; ++it)
+            if (2 * it + (rr >> 4) < b) *reinterpret_cast<u32x4*>(reinterpret_cast<T*>(p.Z) + ((int64_t)(2 * it + (rr >> 4)) * M + m) * R + r) = v[it];
         }
       }
     }
@@ -302,18 +325,23 @@ int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, 
     p.St = scratch;
   }
   const int BR = p.npc * 8;
-  const size_t lds = (size_t)(b / 2) * (YM_BM * (BR + 4) + 16) * 4;
-  void* fn = dtype == BLR_F16 ? (void*)blast_ymix_kernel<f16> : (void*)blast_ymix_kernel<bf16>;
-  static bool attr_set[2] = {false, false};
-  if (!attr_set[dtype == BLR_F16 ? 0 : 1]) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  const size_t lds_y = (size_t)(b / 2) * (YM_BM * (BR + 4) + 16) * 4;
+  const size_t lds_z = (size_t)b * 16 * (BR / 2 + 4) * 4;                 // the rows of one product group on their way out
+  static const int e_stage = env_i("BLR_YM_STAGE", 1);
+  const bool stage = e_stage && lds_y + lds_z <= 160 * 1024;
+  const size_t lds = lds_y + (stage ? lds_z : 0);
+  const int fi = (dtype == BLR_F16 ? 0 : 2) + (stage ? 1 : 0);
+  void* const fns[4] = {(void*)blast_ymix_kernel<f16, false>, (void*)blast_ymix_kernel<f16, true>,
+                        (void*)blast_ymix_kernel<bf16, false>, (void*)blast_ymix_kernel<bf16, true>};
+  static bool attr_set[4] = {false, false, false, false};
+  if (!attr_set[fi]) {
+    hipError_t e = hipFuncSetAttribute(fns[fi], hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) { set_error("blast_ymix: cannot raise the LDS limit: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
-    attr_set[dtype == BLR_F16 ? 0 : 1] = true;
+    attr_set[fi] = true;
   }
-  const dim3 grid((unsigned)(nrt * nmt)), block(YM_NT);
-  if (dtype == BLR_F16) hipLaunchKernelGGL(blast_ymix_kernel<f16>, grid, block, lds, st, p);
-  else hipLaunchKernelGGL(blast_ymix_kernel<bf16>, grid, block, lds, st, p);
-  BLR_CHECK_LAUNCH("blast_ymix");
+  void* args[] = {&p};
+  hipError_t e = hipLaunchKernel(fns[fi], dim3((unsigned)(nrt * nmt)), dim3(YM_NT), args, lds, st);
+  if (e != hipSuccess) { set_error("blast_ymix: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
 }
 
