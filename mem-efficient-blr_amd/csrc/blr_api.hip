@@ -173,10 +173,14 @@ bool epilogue_pending(const void** bias, int* act) {
 }
 void epilogue_taken() { tl_ep.used = true; }
 
-static void attach_epilogue(GemmArgs& g) {
+static void attach_epilogue_peek(GemmArgs& g) {      // the armed output stage, without claiming it
   if (!tl_ep.armed) return;
   g.bias = tl_ep.bias; g.act = tl_ep.act;
   g.gate = tl_ep.gate; g.gate_rows = tl_ep.gate_rows; g.ld_gate = tl_ep.ld_gate; g.resid = tl_ep.resid; g.ld_resid = tl_ep.ld_resid;
+}
+static void attach_epilogue(GemmArgs& g) {
+  if (!tl_ep.armed) return;
+  attach_epilogue_peek(g);
   tl_ep.used = true;
 }
 
@@ -339,6 +343,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   else if (s_layout == BLR_S_RIJ) { sr = (int64_t)b * b; si = b; sj = 1; }
   else { si = (int64_t)b * r; sj = r; sr = 1; }
   int rc = 1;
+  int mixu_prepared = 0;
   // A few dozen rows are still a weight-streaming problem: 256-row tiles would leave most compute units without one and the
   // others with a long stream each (4096 -> 4096 at 17 rows: 36 us through the tiles, 12 us at 16 rows through the few-row
   // kernels).  Up to 128 rows the three launches of the few-row path run over tiles of 16 rows with the weights held in registers
@@ -376,6 +381,13 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
     g1.C = Y; g1.ldc = r; g1.sC = (int64_t)M * r; g1.cn = 1;
     g1.M = M; g1.N = r; g1.K = P; g1.batch = b;
     g1.sat8 = sat8;
+    if (mixu) {                                     // the GEMM's launch also re-lays U and S for the kernel that follows, if it can
+      GemmArgs e2 = {};
+      attach_epilogue_peek(e2);
+      static const int side_on = getenv("BLR_MIXU_SIDE") ? atoi(getenv("BLR_MIXU_SIDE")) : 1;      // 0: a launch of its own
+      if (side_on && blast_mixu_plan(Y, S, U, out, ldo, e2, M, b, r, Q, si, sj, sr, dtype, Z, ybytes, &g1.side)) g1.side_taken = &mixu_prepared;
+      else g1.side.items = 0;
+    }
     rc = gemm_launch(g1, dtype, st);
     if (rc) return rc;
     if (!mixu) {
@@ -393,7 +405,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   g2.M = M; g2.N = Q; g2.K = r; g2.batch = b;
   if (!sat8) attach_epilogue(g2);
   if (mixu) {                                       // (Y is in memory: the branch above ran the GEMM and skipped the mix)
-    rc = blast_mixu_launch(Y, S, U, out, ldo, g2, M, b, r, Q, si, sj, sr, s_layout, dtype, Z, ybytes, st);
+    rc = blast_mixu_launch(Y, S, U, out, ldo, g2, M, b, r, Q, si, sj, sr, s_layout, dtype, Z, ybytes, st, mixu_prepared != 0);
     if (rc != 1) return rc;
     rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st, sat8);
     if (rc) return rc;

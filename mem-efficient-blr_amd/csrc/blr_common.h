@@ -101,6 +101,34 @@ static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; 
     }                                                                       \
   } while (0)
 
+// ---- a small job that rides along with a GEMM launch -------------------------------------------------------------
+// What blast_mixu_kernel wants re-laid before it runs (U (16, Q, R) -> Ut (i, rank / 8, q, 8); S(i, j, r) with any strides ->
+// Sp (r / 2, j / 4, i, r % 2, 4)) depends on the weights only, and the GEMM x V that precedes it in the same call touches neither:
+// extra workgroups of that GEMM's launch do it, which saves a launch of its own (4.7 us for 1.6 MB: start-up and one trip
+// to memory).  items: 16-byte pieces of Ut, then 8-byte pieces of Sp; 0 = no job.
+struct SidePrep {
+  const void* U; const void* S; void* Ut; void* Sp;
+  int Q, R;
+  int64_t s_si, s_sj, s_sr;
+  int64_t items;
+};
+template <typename T>
+__device__ __forceinline__ void side_prep_item(const SidePrep& s, int64_t idx) {
+  const T* U = reinterpret_cast<const T*>(s.U); const T* S = reinterpret_cast<const T*>(s.S);
+  T* Ut = reinterpret_cast<T*>(s.Ut); T* Sp = reinterpret_cast<T*>(s.Sp);
+  const int R8 = s.R / 8, Q = s.Q;
+  const int64_t nu = (int64_t)16 * R8 * Q;
+  if (idx < nu) {                                   // neighbouring threads read neighbouring pieces of a row of U
+    const int o = (int)(idx % R8), q = (int)((idx / R8) % Q), i = (int)(idx / ((int64_t)Q * R8));
+    *reinterpret_cast<u32x4*>(Ut + (((int64_t)i * R8 + o) * Q + q) * 8) = *reinterpret_cast<const u32x4*>(U + idx * 8);
+  } else if (idx - nu < (int64_t)s.R * 64) {
+    const int64_t k = idx - nu;
+    const int l = (int)(k & 63), r = (int)(k >> 6), n = l & 15, g = l >> 4;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) Sp[(((int64_t)(r >> 1) * 64 + l) * 2 + (r & 1)) * 4 + t] = S[(int64_t)n * s.s_si + (int64_t)(4 * g + t) * s.s_sj + (int64_t)r * s.s_sr];
+  }
+}
+
 // ---- tiled GEMM (blr_gemm.hip) ----------------------------------------------------------
 enum { EPI_PLAIN = 0, EPI_MONARCH_SCATTER = 1 };
 struct GemmArgs {
@@ -120,6 +148,8 @@ struct GemmArgs {
   void* splitk_ws;  // optional scratch for splitting the reduction (gemm_splitk_bytes says how much); null: never split
   size_t splitk_bytes;
   int kc;           // set by gemm_launch for the split kernels: k values per slice
+  SidePrep side;    // optional job for extra workgroups of the launch (items > 0); *side_taken is set to 1 by a launch that carries it
+  int* side_taken;  // (host pointer; the kernels that cannot carry the job leave it alone and the caller launches it itself)
 };
 // dtype: blr_dtype.  Returns blr_status.
 int gemm_launch(const GemmArgs& a, int dtype, hipStream_t st);
@@ -143,7 +173,11 @@ int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, 
 // the fused output stage (bias, act, gate, resid) is taken from `ep`.  Same return convention; scratch as above.
 int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
                       int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
-                      hipStream_t st);
+                      hipStream_t st, bool prepared = false);
+// Whether blast_mixu_launch takes the shape, and the job that re-lays U and S into `scratch` for it (what a GEMM launch earlier
+// in the call may carry; blast_mixu_launch is then told `prepared`).
+bool blast_mixu_plan(const void* Y, const void* S, const void* U, const void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
+                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, void* scratch, size_t scratch_bytes, SidePrep* job);
 
 // ---- streaming (decode) engine (blr_stream.hip) -------------------------------------------
 struct StreamBlastArgs {

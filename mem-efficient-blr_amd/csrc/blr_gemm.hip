@@ -410,7 +410,7 @@ __device__ __forceinline__ uint32_t ring_lds_addr(const void* p) {
 }
 
 template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false, int NWV = 4, bool PARTIAL = false>
-__global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m) {
+__global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m, int side_wgs) {
   constexpr int NA = ring_na<SHALLOW>(), NB = ring_nb<SHALLOW>();
   constexpr int ASTG = BM * 64, BSTG = BN * 64, BRING = NA * ASTG;   // stage sizes, start of the B ring
   constexpr int WGN = (NWV == 8 && BN == 256) ? 4 : 2, WGM = NWV / WGN;   // waves: 2 x 2, or 2 x 4 / 4 x 2 (two per SIMD)
@@ -427,6 +427,13 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   const int wm = wave / WGN, wn = wave % WGN;
   const int tiles = tiles_m * tiles_n;
   int u = blockIdx.x;
+  if (side_wgs > 0) {                                // the first workgroups of the launch carry the side job, not a tile (behind the
+    if (u < side_wgs) {                              // tiles, in the tail of the launch, they measured 2 % of a DiT-XL/2 forward slower)
+      for (int64_t idx = (int64_t)u * (NWV * 64) + tid; idx < g.side.items; idx += (int64_t)side_wgs * (NWV * 64)) side_prep_item<T>(g.side, idx);
+      return;
+    }
+    u -= side_wgs;
+  }
   if (per_xcd > 0) u = (u & 7) * per_xcd + (u >> 3);
   if (u >= tiles * g.batch) return;
   // interleaved columns: the batches of one tile write into the same cache lines, so they run next to each other (same
@@ -868,11 +875,16 @@ static int launch_ring(const GemmArgs& g, hipStream_t st) {
   if (total > (1ll << 30)) { set_error("gemm: too many tiles"); return BLR_ERR_UNSUPPORTED; }
   int per_xcd = xcd_on ? (int)cdiv(total, 8) : 0;
   int group_m = gm_env < 1 ? 1 : gm_env;
-  dim3 grid((unsigned)(per_xcd > 0 ? per_xcd * 8 : total));
+  // a side job: one thread per item, in workgroups ahead of the tiles (a multiple of eight of them, so that tile u stays on XCD u % 8)
+  int side_wgs = 0;
+  if (!PARTIAL && g.side.items > 0 && g.side_taken) side_wgs = (int)(cdiv(cdiv(g.side.items, NWV * 64), 8) * 8);
+  if (side_wgs > 4096) side_wgs = 4096;
+  dim3 grid((unsigned)((per_xcd > 0 ? per_xcd * 8 : total) + side_wgs));
   GemmArgs ga = g;
-  void* args[] = {&ga, &tiles_m, &tiles_n, &per_xcd, &group_m};
+  void* args[] = {&ga, &tiles_m, &tiles_n, &per_xcd, &group_m, &side_wgs};
   hipError_t e = hipLaunchKernel(fn, grid, dim3(NWV * 64), args, lds, st);
   if (e != hipSuccess) { set_error("gemm_ring: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  if (side_wgs > 0) *g.side_taken = 1;
   return BLR_OK;
 }
 

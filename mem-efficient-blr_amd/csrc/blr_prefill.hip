@@ -558,23 +558,11 @@ __global__ __launch_bounds__(MU_NT) void blast_mixu_kernel(MixuParams p) {
   TR6(15);
 }
 
-// U (16, Q, R) -> Ut (i, rank / 8, q, 8) and S(i, j, r) with any strides -> Sp (r / 2, j / 4, i, r % 2, 4): one thread per 16-byte
-// piece of Ut, then one per 8-byte piece of Sp.
+// The re-laying of U and S (side_prep_item) as a launch of its own: one thread per piece.
 template <typename T>
-__global__ __launch_bounds__(256) void mixu_prep_kernel(const T* __restrict__ U, const T* __restrict__ S, T* __restrict__ Ut, T* __restrict__ Sp,
-                                                         int Q, int R, int64_t s_si, int64_t s_sj, int64_t s_sr) {
+__global__ __launch_bounds__(256) void mixu_prep_kernel(SidePrep s) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int R8 = R / 8;
-  const int64_t nu = (int64_t)16 * R8 * Q;
-  if (idx < nu) {                                   // neighbouring threads read neighbouring pieces of a row of U
-    const int o = (int)(idx % R8), q = (int)((idx / R8) % Q), i = (int)(idx / ((int64_t)Q * R8));
-    *reinterpret_cast<u32x4*>(Ut + (((int64_t)i * R8 + o) * Q + q) * 8) = *reinterpret_cast<const u32x4*>(U + idx * 8);
-  } else if (idx - nu < (int64_t)R * 64) {
-    const int64_t k = idx - nu;
-    const int l = (int)(k & 63), r = (int)(k >> 6), n = l & 15, g = l >> 4;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) Sp[(((int64_t)(r >> 1) * 64 + l) * 2 + (r & 1)) * 4 + t] = S[(int64_t)n * s_si + (int64_t)(4 * g + t) * s_sj + (int64_t)r * s_sr];
-  }
+  if (idx < s.items) side_prep_item<T>(s, idx);
 }
 
 namespace {
@@ -591,38 +579,50 @@ void* mixu_fn(int ntq) {
 }
 }  // namespace
 
+bool blast_mixu_plan(const void* Y, const void* S, const void* U, const void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
+                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, void* scratch, size_t scratch_bytes, SidePrep* job) {
+  if (dtype != BLR_F16 && dtype != BLR_BF16) return false;
+  if (b != 16 || Q % 8 || Q > 80 || Q < 8 || R % 32 || M < 1) return false;
+  if (!aligned(Y, 16) || !aligned(U, 16) || !aligned(out, 16) || ldo % 8) return false;
+  if ((ep.bias && !aligned(ep.bias, 16)) || (ep.gate && (!aligned(ep.gate, 16) || ep.ld_gate % 8 || ep.gate_rows < 1)) ||
+      (ep.resid && (!aligned(ep.resid, 16) || ep.ld_resid % 8))) return false;
+  const int64_t y_bytes = (int64_t)b * M * R * 2;
+  if (y_bytes >= (int64_t)YM_OOB || (int64_t)b * Q * R * 2 >= (int64_t)YM_OOB || (int64_t)b * b * R * 2 >= (int64_t)YM_OOB) return false;
+  if (cdiv(M, MU_BM) >= 2147483647LL) return false;
+  if (!(dtype == BLR_F16 ? mixu_fn<f16>((int)cdiv(Q, 16)) : mixu_fn<bf16>((int)cdiv(Q, 16)))) return false;
+  const size_t ut_bytes = align_up((size_t)b * Q * R * 2, 256), sp_bytes = (size_t)b * b * R * 2;
+  if (!scratch || scratch_bytes < ut_bytes + sp_bytes || !aligned(scratch, 16)) return false;
+  if (job) {
+    job->U = U; job->S = S; job->Ut = scratch; job->Sp = reinterpret_cast<char*>(scratch) + ut_bytes;
+    job->Q = Q; job->R = R; job->s_si = s_si; job->s_sj = s_sj; job->s_sr = s_sr;
+    job->items = (int64_t)b * (R / 8) * Q + (int64_t)R * 64;
+  }
+  return true;
+}
+
 // out (M, b Q) = [mix(S, Y)_i U_i]_i with the fused output stage of `ep` (bias, act, gate, resid; its other members are not
 // read).  Y (b, M, R), U (b, Q, R) of dtype.  scratch: room for U and S re-laid (b Q R + b b R elements, rounded up to 256
-// bytes each).  Returns BLR_OK, a negative blr_status, or 1 when the shape is not for this kernel (b other than 16, blocks wider than
-// 80 columns or not a multiple of 8, rank not a multiple of 32, unaligned operands, fp32).
+// bytes each); prepared: an earlier launch of the call has already put them there.  Returns BLR_OK, a negative blr_status, or 1
+// when the shape is not for this kernel (b other than 16, blocks wider than 80 columns or not a multiple of 8, rank not a
+// multiple of 32, unaligned operands, fp32).
 int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
                       int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
-                      hipStream_t st) {
-  if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
-  if (b != 16 || Q % 8 || Q > 80 || Q < 8 || R % 32 || M < 1) return 1;
-  if (!aligned(Y, 16) || !aligned(U, 16) || !aligned(out, 16) || ldo % 8) return 1;
-  if ((ep.bias && !aligned(ep.bias, 16)) || (ep.gate && (!aligned(ep.gate, 16) || ep.ld_gate % 8 || ep.gate_rows < 1)) ||
-      (ep.resid && (!aligned(ep.resid, 16) || ep.ld_resid % 8))) return 1;
-  const int64_t y_bytes = (int64_t)b * M * R * 2;
-  if (y_bytes >= (int64_t)YM_OOB || (int64_t)b * Q * R * 2 >= (int64_t)YM_OOB || (int64_t)b * b * R * 2 >= (int64_t)YM_OOB) return 1;
-  if (cdiv(M, MU_BM) >= 2147483647LL) return 1;
+                      hipStream_t st, bool prepared) {
+  (void)s_layout;
+  SidePrep job = {};
+  if (!blast_mixu_plan(Y, S, U, out, ldo, ep, M, b, R, Q, s_si, s_sj, s_sr, dtype, scratch, scratch_bytes, &job)) return 1;
+  void* fn = dtype == BLR_F16 ? mixu_fn<f16>((int)cdiv(Q, 16)) : mixu_fn<bf16>((int)cdiv(Q, 16));
   MixuParams p = {};
-  p.Y = Y; p.out = out; p.ldo = ldo; p.M = M; p.R = R; p.Q = Q; p.y_bytes = (uint32_t)y_bytes;
+  p.Y = Y; p.out = out; p.ldo = ldo; p.M = M; p.R = R; p.Q = Q; p.y_bytes = (uint32_t)((int64_t)b * M * R * 2);
   p.bias = ep.bias; p.act = ep.act; p.gate = ep.gate; p.gate_rows = ep.gate ? ep.gate_rows : 1; p.ld_gate = ep.ld_gate;
   p.resid = ep.resid; p.ld_resid = ep.ld_resid;
-  const size_t ut_bytes = align_up((size_t)b * Q * R * 2, 256), sp_bytes = (size_t)b * b * R * 2;
-  if (!scratch || scratch_bytes < ut_bytes + sp_bytes || !aligned(scratch, 16)) return 1;
-  void* Ut = scratch;
-  void* Sp = reinterpret_cast<char*>(scratch) + ut_bytes;
-  {
-    const unsigned tg = (unsigned)cdiv((int64_t)b * (R / 8) * Q + (int64_t)R * 64, 256);
-    if (dtype == BLR_F16) hipLaunchKernelGGL(mixu_prep_kernel<f16>, dim3(tg), dim3(256), 0, st, (const f16*)U, (const f16*)S, (f16*)Ut, (f16*)Sp, Q, R, s_si, s_sj, s_sr);
-    else hipLaunchKernelGGL(mixu_prep_kernel<bf16>, dim3(tg), dim3(256), 0, st, (const bf16*)U, (const bf16*)S, (bf16*)Ut, (bf16*)Sp, Q, R, s_si, s_sj, s_sr);
+  p.Ut = job.Ut; p.Sp = job.Sp;
+  if (!prepared) {
+    const unsigned tg = (unsigned)cdiv(job.items, 256);
+    if (dtype == BLR_F16) hipLaunchKernelGGL(mixu_prep_kernel<f16>, dim3(tg), dim3(256), 0, st, job);
+    else hipLaunchKernelGGL(mixu_prep_kernel<bf16>, dim3(tg), dim3(256), 0, st, job);
     BLR_CHECK_LAUNCH("mixu_prep");
   }
-  p.Ut = Ut; p.Sp = Sp;
-  void* fn = dtype == BLR_F16 ? mixu_fn<f16>((int)cdiv(Q, 16)) : mixu_fn<bf16>((int)cdiv(Q, 16));
-  if (!fn) return 1;
   void* args[] = {&p};
   hipError_t e = hipLaunchKernel(fn, dim3((unsigned)cdiv(M, MU_BM)), dim3(MU_NT), args, 0, st);
   if (e != hipSuccess) { set_error("blast_mixu: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
