@@ -375,6 +375,7 @@ struct MixuParams {
   const void* Y; const void* Sp; const void* Ut; void* out; int64_t ldo;     // Sp (r / 2, j / 4, i, r % 2, 4), Ut (i, rank / 8, q, 8)
   int M, R, Q;
   uint32_t y_bytes;
+  int rotate;
   const void* bias; int act;
   const void* gate; int gate_rows; int64_t ld_gate;
   const void* resid; int64_t ld_resid;
@@ -390,6 +391,11 @@ __global__ __launch_bounds__(MU_NT) void blast_mixu_kernel(MixuParams p) {
   const int m0 = (int)blockIdx.x * MU_BM;
   const int NB = (R + MU_RB - 1) / MU_RB;             // the last block may hold 32 ranks: what lies past them is not asked for
   const bool half_u = (R % MU_RB) != 0 && g >= 2, half_y = (R % MU_RB) != 0 && (l & 7) >= 4;
+  // Workgroups walk the blocks of ranks in turn from different starting points: all of them read the same ranks of U and S
+  // otherwise, at the same moment, from the same lines of the eight L2s.  (The sum over the blocks is in fp32 and its order is
+  // fixed per row tile.)
+  const int rot = p.rotate ? (int)(blockIdx.x % (unsigned)NB) : 0;
+  auto blk = [&](int k) { const int kk = k + rot; return kk >= NB ? kk - NB : kk; };
   TR6(0);
   const __amdgpu_buffer_rsrc_t ybuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.Y), 0, p.y_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t sbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.Sp), 0, (uint32_t)(256 * R * 2), 0x00020000);
@@ -447,7 +453,7 @@ __global__ __launch_bounds__(MU_NT) void blast_mixu_kernel(MixuParams p) {
   // and nothing else.
   auto step = [&](int k, auto SS, Regs& cur) {
     constexpr int s = decltype(SS)::value;
-    const int kn = min(k + 1, NB - 1);
+    const int kn = blk(min(k + 1, NB - 1));
     // the mix of this wave's four ranks: operand B = Y_r(j = 4 g .. 4 g + 3, m = n), gathered from the four rows of its lane
     u32x2 yv[4];
 #pragma unroll
@@ -475,11 +481,12 @@ __global__ __launch_bounds__(MU_NT) void blast_mixu_kernel(MixuParams p) {
   };
   using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>;
   Regs ra, rb;
-  // Y is the operand that comes from memory rather than from L2: two blocks of it are in flight per workgroup (one asked for
-  // 32 KB per block time, 12 GB/s per compute unit, and the block time was the latency of that request).  Block k asks for
-  // block k + 2 into the registers `yl` that block k gave to LDS, and puts block k + 1 from `ys` into LDS at its end.
+  // Block k asks for Y of block k + 2 into the registers `yl` that block k gave to LDS, and puts block k + 1 from `ys` into LDS at
+  // its end.  (Loads return to a wave in the order it asked, and S and U are asked for one block ahead, so Y in effect has one
+  // block's time as well; what bounds a step is the 112 KB per workgroup that 256 workgroups draw from L2 and memory, about
+  // 1.4 us against 0.5 us for a step without loads.)
   auto block = [&](int k, u32x4 (&yl)[4], const u32x4 (&ys)[4]) {
-    load_y(yl, min(k + 2, NB - 1));
+    load_y(yl, blk(min(k + 2, NB - 1)));
     step(k, S0{}, ra);
     step(k, S1{}, rb);
     store_y(ys);                                    // every wave is past the barrier of the step: nobody reads this block of Y any more
@@ -487,8 +494,8 @@ __global__ __launch_bounds__(MU_NT) void blast_mixu_kernel(MixuParams p) {
   };
 
   u32x4 y0[4], y1[4];
-  load_y(y0, 0); load_s(ra, 0, 0); load_u(ra, 0, 0); load_s(rb, 0, 1); load_u(rb, 0, 1);
-  load_y(y1, min(1, NB - 1));
+  load_y(y0, blk(0)); load_s(ra, blk(0), 0); load_u(ra, blk(0), 0); load_s(rb, blk(0), 1); load_u(rb, blk(0), 1);
+  load_y(y1, blk(min(1, NB - 1)));
   store_y(y0);
   mu_barrier();
   TR6(1);
@@ -617,6 +624,7 @@ int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, in
   p.bias = ep.bias; p.act = ep.act; p.gate = ep.gate; p.gate_rows = ep.gate ? ep.gate_rows : 1; p.ld_gate = ep.ld_gate;
   p.resid = ep.resid; p.ld_resid = ep.ld_resid;
   p.Ut = job.Ut; p.Sp = job.Sp;
+  { static const int e_rot = env_i("BLR_MIXU_ROTATE", 1); p.rotate = e_rot; }
   if (!prepared) {
     const unsigned tg = (unsigned)cdiv(job.items, 256);
     if (dtype == BLR_F16) hipLaunchKernelGGL(mixu_prep_kernel<f16>, dim3(tg), dim3(256), 0, st, job);
