@@ -932,6 +932,10 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       // (a reduction of a few steps only: the smaller tile, three workgroups per compute unit - 4096 x 288 x 72 in 16 batches
       // 1.7 us faster than with 256 x 128)
       if (g.K <= 128 && r128 >= 3 * (int64_t)cus) { rt = 128128; if (!per_cu) per_cu = 2; }
+      // a wide output with a reduction of a thousand or two: enough 256 x 256 tiles for two rounds, and the big tile's lower LDS
+      // traffic per matrix instruction beats the overlap of two smaller workgroups (2048 x 22016 x 1024: 164.7 -> 154.1 us for
+      // the whole low-rank call; four batches of 2048 x 5504 x 1024: Monarch 184.6 -> 176.8 us)
+      else if (g.K >= 1024 && g.K <= 2048 && g.N >= 2048 && t256 >= 2 * (int64_t)cus) rt = 256256;
       else if (g.K <= 2048 && t128 >= 2 * (int64_t)cus) { rt = 256128; if (!per_cu) per_cu = 2; }
       else if (g.K <= 512 && r128 >= fill) rt = 128128;
       // a narrow output (one 128-column tile, mostly empty at 256): more, smaller tiles (4096 x 72 x 576 in 16 batches:
