@@ -369,6 +369,17 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   // wherever the kernel takes the shape.
   static const int mixu_mode = getenv("BLR_BLAST_MIXU") ? atoi(getenv("BLR_BLAST_MIXU")) : 2;
   const bool mixu_shape = !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && b == 16 && u_layout == BLR_U_QR && Q % 8 == 0 && Q <= 80 && r % 32 == 0;
+  // Narrow input blocks as well (at most 96 columns): the whole call is one launch that forms Y per step of the rank walk in the
+  // compute unit and keeps neither Y nor Z in memory (blast_one_kernel).  BLR_BLAST_ONE=0 switches it off.
+  static const int one_mode = getenv("BLR_BLAST_ONE") ? atoi(getenv("BLR_BLAST_ONE")) : 1;
+  if (one_mode && mixu_shape && !y_out && P <= 96 && P % 8 == 0) {
+    GemmArgs e1 = {};
+    attach_epilogue_peek(e1);
+    rc = blast_one_launch(x, ldx, U, V, S, out, ldo, e1, M, in_f, b, r, Q, si, sj, sr, dtype, ws, ws_bytes, st);
+    if (rc == BLR_OK && !sat8) { GemmArgs claim = {}; attach_epilogue(claim); }
+    if (rc != 1) return rc;
+    rc = 1;
+  }
   const bool mixu = mixu_shape && (mixu_mode >= 2 || (mixu_mode == 1 && (P > fuse_max_p || fused < 0)));
   if (!mixu && !y_out && !sat8 && fused >= 0 && (fused == 1 || P <= fuse_max_p))
     rc = blast_ymix_launch(x, ldx, V, S, Z, M, in_f, b, r, si, sj, sr, s_layout, dtype, Y, ybytes, st);   // (the unused room of Y holds S transposed)

@@ -179,6 +179,12 @@ int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, in
 bool blast_mixu_plan(const void* Y, const void* S, const void* U, const void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
                      int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, void* scratch, size_t scratch_bytes, SidePrep* job);
 
+// The whole BLAST call in one launch for 16 input blocks of at most 96 columns and 16 output blocks of at most 80 (U (b, Q, R)):
+// neither Y nor Z in memory.  scratch: room for V, U and S re-laid.  Same return convention as the two above.
+int blast_one_launch(const void* x, int64_t ldx, const void* U, const void* V, const void* S, void* out, int64_t ldo, const GemmArgs& ep,
+                     int M, int in_f, int b, int R, int Q, int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype,
+                     void* scratch, size_t scratch_bytes, hipStream_t st);
+
 // ---- streaming (decode) engine (blr_stream.hip) -------------------------------------------
 struct StreamBlastArgs {
   const void* x; int64_t ldx;

@@ -637,6 +637,274 @@ int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, in
   return BLR_OK;
 }
 
+// ---- narrow input AND output blocks: the whole call in one launch, neither Y nor Z in memory ------------------------------
+//
+// With input blocks of at most 96 columns the chunk of V that a step of blast_mixu_kernel's walk over the rank needs (16 input
+// blocks x P x 32 ranks) is as small as its chunk of U, so the workgroup forms the step's Y itself instead of reading it: wave w
+// keeps its rows of x for input blocks 2 w and 2 w + 1 in registers (operand B, 16 rows x P), loads the 32 ranks of V_2w and
+// V_2w+1 (operand A: V re-laid like U, rank-major with k contiguous, in the order the lanes read it, k padded to 32 KS with
+// zeros) and leaves Y^T (ranks x rows) as T in LDS - four consecutive ranks per lane.  The rest of the step is the step of
+// blast_mixu_kernel: mix of four ranks per wave into Z (LDS), barrier, products with U_2w, U_2w+1 into the 16 x 16 Q results
+// that stay in registers for the whole call.  Three barriers per step; Y and Z have one buffer each (every reader of a buffer is
+// past the barrier that precedes its next writer in program order).
+struct OneParams {
+  const void* x; int64_t ldx; uint32_t x_bytes;
+  const void* Vp; const void* Sp; const void* Ut; void* out; int64_t ldo;     // Vp (step, j, half, kstep, lane, 8), Sp, Ut as for blast_mixu_kernel
+  int M, P, R, Q;
+  const void* bias; int act;
+  const void* gate; int gate_rows; int64_t ld_gate;
+  const void* resid; int64_t ld_resid;
+};
+
+template <typename T, int NTQ, int KS>
+__global__ __launch_bounds__(MU_NT) void blast_one_kernel(OneParams p) {
+  constexpr int LDY = 40;                                    // two-byte elements per LDS row of Y and Z (32 ranks / slots + 8)
+  constexpr int OSN = 16 * (16 * 80 + 8);                      // the tile on its way out: 16 rows of up to 16 x 80 columns (+ 8)
+  __shared__ __attribute__((aligned(16))) uint16_t one_lds[2 * 256 * LDY > OSN ? 2 * 256 * LDY : OSN];
+  uint16_t* const y_s = one_lds;                             // [input block j][row m][rank of the step]
+  uint16_t* const z_s = one_lds + 256 * LDY;                 // [output block i][row m][slot]
+  const int tid = threadIdx.x, wv = tid >> 6, l = tid & 63, n = l & 15, g = l >> 4;
+  const int M = p.M, P = p.P, R = p.R, Q = p.Q;
+  const int m0 = (int)blockIdx.x * MU_BM;
+  const int NSTEP = R / 32;
+  const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.x), 0, p.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t vbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.Vp), 0, (uint32_t)((int64_t)NSTEP * 16 * 2 * KS * 1024), 0x00020000);
+  const __amdgpu_buffer_rsrc_t sbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.Sp), 0, (uint32_t)(256 * R * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t ubuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.Ut), 0, (uint32_t)((int64_t)16 * Q * R * 2), 0x00020000);
+  // the rows of x: operand B of the first products, lane (n, g) = row m0 + n, k = 32 ks + 8 g .. + 7 of input block 2 wv + jj
+  u32x4 xr[2][KS];
+#pragma unroll
+  for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int k = 32 * ks + 8 * g;
+      const uint32_t off = (m0 + n < M && k < P) ? (uint32_t)((int64_t)(m0 + n) * p.ldx + (int64_t)(2 * wv + jj) * P + k) * 2u : YM_OOB;
+      xr[jj][ks] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xbuf, off, 0, 0));
+    }
+  const uint32_t voff = (uint32_t)((2 * wv) * 2 * KS * 1024 + l * 16);     // + ((jj 2 + nt) KS + ks) 1024; a step is 16 * 2 * KS KiB further
+  const uint32_t soff = (uint32_t)((2 * wv) * 64 + l) * 16u;
+  const uint32_t uoff = (uint32_t)(((int64_t)(2 * wv) * (R / 8) + g) * Q + n) * 16u;
+  const uint32_t uoff_last = 16 * (NTQ - 1) + n < Q ? uoff : YM_OOB;
+  const uint32_t uis = (uint32_t)((R / 8) * Q) * 16u;
+  struct Regs { u32x4 s[2]; u32x4 u[2][NTQ]; };
+  u32x4 vr[2][2][KS];
+  auto load_v = [&](int s) {
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          vr[jj][nt][ks] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vbuf, voff + (uint32_t)(((jj * 2 + nt) * KS + ks) * 1024), (uint32_t)s * (uint32_t)(16 * 2 * KS * 1024), 0));
+  };
+  auto load_s = [&](Regs& r, int s) {                        // ranks 32 s + 4 wv + q
+#pragma unroll
+    for (int q = 0; q < 2; ++q) r.s[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(sbuf, soff + (uint32_t)q * 1024u, (uint32_t)(32 * s) * 512u, 0));
+  };
+  auto load_u = [&](Regs& r, int s) {
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+      for (int nt = 0; nt < NTQ; ++nt)
+        r.u[ii][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ubuf, (nt == NTQ - 1 ? uoff_last : uoff) + (uint32_t)nt * 256u,
+                                                                                        (uint32_t)(4 * s * Q) * 16u + (uint32_t)ii * uis, 0));
+  };
+  f32x4 acc[2][NTQ];
+#pragma unroll
+  for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+    for (int nt = 0; nt < NTQ; ++nt) acc[ii][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // Workgroups start at different steps (the fp32 sums keep a fixed order per row tile): they would otherwise all ask the L2s
+  // for the same lines of V, U and S at the same moment.
+  const int rot = (int)(blockIdx.x % (unsigned)NSTEP);
+  auto stp = [&](int s) { const int v = s + rot; return v >= NSTEP ? v - NSTEP : v; };
+
+  // No load sits under a condition (the compiler would then wait for everything in flight where the paths meet): the last steps
+  // ask again for the last step, which costs their turns in the memory pipeline and nothing else.
+  auto step = [&](int s, Regs& cur) {
+    const int s1 = stp(min(s + 1, NSTEP - 1)), s2 = stp(min(s + 2, NSTEP - 1));
+    // Y^T of the step: ranks 16 nt + 4 g + t of rows m = n, input blocks 2 wv and 2 wv + 1
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        f32x4 y = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) y = YmDot<T>::mfma(vr[jj][nt][ks], xr[jj][ks], y);
+        *reinterpret_cast<u32x2*>(&y_s[((2 * wv + jj) * 16 + n) * LDY + 16 * nt + 4 * g]) = u32x2{ym_pack<T>(y[0], y[1]), ym_pack<T>(y[2], y[3])};
+      }
+    load_v(s1);
+    mu_barrier();                                   // Y of the step is whole
+    // the mix of this wave's four ranks: operand B = Y_r(j = 4 g .. 4 g + 3, m = n), gathered from the four rows of its lane
+    u32x2 yv[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) yv[t] = *reinterpret_cast<const u32x2*>(&y_s[((4 * g + t) * 16 + n) * LDY + 4 * wv]);
+    f32x4 d[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+      const u32x2 yb = {__builtin_amdgcn_perm(yv[1][q >> 1], yv[0][q >> 1], sel), __builtin_amdgcn_perm(yv[3][q >> 1], yv[2][q >> 1], sel)};
+      d[q] = YmDot<T>::mfma16(u32x2{cur.s[q >> 1][2 * (q & 1)], cur.s[q >> 1][2 * (q & 1) + 1]}, yb, f32x4{0.f, 0.f, 0.f, 0.f});
+    }
+    load_s(cur, s2);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      *reinterpret_cast<u32x2*>(&z_s[((4 * g + t) * 16 + n) * LDY + 4 * wv]) = u32x2{ym_pack<T>(d[0][t], d[1][t]), ym_pack<T>(d[2][t], d[3][t])};
+    mu_barrier();                                   // Z of the step is whole; nobody reads this step's Y any more
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+      const u32x4 zv = *reinterpret_cast<const u32x4*>(&z_s[((2 * wv + ii) * 16 + n) * LDY + 8 * g]);
+#pragma unroll
+      for (int nt = 0; nt < NTQ; ++nt) acc[ii][nt] = YmDot<T>::mfma(cur.u[ii][nt], zv, acc[ii][nt]);
+    }
+    load_u(cur, s2);
+  };
+  Regs ra, rb;
+  load_v(stp(0));
+  load_s(ra, stp(0)); load_u(ra, stp(0));
+  load_s(rb, stp(min(1, NSTEP - 1))); load_u(rb, stp(min(1, NSTEP - 1)));
+  int s = 0;
+  for (; s + 1 < NSTEP; s += 2) { step(s, ra); step(s + 1, rb); }
+  if (s < NSTEP) step(s, ra);
+  mu_barrier();                                     // every wave is through with Z: the tile may go over it
+
+  // the tile (16 rows x 16 Q columns) leaves through LDS in whole rows, as in blast_mixu_kernel
+  using V4 = typename TypeTraits<T>::vec4;
+  using V8 = typename TypeTraits<T>::vec8;
+  const int OLD = 16 * Q + 8;
+  uint16_t* const o_s = one_lds;
+#pragma unroll
+  for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+    for (int nt = 0; nt < NTQ; ++nt) {
+      const int q = 16 * nt + 4 * g;
+      if (q < Q) {
+        V4 o;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) o[t] = TypeTraits<T>::from_f32(acc[ii][nt][t]);
+        *reinterpret_cast<V4*>(&o_s[n * OLD + (2 * wv + ii) * Q + q]) = o;
+      }
+    }
+  mu_barrier();
+  const int ppr = 2 * Q;
+  for (int pi = tid; pi < 16 * ppr; pi += MU_NT) {
+    const int mr = pi / ppr, col = (pi - mr * ppr) * 8, m = m0 + mr;
+    if (m >= M) break;
+    const V8 rv8 = *reinterpret_cast<const V8*>(&o_s[mr * OLD + col]);
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = TypeTraits<T>::to_f32(rv8[e]);
+    if (p.bias) {
+      const V8 bv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(p.bias) + col);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += TypeTraits<T>::to_f32(bv[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = apply_act(v[e], p.act);
+    if (p.gate || p.resid) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = TypeTraits<T>::to_f32(TypeTraits<T>::from_f32(v[e]));
+      if (p.gate) {
+        const V8 gv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(p.gate) + (int64_t)(m / p.gate_rows) * p.ld_gate + col);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= TypeTraits<T>::to_f32(gv[e]);
+      }
+      if (p.resid) {
+        const V8 rv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(p.resid) + (int64_t)m * p.ld_resid + col);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += TypeTraits<T>::to_f32(rv[e]);
+      }
+    }
+    V8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = TypeTraits<T>::from_f32(v[e]);
+    *reinterpret_cast<V8*>(reinterpret_cast<T*>(p.out) + (int64_t)m * p.ldo + col) = o;
+  }
+}
+
+// V (16, P, R) -> Vp (step, j, half of the step's ranks, k step, lane (n, g), 8): element e of lane (n, g) is
+// V_j[32 ks + 8 g + e][32 step + 16 half + n], zero past P; then U and S as side_prep_item lays them.  One thread per 16-byte piece.
+template <typename T>
+__global__ __launch_bounds__(256) void one_prep_kernel(const T* __restrict__ V, T* __restrict__ Vp, int P, int KS, SidePrep s) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t nv = (int64_t)(s.R / 32) * 16 * 2 * KS * 64;
+  if (idx < nv) {
+    const int l = (int)(idx & 63), n = l & 15, g = l >> 4;
+    int64_t c = idx >> 6;
+    const int ks = (int)(c % KS); c /= KS;
+    const int half = (int)(c & 1); c >>= 1;
+    const int j = (int)(c & 15), step = (int)(c >> 4);
+    typename TypeTraits<T>::vec8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int k = 32 * ks + 8 * g + e;
+      o[e] = k < P ? V[((int64_t)j * P + k) * s.R + 32 * step + 16 * half + n] : (T)0.0f;
+    }
+    *reinterpret_cast<typename TypeTraits<T>::vec8*>(Vp + idx * 8) = o;
+  } else if (idx - nv < s.items) {
+    side_prep_item<T>(s, idx - nv);
+  }
+}
+
+namespace {
+template <typename T, int KS>
+void* one_fn_ks(int Q) {
+  return Q <= 48 ? (void*)blast_one_kernel<T, 3, KS> : (void*)blast_one_kernel<T, 5, KS>;
+}
+template <typename T>
+void* one_fn(int Q, int ks) {
+  switch (ks) {
+    case 1: return one_fn_ks<T, 1>(Q);
+    case 2: return one_fn_ks<T, 2>(Q);
+    case 3: return one_fn_ks<T, 3>(Q);
+    default: return nullptr;
+  }
+}
+}  // namespace
+
+// out = BLAST(x) for 16 input blocks of at most 96 columns and 16 output blocks of at most 80, U (b, Q, R): one launch after the
+// re-laying of V, U and S into scratch (b (32 ceil(P / 32) + Q + b) R elements, each part rounded up to 256 bytes).  The fused
+// output stage is taken from `ep`.  Returns BLR_OK, a negative blr_status, or 1 when the shape is not for this kernel.
+int blast_one_launch(const void* x, int64_t ldx, const void* U, const void* V, const void* S, void* out, int64_t ldo, const GemmArgs& ep,
+                     int M, int in_f, int b, int R, int Q, int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype,
+                     void* scratch, size_t scratch_bytes, hipStream_t st) {
+  if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
+  if (b != 16 || in_f % 16) return 1;
+  const int P = in_f / 16, KS = (int)cdiv(P, 32);
+  if (P % 8 || P > 96 || Q % 8 || Q > 80 || Q < 8 || R % 32 || M < 1) return 1;
+  if (!aligned(x, 16) || ldx % 8 || !aligned(U, 16) || !aligned(V, 16) || !aligned(out, 16) || ldo % 8) return 1;
+  if ((ep.bias && !aligned(ep.bias, 16)) || (ep.gate && (!aligned(ep.gate, 16) || ep.ld_gate % 8 || ep.gate_rows < 1)) ||
+      (ep.resid && (!aligned(ep.resid, 16) || ep.ld_resid % 8))) return 1;
+  const int64_t x_elems = (int64_t)(M - 1) * ldx + in_f;
+  if (x_elems * 2 >= (int64_t)YM_OOB || (int64_t)b * Q * R * 2 >= (int64_t)YM_OOB || (int64_t)b * b * R * 2 >= (int64_t)YM_OOB ||
+      (int64_t)b * 32 * KS * R * 2 >= (int64_t)YM_OOB || cdiv(M, MU_BM) >= 2147483647LL) return 1;
+  const size_t vp_bytes = align_up((size_t)b * 32 * KS * R * 2, 256), ut_bytes = align_up((size_t)b * Q * R * 2, 256), sp_bytes = (size_t)b * b * R * 2;
+  if (!scratch || scratch_bytes < vp_bytes + ut_bytes + sp_bytes || !aligned(scratch, 16)) return 1;
+  void* fn = dtype == BLR_F16 ? one_fn<f16>(Q, KS) : one_fn<bf16>(Q, KS);
+  if (!fn) return 1;
+  char* sp = reinterpret_cast<char*>(scratch);
+  SidePrep job = {};
+  job.U = U; job.S = S; job.Ut = sp + vp_bytes; job.Sp = sp + vp_bytes + ut_bytes;
+  job.Q = Q; job.R = R; job.s_si = s_si; job.s_sj = s_sj; job.s_sr = s_sr;
+  job.items = (int64_t)b * (R / 8) * Q + (int64_t)R * 64;
+  {
+    const int64_t nv = (int64_t)(R / 32) * 16 * 2 * KS * 64;
+    const unsigned tg = (unsigned)cdiv(nv + job.items, 256);
+    if (dtype == BLR_F16) hipLaunchKernelGGL(one_prep_kernel<f16>, dim3(tg), dim3(256), 0, st, (const f16*)V, (f16*)sp, P, KS, job);
+    else hipLaunchKernelGGL(one_prep_kernel<bf16>, dim3(tg), dim3(256), 0, st, (const bf16*)V, (bf16*)sp, P, KS, job);
+    BLR_CHECK_LAUNCH("one_prep");
+  }
+  OneParams p = {};
+  p.x = x; p.ldx = ldx; p.x_bytes = (uint32_t)(x_elems * 2); p.Vp = sp; p.Sp = job.Sp; p.Ut = job.Ut; p.out = out; p.ldo = ldo;
+  p.M = M; p.P = P; p.R = R; p.Q = Q;
+  p.bias = ep.bias; p.act = ep.act; p.gate = ep.gate; p.gate_rows = ep.gate ? ep.gate_rows : 1; p.ld_gate = ep.ld_gate;
+  p.resid = ep.resid; p.ld_resid = ep.ld_resid;
+  void* args[] = {&p};
+  hipError_t e = hipLaunchKernel(fn, dim3((unsigned)cdiv(M, MU_BM)), dim3(MU_NT), args, 0, st);
+  if (e != hipSuccess) { set_error("blast_one: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  return BLR_OK;
+}
+
 }  // namespace blr
 
 #ifdef BLR_TRACE

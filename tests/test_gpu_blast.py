@@ -114,14 +114,17 @@ def test_blast_fused_algorithm(name, shape, dtype):
 
 
 NARROW_OUT = [(16, 288, 72, 576, (300,)), (16, 136, 40, 64, (129,)), (16, 200, 80, 96, (4, 50)), (16, 256, 8, 32, (131,)),
-              (16, 144, 24, 160, (1000,))]
+              (16, 144, 24, 160, (1000,)),
+              # input blocks of at most 96 columns as well: the whole call is one launch (one to three 32-column steps of x V)
+              (16, 72, 72, 288, (300,)), (16, 40, 24, 96, (177,)), (16, 96, 80, 64, (4, 50)), (16, 8, 8, 32, (133,)), (16, 64, 40, 160, (1000,))]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", NARROW_OUT)
 def test_blast_bmm_narrow_output_blocks(shape, dtype):
     """Output blocks of at most 80 columns with the bmm layouts above 128 rows: the mix and the product with U are one launch
-    that keeps the results of all 16 output blocks of a 16-row tile in registers (Z is never written).  Row counts that are
+    that keeps the results of all 16 output blocks of a 16-row tile in registers (Z is never written); with input blocks of at most
+    96 columns that launch forms Y as well and is the whole call.  Row counts that are
     not multiples of 16, 1 to 5 column tiles per block, one to eighteen 32-rank chunks; then the same call with S handed over
     as (j, i, r) through the C ABI, which the kernel transposes first, and with bias, activation, gate and residual."""
     from triton_funcs import _lib as L
