@@ -362,20 +362,20 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   // block on that costs more than the round trip of Y it saves (measured at 4096 rows: 1152 -> 1152, r = 288: 64 against
   // 68 us; 4608 -> 1152, r = 576: 154 against 122 us; Llama-7B gate_up at 2048 rows: 201 against 186 us).
   static const int fuse_max_p = getenv("BLR_BLAST_FUSE_MAX_P") ? atoi(getenv("BLR_BLAST_FUSE_MAX_P")) : 128;
-  // Narrow output blocks with the rank contiguous in U: the mix and the product with U run as one launch that reads Y once and
+  // Narrow output blocks (either layout of U: it is re-laid for the kernel anyway): the mix and the product with U run as one launch that reads Y once and
   // never writes Z (blast_mixu_kernel); the first half is then the plain GEMM, which leaves Y.  Measured at 4096 rows against the
   // mix kernel + batched GEMM: 4608 -> 1152, r = 576: 90 against 122 us; against the fused first half + batched GEMM: 1152 -> 1152,
   // r = 288: 47 against 51 us.  BLR_BLAST_MIXU: 0 never, 1 only where the first half would not be fused anyway, 2 (default)
   // wherever the kernel takes the shape.
   static const int mixu_mode = getenv("BLR_BLAST_MIXU") ? atoi(getenv("BLR_BLAST_MIXU")) : 2;
-  const bool mixu_shape = !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && b == 16 && u_layout == BLR_U_QR && Q % 8 == 0 && Q <= 80 && r % 32 == 0;
+  const bool mixu_shape = !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && b == 16 && Q % 8 == 0 && Q <= 80 && r % 32 == 0;
   // Narrow input blocks as well (at most 96 columns): the whole call is one launch that forms Y per step of the rank walk in the
   // compute unit and keeps neither Y nor Z in memory (blast_one_kernel).  BLR_BLAST_ONE=0 switches it off.
   static const int one_mode = getenv("BLR_BLAST_ONE") ? atoi(getenv("BLR_BLAST_ONE")) : 1;
   if (one_mode && mixu_shape && !y_out && P <= 96 && P % 8 == 0) {
     GemmArgs e1 = {};
     attach_epilogue_peek(e1);
-    rc = blast_one_launch(x, ldx, U, V, S, out, ldo, e1, M, in_f, b, r, Q, si, sj, sr, dtype, ws, ws_bytes, st);
+    rc = blast_one_launch(x, ldx, U, V, S, out, ldo, e1, M, in_f, b, r, Q, si, sj, sr, dtype, ws, ws_bytes, st, u_layout == BLR_U_RQ);
     if (rc == BLR_OK && !sat8) { GemmArgs claim = {}; attach_epilogue(claim); }
     if (rc != 1) return rc;
     rc = 1;
@@ -396,7 +396,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
       GemmArgs e2 = {};
       attach_epilogue_peek(e2);
       static const int side_on = getenv("BLR_MIXU_SIDE") ? atoi(getenv("BLR_MIXU_SIDE")) : 1;      // 0: a launch of its own
-      if (side_on && blast_mixu_plan(Y, S, U, out, ldo, e2, M, b, r, Q, si, sj, sr, dtype, Z, ybytes, &g1.side)) g1.side_taken = &mixu_prepared;
+      if (side_on && blast_mixu_plan(Y, S, U, out, ldo, e2, M, b, r, Q, si, sj, sr, dtype, Z, ybytes, &g1.side, u_layout == BLR_U_RQ)) g1.side_taken = &mixu_prepared;
       else g1.side.items = 0;
     }
     rc = gemm_launch(g1, dtype, st);
@@ -416,7 +416,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   g2.M = M; g2.N = Q; g2.K = r; g2.batch = b;
   if (!sat8) attach_epilogue(g2);
   if (mixu) {                                       // (Y is in memory: the branch above ran the GEMM and skipped the mix)
-    rc = blast_mixu_launch(Y, S, U, out, ldo, g2, M, b, r, Q, si, sj, sr, s_layout, dtype, Z, ybytes, st, mixu_prepared != 0);
+    rc = blast_mixu_launch(Y, S, U, out, ldo, g2, M, b, r, Q, si, sj, sr, s_layout, dtype, Z, ybytes, st, mixu_prepared != 0, u_layout == BLR_U_RQ);
     if (rc != 1) return rc;
     rc = blast_mix_launch(Y, S, Z, M, b, r, si, sj, sr, dtype, st, sat8);
     if (rc) return rc;

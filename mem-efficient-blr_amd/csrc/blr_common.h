@@ -109,6 +109,7 @@ static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; 
 struct SidePrep {
   const void* U; const void* S; void* Ut; void* Sp;
   int Q, R;
+  int u_rq;          // U comes as (16, R, Q) instead of (16, Q, R)
   int64_t s_si, s_sj, s_sr;
   int64_t items;
 };
@@ -118,7 +119,13 @@ __device__ __forceinline__ void side_prep_item(const SidePrep& s, int64_t idx) {
   T* Ut = reinterpret_cast<T*>(s.Ut); T* Sp = reinterpret_cast<T*>(s.Sp);
   const int R8 = s.R / 8, Q = s.Q;
   const int64_t nu = (int64_t)16 * R8 * Q;
-  if (idx < nu) {                                   // neighbouring threads read neighbouring pieces of a row of U
+  if (idx < nu && s.u_rq) {                         // U (i, r, q): neighbouring threads take neighbouring columns q, eight ranks each
+    const int q = (int)(idx % Q), o = (int)((idx / Q) % R8), i = (int)(idx / ((int64_t)Q * R8));
+    typename TypeTraits<T>::vec8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = U[((int64_t)i * s.R + 8 * o + e) * Q + q];
+    *reinterpret_cast<typename TypeTraits<T>::vec8*>(Ut + idx * 8) = v;
+  } else if (idx < nu) {                            // U (i, q, r): neighbouring threads read neighbouring pieces of a row of U
     const int o = (int)(idx % R8), q = (int)((idx / R8) % Q), i = (int)(idx / ((int64_t)Q * R8));
     *reinterpret_cast<u32x4*>(Ut + (((int64_t)i * R8 + o) * Q + q) * 8) = *reinterpret_cast<const u32x4*>(U + idx * 8);
   } else if (idx - nu < (int64_t)s.R * 64) {
@@ -169,21 +176,21 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
 int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, void* Z, int M, int in_f, int b, int R,
                       int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
                       hipStream_t st);
-// Second half for output blocks of at most 80 columns: out_i = mix(S, Y)_i U_i with U (b, Q, R), in one launch and without Z;
+// Second half for output blocks of at most 80 columns: out_i = mix(S, Y)_i U_i with U (b, Q, R) (u_rq: (b, R, Q)), in one launch and without Z;
 // the fused output stage (bias, act, gate, resid) is taken from `ep`.  Same return convention; scratch as above.
 int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
                       int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
-                      hipStream_t st, bool prepared = false);
+                      hipStream_t st, bool prepared = false, bool u_rq = false);
 // Whether blast_mixu_launch takes the shape, and the job that re-lays U and S into `scratch` for it (what a GEMM launch earlier
 // in the call may carry; blast_mixu_launch is then told `prepared`).
 bool blast_mixu_plan(const void* Y, const void* S, const void* U, const void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
-                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, void* scratch, size_t scratch_bytes, SidePrep* job);
+                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, void* scratch, size_t scratch_bytes, SidePrep* job, bool u_rq = false);
 
 // The whole BLAST call in one launch for 16 input blocks of at most 96 columns and 16 output blocks of at most 80 (U (b, Q, R)):
 // neither Y nor Z in memory.  scratch: room for V, U and S re-laid.  Same return convention as the two above.
 int blast_one_launch(const void* x, int64_t ldx, const void* U, const void* V, const void* S, void* out, int64_t ldo, const GemmArgs& ep,
                      int M, int in_f, int b, int R, int Q, int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype,
-                     void* scratch, size_t scratch_bytes, hipStream_t st);
+                     void* scratch, size_t scratch_bytes, hipStream_t st, bool u_rq = false);
 
 // ---- streaming (decode) engine (blr_stream.hip) -------------------------------------------
 struct StreamBlastArgs {

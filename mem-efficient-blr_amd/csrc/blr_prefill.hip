@@ -587,7 +587,7 @@ void* mixu_fn(int ntq) {
 }  // namespace
 
 bool blast_mixu_plan(const void* Y, const void* S, const void* U, const void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
-                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, void* scratch, size_t scratch_bytes, SidePrep* job) {
+                     int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype, void* scratch, size_t scratch_bytes, SidePrep* job, bool u_rq) {
   if (dtype != BLR_F16 && dtype != BLR_BF16) return false;
   if (b != 16 || Q % 8 || Q > 80 || Q < 8 || R % 32 || M < 1) return false;
   if (!aligned(Y, 16) || !aligned(U, 16) || !aligned(out, 16) || ldo % 8) return false;
@@ -601,7 +601,7 @@ bool blast_mixu_plan(const void* Y, const void* S, const void* U, const void* ou
   if (!scratch || scratch_bytes < ut_bytes + sp_bytes || !aligned(scratch, 16)) return false;
   if (job) {
     job->U = U; job->S = S; job->Ut = scratch; job->Sp = reinterpret_cast<char*>(scratch) + ut_bytes;
-    job->Q = Q; job->R = R; job->s_si = s_si; job->s_sj = s_sj; job->s_sr = s_sr;
+    job->Q = Q; job->R = R; job->u_rq = u_rq ? 1 : 0; job->s_si = s_si; job->s_sj = s_sj; job->s_sr = s_sr;
     job->items = (int64_t)b * (R / 8) * Q + (int64_t)R * 64;
   }
   return true;
@@ -614,10 +614,10 @@ bool blast_mixu_plan(const void* Y, const void* S, const void* U, const void* ou
 // multiple of 32, unaligned operands, fp32).
 int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, int64_t ldo, const GemmArgs& ep, int M, int b, int R, int Q,
                       int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
-                      hipStream_t st, bool prepared) {
+                      hipStream_t st, bool prepared, bool u_rq) {
   (void)s_layout;
   SidePrep job = {};
-  if (!blast_mixu_plan(Y, S, U, out, ldo, ep, M, b, R, Q, s_si, s_sj, s_sr, dtype, scratch, scratch_bytes, &job)) return 1;
+  if (!blast_mixu_plan(Y, S, U, out, ldo, ep, M, b, R, Q, s_si, s_sj, s_sr, dtype, scratch, scratch_bytes, &job, u_rq)) return 1;
   void* fn = dtype == BLR_F16 ? mixu_fn<f16>((int)cdiv(Q, 16)) : mixu_fn<bf16>((int)cdiv(Q, 16));
   MixuParams p = {};
   p.Y = Y; p.out = out; p.ldo = ldo; p.M = M; p.R = R; p.Q = Q; p.y_bytes = (uint32_t)((int64_t)b * M * R * 2);
@@ -862,12 +862,12 @@ void* one_fn(int Q, int ks) {
 }
 }  // namespace
 
-// out = BLAST(x) for 16 input blocks of at most 96 columns and 16 output blocks of at most 80, U (b, Q, R): one launch after the
+// out = BLAST(x) for 16 input blocks of at most 96 columns and 16 output blocks of at most 80, U (b, Q, R) or (u_rq) (b, R, Q): one launch after the
 // re-laying of V, U and S into scratch (b (32 ceil(P / 32) + Q + b) R elements, each part rounded up to 256 bytes).  The fused
 // output stage is taken from `ep`.  Returns BLR_OK, a negative blr_status, or 1 when the shape is not for this kernel.
 int blast_one_launch(const void* x, int64_t ldx, const void* U, const void* V, const void* S, void* out, int64_t ldo, const GemmArgs& ep,
                      int M, int in_f, int b, int R, int Q, int64_t s_si, int64_t s_sj, int64_t s_sr, int dtype,
-                     void* scratch, size_t scratch_bytes, hipStream_t st) {
+                     void* scratch, size_t scratch_bytes, hipStream_t st, bool u_rq) {
   if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
   if (b != 16 || in_f % 16) return 1;
   const int P = in_f / 16, KS = (int)cdiv(P, 32);
@@ -885,7 +885,7 @@ int blast_one_launch(const void* x, int64_t ldx, const void* U, const void* V, c
   char* sp = reinterpret_cast<char*>(scratch);
   SidePrep job = {};
   job.U = U; job.S = S; job.Ut = sp + vp_bytes; job.Sp = sp + vp_bytes + ut_bytes;
-  job.Q = Q; job.R = R; job.s_si = s_si; job.s_sj = s_sj; job.s_sr = s_sr;
+  job.Q = Q; job.R = R; job.u_rq = u_rq ? 1 : 0; job.s_si = s_si; job.s_sj = s_sj; job.s_sr = s_sr;
   job.items = (int64_t)b * (R / 8) * Q + (int64_t)R * 64;
   {
     const int64_t nv = (int64_t)(R / 32) * 16 * 2 * KS * 64;

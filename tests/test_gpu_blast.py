@@ -134,6 +134,8 @@ def test_blast_bmm_narrow_output_blocks(shape, dtype):
     ref = _ref(x, U, Vt, S, dtype)[0]
     out = _run_blast("triton_blast_bmm_fp16", x, U, Vt, S, dtype, "tiled")
     assert_close(out, ref.reshape(tuple(out.shape)), dtype, "narrow output blocks")
+    out = _run_blast("triton_blast_full_fp16", x, U, Vt, S, dtype, "tiled")          # U as (b, r, q), S as (j, i, r): re-laid as well
+    assert_close(out, ref.reshape(tuple(out.shape)), dtype, "narrow output blocks, U (b, r, q)")
     M, in_f, out_f = int(np.prod(lead)), b * p, b * q
     Ub, Vb, _ = O.blast_to_bmm_layout(U, Vt, S)
     _, _, Sp = O.blast_to_partial_layout(U, Vt, S)
