@@ -338,11 +338,15 @@ def main():
             dit = {"batch": 16, "tokens_per_image": 256, "dtype": "f16"}
             import contextlib
             with contextlib.redirect_stdout(sys.stderr):          # the harness reports what it replaced; stdout carries the one JSON line only
-                for method in ("blast", "low_rank", "dense"):
+                # BLAST and dense are within a few per cent of each other and the card drifts by as much between one measurement and
+                # the next: both are measured twice, in alternating order, and the faster pass of each is reported
+                for method in ("blast", "low_rank", "dense", "blast", "dense"):
                     lc = {k: {"rank": v.get("rank"), "b": v.get("b"), "func": v["triton"]["func"]} for k, v in ncfg[method].items()}
                     ms = dit_xl.benchmark(method, "triton", lc, 256, 10, dev, f16, batch=16)
+                    ms = min(ms, dit.get(f"{method}_ms", ms))
                     dit[f"{method}_img_per_s"] = round(16 / (ms * 1e-3), 1)
                     dit[f"{method}_ms"] = round(ms, 3)
+                dit["passes"] = {"blast": 2, "dense": 2, "low_rank": 1, "nn_linear": 1}
                 ms = dit_xl.benchmark(None, None, None, 256, 10, dev, f16, batch=16)        # stock nn.Linear (hipBLASLt) for scale
             dit["nn_linear_img_per_s"] = round(16 / (ms * 1e-3), 1)
             torch.cuda.empty_cache()
