@@ -565,7 +565,7 @@ static size_t monarch_rows_bytes(int M, int in_f, int b, int rank, int dtype) {
   if (P > 1024)
     for (int ks = (P + 1023) / 1024; ks <= 8; ++ks)
       if (P % ks == 0 && (P / ks) % 8 == 0) { mks = ks; break; }
-  return align_up((size_t)b * mks * M * rank * 2, 256) + align_up((size_t)b * M * rank * 2, 256);
+  return align_up((size_t)b * mks * M * rank * (mks > 1 ? 4 : 2), 256) + align_up((size_t)b * M * rank * 2, 256);   // slices: fp32 partial sums
 }
 
 size_t blr_monarch_workspace_bytes(int M, int in_f, int out_f, int b, int rank, int dtype, int algo) {
@@ -650,7 +650,7 @@ static int low_rank_slices(int in_f) {
 static size_t low_rank_rows_bytes(int M, int in_f, int r, int dtype) {
   const int bi = low_rank_slices(in_f);
   if (M <= 16 || M > 128 || dtype == BLR_F32 || !bi) return 0;
-  return align_up((size_t)bi * M * r * 2, 256) + align_up((size_t)M * r * 2, 256);
+  return align_up((size_t)bi * M * r * 4, 256) + align_up((size_t)M * r * 2, 256);   // fp32 partial sums of the slices, then z
 }
 
 size_t blr_low_rank_workspace_bytes(int M, int in_f, int out_f, int r, int dtype, int algo) {

@@ -6,11 +6,14 @@ namespace blr {
 
 // Bytes of the fixed-place workspace block that holds the tagged values exchanged by workgroups.
 size_t decode2_region_bytes();
+// Bytes of the fixed-place workspace block behind it that the multi-launch paths use as ordinary scratch (y, z, re-laid S).
+// It is a block of its own so that no plain value is ever left where a single-launch kernel looks for a tagged one.
+size_t decode2_plain_bytes();
 // Whether the call can be served by the two-stage decode kernel at all (layout, dtype, M).
 bool decode2_applicable(const StreamBlastArgs& a);
 // Returns BLR_OK, a negative blr_status, or 1 when the shape does not fit the kernel's tiling
 // (the caller then uses the phase engine).
-int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
+int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, unsigned* epoch_word, unsigned* arrive_word,
                          unsigned* err_word, hipStream_t st);
 
 // The same call on the one-workgroup-per-compute-unit kernel (blr_decode3.hip; up to four token rows).  Returns BLR_OK, a

@@ -1280,6 +1280,7 @@ void* d2_kernel(int MT, int wbits) {
 }  // namespace
 
 size_t decode2_region_bytes() { return (size_t)16 << 20; }
+size_t decode2_plain_bytes() { return (size_t)8 << 20; }
 
 bool decode2_applicable(const StreamBlastArgs& a) {
   static const int enabled = env_i("BLR_DECODE2", 1);
@@ -1302,13 +1303,13 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
 
 // region: the fixed-place 16 MiB block of the workspace reserved for tagged pairs; ctrl3: three
 // words on separate cache lines (epoch, arrivals, error).
-int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
+int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, unsigned* epoch_word, unsigned* arrive_word,
                          unsigned* err_word, hipStream_t st) {
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
   static const int rows_min_m = env_i("BLR_DECODE_ROWS_MIN_M", 2);
   if (M >= rows_min_m || a.wbits == 4 || a.rows_only) {   // (4-bit codes at one row too: 15.8 against 16.9 - 20.6 us on the single-row kernels)
-    const int rc = decode_rows_launch(a, region, decode2_region_bytes(), st);
+    const int rc = decode_rows_launch(a, plain, decode2_plain_bytes(), st);
     if (rc != 1) return rc;
   }
   if (a.rows_only) { set_error("blast_q: code rows that are not whole 16-byte pieces need in_f / b, r and out_f / b to be multiples of 8 and at most 4096"); return BLR_ERR_UNSUPPORTED; }
@@ -1317,10 +1318,10 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     // about 12 us at 4096 -> 4096), the two launches for deeper input blocks (11008 -> 4096: input blocks of 2752 rows)
     int rc = decode3_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
     if (rc != 1) return rc;
-    rc = decode_pair_launch(a, region, decode2_region_bytes(), st);
+    rc = decode_pair_launch(a, plain, decode2_plain_bytes(), st);
     if (rc != 1) return rc;
   } else {
-    int rc = decode_pair_launch(a, region, decode2_region_bytes(), st);
+    int rc = decode_pair_launch(a, plain, decode2_plain_bytes(), st);
     if (rc != 1) return rc;
     rc = decode3_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
     if (rc != 1) return rc;

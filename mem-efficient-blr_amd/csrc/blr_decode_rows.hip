@@ -48,6 +48,8 @@ struct RowsParams {
   const void* bias; int act;              // fused output stage (bias of T indexed like a row of out, or null; blr_act), applied to
                                           // the result rounded to T - what a separate elementwise kernel would see
   int ep;
+  int out_f32;                            // the product is one slice of a reduction: out holds fp32 partial sums (plain row-major
+                                          // store, no scales, no output stage) that the next launch adds in slice order
   const f16* scales;                      // codes: the product's column n of entry bt is multiplied by scales[bt * N + n]; else null
   int M, K, N;
   int kw;                                 // rows of a wave's share per round (a multiple of 32)
@@ -297,7 +299,11 @@ __global__ __launch_bounds__(DR_NT) void rows_product_kernel(RowsParams p) {
         tot[e] = apply_act(v, p.act);
       }
   }
-  if (mrow0 + m < p.M && c4 < cw && col < N) {
+  if (p.out_f32) {
+    // (N is a multiple of 8 and col of 4: the four columns are all inside)
+    if (mrow0 + m < p.M && c4 < cw && col < N)
+      *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.out) + (int64_t)(mrow0 + m) * p.o_ms + (int64_t)bt * p.o_bs + col) = tot;
+  } else if (mrow0 + m < p.M && c4 < cw && col < N) {
     T* o = reinterpret_cast<T*>(p.out) + (int64_t)(mrow0 + m) * p.o_ms + (int64_t)bt * p.o_bs;
     int ocol = col;
     if (p.per > 0) {                                     // (per is a multiple of 4: the four columns stay together)
@@ -408,23 +414,25 @@ __global__ __launch_bounds__(256) void rows_mix_kernel(const T* __restrict__ Y, 
   *reinterpret_cast<V4*>(Z + ((int64_t)i * M + m) * R + r4 * 4) = o;
 }
 
-// Low rank seen as BLAST with one output block and S = 1: z[m][r] = sum_j y[j][m][r] (the k-slices of x A), fp32 sums in slice order.
+// Low rank seen as BLAST with one output block and S = 1: z[m][r] = sum_j y[j][m][r] (the k-slices of x A).  The slices are
+// fp32 partial sums, added in slice order and rounded to T once - the reduction is then accumulated in fp32 from end to end,
+// as a single-pass product does (reference triton_funcs/low_rank_kernels.py:98-112, dense_kernels.py:80-98).
 template <typename T>
-__global__ __launch_bounds__(256) void rows_sum_kernel(const T* __restrict__ Y, T* __restrict__ Z, int b, int64_t MR4, RowsPrefetch pf, uint32_t nmix) {
+__global__ __launch_bounds__(256) void rows_sum_kernel(const float* __restrict__ Y, T* __restrict__ Z, int b, int64_t MR4, RowsPrefetch pf, uint32_t nmix) {
   if (blockIdx.x >= nmix) { rows_prefetch(pf, nmix); return; }
   const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (item >= MR4) return;
   using V4 = typename TypeTraits<T>::vec4;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   for (int j0 = 0; j0 < b; j0 += 8) {
-    V4 v[8];
+    f32x4 v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const V4*>(Y + ((int64_t)min(j0 + u, b - 1) * MR4 + item) * 4);
+    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const f32x4*>(Y + ((int64_t)min(j0 + u, b - 1) * MR4 + item) * 4);
 #pragma unroll
     for (int u = 0; u < 8; ++u)
       if (j0 + u < b)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] += TypeTraits<T>::to_f32(v[u][e]);
+        for (int e = 0; e < 4; ++e) acc[e] += v[u][e];
   }
   V4 o;
 #pragma unroll
@@ -433,9 +441,10 @@ __global__ __launch_bounds__(256) void rows_sum_kernel(const T* __restrict__ Y, 
 }
 
 // Monarch with its input blocks cut into ks slices (so that the first product spreads over the chip): the slices are added and
-// the permutation applied in one pass, z[l][m][r] = sum_s y[(r / per) ks + s][m][l per + r % per]; thread = four ranks.
+// the permutation applied in one pass, z[l][m][r] = sum_s y[(r / per) ks + s][m][l per + r % per]; thread = four ranks.  The
+// slices are fp32 partial sums (one rounding, after the sum).
 template <typename T>
-__global__ __launch_bounds__(256) void rows_perm_sum_kernel(const T* __restrict__ Y, T* __restrict__ Z, int ks, int M, int R, int per, int64_t items,
+__global__ __launch_bounds__(256) void rows_perm_sum_kernel(const float* __restrict__ Y, T* __restrict__ Z, int ks, int M, int R, int per, int64_t items,
                                                             RowsPrefetch pf, uint32_t nmix) {
   if (blockIdx.x >= nmix) { rows_prefetch(pf, nmix); return; }
   const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -448,9 +457,9 @@ __global__ __launch_bounds__(256) void rows_perm_sum_kernel(const T* __restrict_
   const int yj = r / per, yr = l * per + (r - yj * per);
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   for (int s = 0; s < ks; ++s) {
-    const V4 v = *reinterpret_cast<const V4*>(Y + (((int64_t)(yj * ks + s) * M + m) * R + yr));
+    const f32x4 v = *reinterpret_cast<const f32x4*>(Y + (((int64_t)(yj * ks + s) * M + m) * R + yr));
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[e] += TypeTraits<T>::to_f32(v[e]);
+    for (int e = 0; e < 4; ++e) acc[e] += v[e];
   }
   V4 o;
 #pragma unroll
@@ -650,7 +659,8 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     for (int ks = (P + 1023) / 1024; ks <= 8; ++ks)
       if (P % ks == 0 && (P / ks) % 8 == 0) { mks = ks; break; }
   }
-  const size_t ybytes = align_up((size_t)b * mks * M * R * 2, 256), zbytes = align_up((size_t)bo * M * R * 2, 256);
+  const bool y_f32 = lowrank || mks > 1;                // y holds slices of one reduction: fp32 partial sums, rounded once after their sum
+  const size_t ybytes = align_up((size_t)b * mks * M * R * (y_f32 ? 4 : 2), 256), zbytes = align_up((size_t)bo * M * R * 2, 256);
   if (ybytes + zbytes > region_bytes) return 1;
   void* Y = region;
   void* Z = reinterpret_cast<char*>(region) + ybytes;
@@ -664,6 +674,7 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   s1.M = M; s1.K = P; s1.N = R; s1.scales = a.wbits != 16 ? (const f16*)a.v_scales : nullptr;
   if (monarch && mks == 1) { s1.out = Z; s1.o_bs = 0; s1.per = a.perm_per; s1.o_ls = (int64_t)M * R; s1.perdiv = fd_make((uint32_t)a.perm_per); }
   if (mks > 1) { s1.a_bs = P / mks; s1.w_bs = (int64_t)(P / mks) * R; s1.K = P / mks; }
+  s1.out_f32 = y_f32 ? 1 : 0;
   RowsParams s2 = {};
   s2.A = Z; s2.lda = R; s2.a_bs = (int64_t)M * R; s2.a_bytes = (uint32_t)((size_t)bo * M * R * 2);
   s2.W = a.U; s2.w_bs = (int64_t)R * Q;
@@ -693,16 +704,16 @@ int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   if (monarch && mks > 1) {
     const int64_t items = (int64_t)bo * M * R / 4;
     const uint32_t nmix = (uint32_t)cdiv(items, 256);
-    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_perm_sum_kernel<f16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const f16*)Y, (f16*)Z, mks, M, R, a.perm_per, items, pf, nmix);
-    else hipLaunchKernelGGL(rows_perm_sum_kernel<bf16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const bf16*)Y, (bf16*)Z, mks, M, R, a.perm_per, items, pf, nmix);
+    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_perm_sum_kernel<f16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const float*)Y, (f16*)Z, mks, M, R, a.perm_per, items, pf, nmix);
+    else hipLaunchKernelGGL(rows_perm_sum_kernel<bf16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const float*)Y, (bf16*)Z, mks, M, R, a.perm_per, items, pf, nmix);
     BLR_CHECK_LAUNCH("rows_perm_sum");
   } else if (monarch)
     rc = BLR_OK;
   else if (lowrank) {
     const int64_t mr4 = (int64_t)M * R / 4;
     const uint32_t nmix = (uint32_t)cdiv(mr4, 256);
-    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_sum_kernel<f16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const f16*)Y, (f16*)Z, b, mr4, pf, nmix);
-    else hipLaunchKernelGGL(rows_sum_kernel<bf16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const bf16*)Y, (bf16*)Z, b, mr4, pf, nmix);
+    if (a.dtype == BLR_F16) hipLaunchKernelGGL(rows_sum_kernel<f16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const float*)Y, (f16*)Z, b, mr4, pf, nmix);
+    else hipLaunchKernelGGL(rows_sum_kernel<bf16>, dim3(nmix + prefetch_blocks(pf)), dim3(256), 0, st, (const float*)Y, (bf16*)Z, b, mr4, pf, nmix);
     BLR_CHECK_LAUNCH("rows_sum");
   } else if (sr == 1 && si % 4 == 0 && sj % 4 == 0 && R % 4 == 0 && aligned(a.S, 8) && (int64_t)M * b * (R / 4) * (R / 4) < ((int64_t)1 << 32) && b < 65536)   // the multiply-high division is exact below 2^32 / divisor
     rc = a.dtype == BLR_F16 ? rows_mix_t<f16>(Y, a.S, Z, M, b, R, si, sj, pf, st) : rows_mix_t<bf16>(Y, a.S, Z, M, b, R, si, sj, pf, st);
@@ -733,7 +744,7 @@ static bool dense_rows_wanted(int M, int out_f) { return M > 16 && M <= DR_MAX_M
 size_t dense_rows_bytes(int M, int in_f, int out_f, int dtype) {
   const int bi = dense_slices(in_f);
   if (!dense_rows_wanted(M, out_f) || (dtype != BLR_F16 && dtype != BLR_BF16) || !bi || out_f % 8) return 0;
-  return bi > 1 ? align_up((size_t)bi * M * out_f * 2, 256) : 0;
+  return bi > 1 ? align_up((size_t)bi * M * out_f * 4, 256) : 0;    // fp32 partial sums of the slices
 }
 
 int dense_rows_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int in_f, int out_f, int dtype,
@@ -748,7 +759,7 @@ int dense_rows_launch(const void* x, int64_t ldx, const void* W, void* out, int6
   s.A = x; s.lda = ldx; s.a_bs = in_f / bi; s.a_bytes = (uint32_t)(x_elems * 2);
   s.W = W; s.w_bs = (int64_t)(in_f / bi) * out_f;
   s.out = bi > 1 ? ws : out; s.o_ms = bi > 1 ? out_f : ldo; s.o_bs = (int64_t)M * out_f; s.o_ns = 1;
-  s.M = M; s.K = in_f / bi; s.N = out_f;
+  s.M = M; s.K = in_f / bi; s.N = out_f; s.out_f32 = bi > 1 ? 1 : 0;
   const void* ep_bias = nullptr; int ep_act = 0;
   if (bi == 1 && epilogue_pending(&ep_bias, &ep_act)) { s.ep = 1; s.bias = ep_bias; s.act = ep_act; }
   int rc = rows_plan(s, bi, dtype, 16, false);
@@ -759,8 +770,8 @@ int dense_rows_launch(const void* x, int64_t ldx, const void* W, void* out, int6
   const int64_t mn4 = (int64_t)M * out_f / 4;
   const uint32_t nsum = (uint32_t)cdiv(mn4, 256);
   const RowsPrefetch none = {};
-  if (dtype == BLR_F16) hipLaunchKernelGGL(rows_sum_kernel<f16>, dim3(nsum), dim3(256), 0, st, (const f16*)ws, (f16*)out, bi, mn4, none, nsum);
-  else hipLaunchKernelGGL(rows_sum_kernel<bf16>, dim3(nsum), dim3(256), 0, st, (const bf16*)ws, (bf16*)out, bi, mn4, none, nsum);
+  if (dtype == BLR_F16) hipLaunchKernelGGL(rows_sum_kernel<f16>, dim3(nsum), dim3(256), 0, st, (const float*)ws, (f16*)out, bi, mn4, none, nsum);
+  else hipLaunchKernelGGL(rows_sum_kernel<bf16>, dim3(nsum), dim3(256), 0, st, (const float*)ws, (bf16*)out, bi, mn4, none, nsum);
   BLR_CHECK_LAUNCH("rows_sum");
   return BLR_OK;
 }

@@ -409,6 +409,13 @@ __device__ __forceinline__ uint32_t ring_lds_addr(const void* p) {
   return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((void __attribute__((address_space(3)))*)(p)));
 }
 
+#ifdef BLR_TRACE
+__device__ unsigned long long g_trace_gemm[4096 * 8];
+#define TRG(i) do { if (threadIdx.x == 0 && blockIdx.x < 4096) g_trace_gemm[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define TRG(i) do {} while (0)
+#endif
+
 template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false, int NWV = 4, bool PARTIAL = false>
 __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m, int side_wgs) {
   constexpr int NA = ring_na<SHALLOW>(), NB = ring_nb<SHALLOW>();
@@ -426,6 +433,7 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
   const int tiles = tiles_m * tiles_n;
+  TRG(0);
   int u = blockIdx.x;
   if (side_wgs > 0) {                                // the first workgroups of the launch carry the side job, not a tile (behind the
     if (u < side_wgs) {                              // tiles, in the tail of the launch, they measured 2 % of a DiT-XL/2 forward slower)
@@ -570,6 +578,7 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   // in flight after A(0), B(0): A(1..NA-2), B(1..NB-2)
   __builtin_amdgcn_s_waitcnt(ring_vmcnt((NA - 2) * LA + (NB - 2) * LB));
   __builtin_amdgcn_s_barrier();
+  TRG(1);
   frags(0, 0, 0, 0);
   int ca = 0, cb = 0;                                // stages of tile t in the two rings
   for (int t = 0; t < KT; ++t) {
@@ -620,6 +629,7 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
     __builtin_amdgcn_sched_barrier(0);
   }
   __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
+  TRG(2);
   if (PARTIAL) {
     // fp32 partial sums of this slice, straight from the accumulators: an instruction stores two rows of 32 floats
     float* P = reinterpret_cast<float*>(g.C) + (int64_t)bt * g.sC;
@@ -652,6 +662,7 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
       }
     }
   __syncthreads();
+  TRG(3);
   if (g.cn != 1) {
     // interleaved columns (column n of batch bt is element n * cn + bt of the row): two-byte stores, lanes along n, so
     // that an instruction touches cn * 128 contiguous bytes; the other batches fill the gaps
@@ -677,6 +688,7 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
       }
     }
   }
+  TRG(4);
 }
 
 
@@ -1261,3 +1273,9 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
 }
 
 }  // namespace blr
+
+#ifdef BLR_TRACE
+extern "C" int blr_debug_trace_gemm(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(blr::g_trace_gemm), (size_t)n * 8, 0, hipMemcpyDeviceToHost);
+}
+#endif

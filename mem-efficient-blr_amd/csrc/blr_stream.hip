@@ -973,7 +973,7 @@ constexpr size_t CTRL_BYTES = 16384;          // barrier shards, finished counte
 constexpr int MAX_COUNTERS = 8192;
 
 struct WsLayout {
-  unsigned* ctrl; unsigned* counters; float* zb0; float* zb1; void* d2; float* buf0; float* buf1; float* part;
+  unsigned* ctrl; unsigned* counters; float* zb0; float* zb1; void* d2; void* plain; float* buf0; float* buf1; float* part;
 };
 constexpr size_t ZCAP_FLOATS = 256 * 1024;    // capacity of each fixed-place Z accumulation buffer (1 MiB)
 
@@ -1171,10 +1171,10 @@ int launch(StreamParams& p, int dtype, int split, hipStream_t st) {
 
 int target_items() { return wgs_per_cu() * (device_cus() > 0 ? device_cus() : 256); }
 
-// Workspace: [ctrl][counters][Z ping][Z pong][tagged pairs][buf0][buf1][partials]; everything before buf0 sits at
+// Workspace: [ctrl][counters][Z ping][Z pong][tagged pairs][plain scratch][buf0][buf1][partials]; everything before buf0 sits at
 // fixed offsets and must be zero before the first call (the kernels leave it consistent afterwards).
 size_t ws_total(size_t buf_elems, size_t part_elems) {
-  return CTRL_BYTES + MAX_COUNTERS * sizeof(unsigned) + 2 * ZCAP_FLOATS * 4 + decode2_region_bytes() +
+  return CTRL_BYTES + MAX_COUNTERS * sizeof(unsigned) + 2 * ZCAP_FLOATS * 4 + decode2_region_bytes() + decode2_plain_bytes() +
          align_up(buf_elems * 4, 256) * 2 + align_up(part_elems * 4, 256);
 }
 WsLayout ws_carve(void* ws, size_t buf_elems) {
@@ -1185,6 +1185,7 @@ WsLayout ws_carve(void* ws, size_t buf_elems) {
   l.zb0 = reinterpret_cast<float*>(p); p += ZCAP_FLOATS * 4;
   l.zb1 = reinterpret_cast<float*>(p); p += ZCAP_FLOATS * 4;
   l.d2 = p; p += decode2_region_bytes();
+  l.plain = p; p += decode2_plain_bytes();
   l.buf0 = reinterpret_cast<float*>(p); p += align_up(buf_elems * 4, 256);
   l.buf1 = reinterpret_cast<float*>(p); p += align_up(buf_elems * 4, 256);
   l.part = reinterpret_cast<float*>(p);
@@ -1219,7 +1220,7 @@ int stream_blast_launch(const StreamBlastArgs& a, hipStream_t st) {
   if (!a.ws || a.ws_bytes < need) { set_error("blast stream: workspace %zu < %zu", a.ws_bytes, need); return BLR_ERR_WORKSPACE; }
   WsLayout w = ws_carve(a.ws, (size_t)a.b * a.M * a.r);
   if (decode2_applicable(a) || a.rows_only) {
-    int rc = decode2_blast_launch(a, w.d2, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
+    int rc = decode2_blast_launch(a, w.d2, w.plain, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
     if (rc <= 0) return rc;                    // served (or failed); 1 = shape outside its tiling
   }
   if (a.rows_only) return BLR_ERR_UNSUPPORTED;
@@ -1324,7 +1325,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
         bl.x = a.x; bl.ldx = a.ldx; bl.U = a.W2; bl.V = a.W1; bl.S = nullptr; bl.out = a.out; bl.ldo = a.ldo;
         bl.M = a.M; bl.in_f = a.in_f; bl.out_f = a.out_f; bl.b = bi; bl.bo = 1; bl.r = a.r;
         bl.dtype = a.dtype; bl.u_layout = BLR_U_RQ; bl.s_layout = BLR_S_IJR; bl.wbits = 16;
-        const int rc = decode_rows_launch(bl, w.d2, decode2_region_bytes(), st);
+        const int rc = decode_rows_launch(bl, w.plain, decode2_plain_bytes(), st);
         if (rc != 1) return rc;
       }
     }
@@ -1353,7 +1354,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
         bl.M = a.M; bl.in_f = a.in_f; bl.out_f = a.out_f; bl.b = bi; bl.bo = 1; bl.r = a.r;
         bl.dtype = a.dtype; bl.u_layout = BLR_U_RQ; bl.s_layout = BLR_S_IJR; bl.wbits = 16;
         if (decode2_applicable(bl)) {
-          int rc = decode2_blast_launch(bl, w.d2, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
+          int rc = decode2_blast_launch(bl, w.d2, w.plain, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
           if (rc <= 0) return rc;
         }
       }
@@ -1388,7 +1389,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
     if (a.out_order == BLR_OUT_INTERLEAVED) { bl.out_bs = 1; bl.out_ns = a.b; }
     else { bl.out_bs = S; bl.out_ns = 1; }
     if (decode2_applicable(bl)) {
-      int rc = decode2_blast_launch(bl, w.d2, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
+      int rc = decode2_blast_launch(bl, w.d2, w.plain, w.ctrl + D2_EPOCH, w.ctrl + D2_ARRIVE, w.ctrl + BAR_ERR, st);
       if (rc <= 0) return rc;
     }
   }

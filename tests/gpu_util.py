@@ -44,3 +44,9 @@ def blast_inputs(b, p, q, r, lead, seed=0):
     Vt = rng.standard_normal((b, r, p)) / np.sqrt(r)
     S = rng.standard_normal((b, b, r))
     return x, U, Vt, S
+
+
+def ulp(ref, dtype):
+    """Spacing of dtype's numbers at |ref| (float64 numpy): 2^(e - 10) for fp16, 2^(e - 7) for bf16, normal range."""
+    a = np.maximum(np.abs(np.asarray(ref, dtype=np.float64)), 2.0 ** -14)
+    return 2.0 ** (np.floor(np.log2(a)) - {torch.float16: 10, torch.bfloat16: 7}[dtype])

@@ -169,3 +169,23 @@ def test_wait_that_gives_up_is_reported_and_leaves_the_workspace_usable(case):
         out = fn()
         assert torch.equal(out, good), f"call {rep} after the give-up differs from the result before it"
     assert L.workspace_status(ws) == 0
+
+
+def test_single_launch_and_multi_launch_calls_alternate_on_one_workspace():
+    """One row of the Llama-7B gate_up layer runs the single-launch kernel, whose workgroups hand values to each other as
+    {value, call epoch} pairs in a block of the workspace; four and sixteen rows run several launches with plain
+    intermediates, which live in a block of their own, so that no plain value can ever be taken for a tagged one.  The
+    three alternate on one workspace; every call is checked against the oracle once and bit for bit afterwards."""
+    dtype = torch.float16
+    cases = {f"gate_up_m{M}": _blast_case(16, 256, 1376, 1024, M, "triton_blast_full_fp16", dtype, 20 + M) for M in (1, 4, 16)}
+    first = {}
+    for rep in range(12):
+        for k in cases:
+            fn, ref = cases[k]
+            out = fn()
+            if k not in first:
+                say(f"[case] alternating {k}")
+                assert_close(out, ref.reshape(tuple(out.shape)), dtype, k)
+                first[k] = out.clone()
+            else:
+                assert torch.equal(out, first[k]), f"{k}: call {rep} differs from the first call"

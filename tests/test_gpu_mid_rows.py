@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import blr_oracle as O
-from gpu_util import assert_close, blast_inputs, dev, rounded, say
+from gpu_util import assert_close, back, blast_inputs, dev, rounded, say, ulp
 
 pytestmark = pytest.mark.gpu
 
@@ -92,8 +92,7 @@ def test_monarch(name, M, shape):
 @pytest.mark.parametrize("M", [17, 64, 128])
 @pytest.mark.parametrize("shape", [(512, 200), (4096, 1024), (2752, 264)], ids=lambda s: "in%d-out%d" % s)
 def test_dense(shape, M, dtype):
-    """One slice (in_f <= 1024), four slices of 1024 and four of 688: the slices' partial products are rounded to the 16-bit
-    type before they are added, hence twice the tolerance."""
+    """One slice (in_f <= 1024), four slices of 1024 and four of 688 (fp32 partial sums, added by a second launch)."""
     from triton_funcs import dense_kernels as D, _lib as L
     in_f, out_f = shape
     rng = np.random.default_rng(70 + M)
@@ -101,9 +100,55 @@ def test_dense(shape, M, dtype):
     say(f"[case] mid rows dense M={M} in={in_f} out={out_f} {dtype}")
     out = D.triton_dense_fp16(dev(x, dtype), dev(w, dtype))
     ref = rounded(x, dtype) @ rounded(w, dtype)
-    assert_close(out, ref, dtype, f"dense M={M}", scale=2.0)
+    assert_close(out, ref, dtype, f"dense M={M}")
     bias = rng.standard_normal(out_f)
     with L.fused_epilogue(dev(bias, dtype), "gelu_tanh"):
         out = D.triton_dense_fp16(dev(x, dtype), dev(w, dtype))
     v = ref + rounded(bias, dtype)
-    assert_close(out, 0.5 * v * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (v + 0.044715 * v ** 3))), dtype, f"dense M={M} + bias + gelu", scale=2.0)
+    assert_close(out, 0.5 * v * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (v + 0.044715 * v ** 3))), dtype, f"dense M={M} + bias + gelu")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4096, 1024), (11008, 256)], ids=lambda s: "in%d-out%d" % s)
+def test_dense_slices_are_rounded_once(shape, dtype):
+    """The reduction of a dense layer at 17..128 rows is cut into slices (4 x 1024, 16 x 688).  Their partial sums stay in
+    fp32 and the result is rounded once, as a single-pass product does (reference triton_funcs/dense_kernels.py:80-98:
+    fp32 accumulator, one cast): every element within one unit in the last place of the fp64 result, plus the error of
+    fp32 accumulation (1e-6 of the sum of the terms' magnitudes)."""
+    from triton_funcs import dense_kernels as D
+    in_f, out_f = shape
+    M = 64
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((M, in_f)); w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)
+    say(f"[case] dense slices rounded once in={in_f} out={out_f} {dtype}")
+    got = back(D.triton_dense_fp16(dev(x, dtype), dev(w, dtype)))
+    xr, wr = rounded(x, dtype), rounded(w, dtype)
+    ref = xr @ wr
+    bound = 1.0 * ulp(ref, dtype) + 1e-6 * (np.abs(xr) @ np.abs(wr))
+    worst = (np.abs(got - ref) / bound).max()
+    assert worst <= 1.0, f"dense {in_f}->{out_f} {dtype}: worst element {worst:.2f} x its bound"
+
+
+def test_slices_whose_partial_sums_leave_the_fp16_range():
+    """Partial sums of +80000 and -75000 (neither is an fp16 number) whose total, 5000-odd, is: the sliced paths must not
+    overflow where a single-pass product does not.  Dense at 64 rows (4 slices of 1024) and low rank at 2 and 64 rows (16
+    slices of 256 rows of A)."""
+    from triton_funcs import dense_kernels as D, low_rank_kernels as K
+    dtype = torch.float16
+    in_f, out_f, M = 4096, 256, 64
+    x = np.ones((M, in_f))
+    w = np.zeros((in_f, out_f))
+    w[:1024] = 80000.0 / 1024; w[1024:2048] = -75000.0 / 1024; w[2048:3072] = 0.25; w[3072:] = -0.125
+    say("[case] dense slices beyond the fp16 range")
+    got = back(D.triton_dense_fp16(dev(x, dtype), dev(w, dtype)))
+    ref = rounded(x, dtype) @ rounded(w, dtype)
+    assert np.isfinite(got).all() and np.abs(got - ref).max() <= ulp(ref, dtype).max()
+    r = 64
+    a = np.zeros((in_f, r)); a[:256] = 80000.0 / 256; a[256:512] = -75000.0 / 256; a[512:] = 1.0 / 64
+    bm = np.eye(r, out_f) / 8.0
+    for rows in (2, 64):
+        say(f"[case] low rank slices beyond the fp16 range, {rows} rows")
+        got = back(K.triton_low_rank_fp16(dev(x[:rows], dtype), dev(a, dtype), dev(bm, dtype)))
+        z = rounded(rounded(x[:rows], dtype) @ rounded(a, dtype), dtype)
+        ref = z @ rounded(bm, dtype)
+        assert np.isfinite(got).all() and np.abs(got - ref).max() <= ulp(ref, dtype).max()
