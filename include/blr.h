@@ -65,8 +65,11 @@ typedef enum { BLR_W2_SR = 0, BLR_W2_RS = 1 } blr_w2_layout;
  * out[n, ll*S + s] of the right_ideal names (reference triton_funcs/monarch_kernels.py:1004). */
 typedef enum { BLR_OUT_INTERLEAVED = 0, BLR_OUT_BLOCKED = 1 } blr_monarch_out;
 
-/* Activation of the fused output stage (the *_fwd_ep entry points). */
-typedef enum { BLR_ACT_NONE = 0, BLR_ACT_GELU_TANH = 1, BLR_ACT_SILU = 2 } blr_act;
+/* Activation of the fused output stage (the *_fwd_ep entry points).  BLR_ACT_SILU_MUL is the gated unit of Llama's MLP over a
+ * fused gate|up projection (reference configs/layers/llama7b.gate_up_proj.yaml:1-8: 4096 -> 22016 = gate | up): with
+ * y = op(x) + bias and h = out_f / 2, out[m, c] = silu(y[m, c]) * y[m, c + h] - out then has h columns (ldo >= h). */
+typedef enum { BLR_ACT_NONE = 0, BLR_ACT_GELU_TANH = 1, BLR_ACT_SILU = 2, BLR_ACT_SILU_MUL = 3 } blr_act;
+typedef enum { BLR_OP_BLAST = 0, BLR_OP_MONARCH = 1, BLR_OP_LOW_RANK = 2, BLR_OP_DENSE = 3 } blr_op;
 
 /* ---- workspaces ---------------------------------------------------------------------------
  * Every *_fwd entry point takes a caller-owned workspace of at least blr_*_workspace_bytes(...) bytes
@@ -213,6 +216,13 @@ int blr_blast_fwd_ep(const void* x, int64_t ldx, const void* U, const void* V, c
                      void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
                      int dtype, int u_layout, int s_layout, int algo,
                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act);
+/* BLR_ACT_SILU_MUL (no reference kernel: SURVEY of the callers' step after the path - Llama's act(gate) * up): above 128 rows
+ * of f16 / bf16, BLAST (even b), low rank and dense compute the tiles of the gate half and of the up half of an output position
+ * in one work item of the last GEMM and write only the product, so the (M, out_f) intermediate never exists; everything else
+ * (few rows, Monarch, fp32) computes the full-width result into the TAIL of the workspace and finishes with one elementwise
+ * launch.  blr_ep_workspace_bytes: bytes to ADD to blr_*_workspace_bytes() for such a call (0 when the GEMM fuses it, and for
+ * every other activation); op: blr_op; b: BLAST's number of blocks (ignored otherwise).                                      */
+size_t blr_ep_workspace_bytes(int op, int M, int out_f, int b, int dtype, int act);
 int blr_monarch_fwd_ep(const void* x, int64_t ldx, const void* w1, const void* w2,
                        void* out, int64_t ldo, int M, int in_f, int out_f, int b, int rank,
                        int dtype, int w2_layout, int out_order, int algo,

@@ -166,8 +166,10 @@ static int quantize_t(const void* w, int64_t outer, int64_t reduce, int64_t inne
 struct PendingEpilogue { const void* bias; int act; bool armed; bool used; const void* gate; int gate_rows; int64_t ld_gate; const void* resid; int64_t ld_resid; };
 static thread_local PendingEpilogue tl_ep = {nullptr, 0, false, false, nullptr, 0, 0, nullptr, 0};
 
+static bool silu_mul_armed() { return tl_ep.armed && tl_ep.act == BLR_ACT_SILU_MUL; }
+
 bool epilogue_pending(const void** bias, int* act) {
-  if (!tl_ep.armed || tl_ep.used || tl_ep.gate || tl_ep.resid) return false;
+  if (!tl_ep.armed || tl_ep.used || tl_ep.gate || tl_ep.resid || tl_ep.act == BLR_ACT_SILU_MUL) return false;
   *bias = tl_ep.bias; *act = tl_ep.act;
   return true;
 }
@@ -176,6 +178,7 @@ void epilogue_taken() { tl_ep.used = true; }
 static void attach_epilogue_peek(GemmArgs& g) {      // the armed output stage, without claiming it
   if (!tl_ep.armed) return;
   g.bias = tl_ep.bias; g.act = tl_ep.act;
+  if (tl_ep.act == BLR_ACT_SILU_MUL) { g.act = BLR_ACT_SILU; g.pair = 1; }   // (the caller sets the distances between the halves)
   g.gate = tl_ep.gate; g.gate_rows = tl_ep.gate_rows; g.ld_gate = tl_ep.ld_gate; g.resid = tl_ep.resid; g.ld_resid = tl_ep.ld_resid;
 }
 static void attach_epilogue(GemmArgs& g) {
@@ -211,18 +214,73 @@ static int bias_act_launch(void* out, int64_t ldo, const PendingEpilogue& ep, in
   return BLR_OK;
 }
 
-// Runs `call` (a plain entry point) with the epilogue armed and finishes whatever the call did not fuse.
+// out[m][c] = silu(y[m][c] + bias[c]) * (y[m][c + h] + bias[c + h]) over a full-width result y (M, 2 h): the gated unit of
+// Llama's MLP where no kernel fuses it.  Rounding points as in the fused form: both factors are rounded to T, then their product.
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ y, int64_t ldy, const T* __restrict__ bias, T* __restrict__ out, int64_t ldo, int M, int h) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * h) return;
+  const int m = (int)(idx / h), c = (int)(idx - (int64_t)m * h);
+  float g = TypeTraits<T>::to_f32(y[(int64_t)m * ldy + c]), u = TypeTraits<T>::to_f32(y[(int64_t)m * ldy + c + h]);
+  if (bias) { g += TypeTraits<T>::to_f32(bias[c]); u += TypeTraits<T>::to_f32(bias[c + h]); }
+  const T gt = TypeTraits<T>::from_f32(apply_act(g, BLR_ACT_SILU)), ut = TypeTraits<T>::from_f32(u);
+  out[(int64_t)m * ldo + c] = TypeTraits<T>::from_f32(TypeTraits<T>::to_f32(gt) * TypeTraits<T>::to_f32(ut));
+}
+
+static int silu_mul_launch(const void* y, int64_t ldy, const void* bias, void* out, int64_t ldo, int M, int h, int dtype, hipStream_t st) {
+  const unsigned grid = (unsigned)cdiv((int64_t)M * h, 256);
+  if (dtype == BLR_F16) hipLaunchKernelGGL(silu_mul_kernel<f16>, dim3(grid), dim3(256), 0, st, (const f16*)y, ldy, (const f16*)bias, (f16*)out, ldo, M, h);
+  else if (dtype == BLR_BF16) hipLaunchKernelGGL(silu_mul_kernel<bf16>, dim3(grid), dim3(256), 0, st, (const bf16*)y, ldy, (const bf16*)bias, (bf16*)out, ldo, M, h);
+  else hipLaunchKernelGGL(silu_mul_kernel<float>, dim3(grid), dim3(256), 0, st, (const float*)y, ldy, (const float*)bias, (float*)out, ldo, M, h);
+  BLR_CHECK_LAUNCH("silu_mul");
+  return BLR_OK;
+}
+
+// BLR_ACT_SILU_MUL is fused into the write-out of the last GEMM (pairs of tiles) for BLAST with an even number of blocks, low
+// rank and dense above 128 rows of f16 / bf16; everything else computes the full-width result into the tail of the workspace
+// and finishes with silu_mul_kernel.
+static bool silu_mul_fused(int op, int M, int out_f, int dtype, int b) {
+  if (dtype == BLR_F32 || M <= 128 || out_f % 16) return false;
+  if (op == BLR_OP_BLAST) return b % 2 == 0;
+  return op == BLR_OP_LOW_RANK || op == BLR_OP_DENSE;
+}
+static size_t silu_mul_scratch(int op, int M, int out_f, int dtype, int b) {
+  return silu_mul_fused(op, M, out_f, dtype, b) ? 0 : align_up((size_t)M * out_f * elt_size(dtype), 256);
+}
+
+// Runs `call(out, ldo, ws_bytes)` (a plain entry point) with the epilogue armed and finishes whatever the call did not fuse.
 struct GateResidual { const void* gate; int gate_rows; int64_t ld_gate; const void* resid; int64_t ld_resid; };
 template <typename F>
-static int with_epilogue(const void* bias, int act, void* out, int64_t ldo, int M, int out_f, int dtype, void* stream, F&& call,
-                         GateResidual gr = {nullptr, 0, 0, nullptr, 0}) {
-  if (act < BLR_ACT_NONE || act > BLR_ACT_SILU) { set_error("epilogue: unknown activation %d", act); return BLR_ERR_BAD_ARG; }
+static int with_epilogue(int op, int b, const void* bias, int act, void* out, int64_t ldo, int M, int out_f, int dtype, void* ws, size_t ws_bytes,
+                         void* stream, F&& call, GateResidual gr = {nullptr, 0, 0, nullptr, 0}) {
+  if (act < BLR_ACT_NONE || act > BLR_ACT_SILU_MUL) { set_error("epilogue: unknown activation %d", act); return BLR_ERR_BAD_ARG; }
+  if (act == BLR_ACT_SILU_MUL) {
+    if (gr.gate || gr.resid) { set_error("epilogue: BLR_ACT_SILU_MUL takes no gate and no residual"); return BLR_ERR_BAD_ARG; }
+    if (M <= 0 || out_f <= 0 || out_f % 2) { set_error("epilogue: BLR_ACT_SILU_MUL needs an even out_f (gate | up)"); return BLR_ERR_BAD_SHAPE; }
+    if (!out || ldo < out_f / 2) { set_error("epilogue: out of BLR_ACT_SILU_MUL has out_f / 2 columns; ldo too small"); return BLR_ERR_BAD_ARG; }
+    if (!dtype_ok(dtype)) { set_error("epilogue: bad dtype"); return BLR_ERR_BAD_ARG; }
+    const size_t extra = silu_mul_scratch(op, M, out_f, dtype, b);
+    if (extra) {                                        // full-width result in the tail of the workspace, then the elementwise kernel
+      if (!ws || ws_bytes < extra) { set_error("epilogue: BLR_ACT_SILU_MUL needs blr_ep_workspace_bytes() = %zu more bytes of workspace here", extra); return BLR_ERR_WORKSPACE; }
+      void* full = reinterpret_cast<char*>(ws) + (ws_bytes - extra) / 256 * 256;
+      tl_ep = {nullptr, 0, false, false, nullptr, 0, 0, nullptr, 0};
+      const int rc = call(full, (int64_t)out_f, (ws_bytes - extra) / 256 * 256);
+      if (rc != BLR_OK) return rc;
+      return silu_mul_launch(full, out_f, bias, out, ldo, M, out_f / 2, dtype, (hipStream_t)stream);
+    }
+    tl_ep = {bias, act, true, false, nullptr, 0, 0, nullptr, 0};
+    const int rc = call(out, ldo, ws_bytes);
+    const bool used = tl_ep.used;
+    tl_ep = {nullptr, 0, false, false, nullptr, 0, 0, nullptr, 0};
+    if (rc == BLR_OK && !used) { set_error("epilogue: BLR_ACT_SILU_MUL was not applied (internal error)"); return BLR_ERR_UNSUPPORTED; }
+    return rc;
+  }
   if (gr.gate && (gr.gate_rows <= 0 || gr.ld_gate < out_f)) { set_error("epilogue: gate needs gate_rows > 0 and ld_gate >= out_f"); return BLR_ERR_BAD_ARG; }
   if (gr.resid && gr.ld_resid < out_f) { set_error("epilogue: ld_resid < out_f"); return BLR_ERR_BAD_ARG; }
   const PendingEpilogue ep = {bias, act, bias != nullptr || act != BLR_ACT_NONE || gr.gate != nullptr || gr.resid != nullptr, false,
                               gr.gate, gr.gate_rows, gr.ld_gate, gr.resid, gr.ld_resid};
   tl_ep = ep;
-  const int rc = call();
+  const int rc = call(out, ldo, ws_bytes);
   const bool used = tl_ep.used, armed = tl_ep.armed;
   tl_ep = {nullptr, 0, false, false, nullptr, 0, 0, nullptr, 0};
   if (rc != BLR_OK || !armed || used) return rc;
@@ -349,7 +407,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   // kernels).  Up to 128 rows the three launches of the few-row path run over tiles of 16 rows with the weights held in registers
   // (at 128 rows 32 / 44 / 43 us against 39 / 48 / 56 us through the tiles on the three Llama-7B layers).
   static const int rows_max_m = getenv("BLR_TILED_ROWS_MAX_M") ? atoi(getenv("BLR_TILED_ROWS_MAX_M")) : 128;
-  if (M <= rows_max_m && !y_out && !z_out && !sat8 && fused <= 0 && dtype != BLR_F32) {
+  if (M <= rows_max_m && !y_out && !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && !silu_mul_armed()) {
     StreamBlastArgs s = {};
     s.x = x; s.ldx = ldx; s.U = U; s.V = V; s.S = S; s.out = out; s.ldo = ldo;
     s.M = M; s.in_f = in_f; s.out_f = out_f; s.b = b; s.r = r;
@@ -368,7 +426,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   // r = 288: 47 against 51 us.  BLR_BLAST_MIXU: 0 never, 1 only where the first half would not be fused anyway, 2 (default)
   // wherever the kernel takes the shape.
   static const int mixu_mode = getenv("BLR_BLAST_MIXU") ? atoi(getenv("BLR_BLAST_MIXU")) : 2;
-  const bool mixu_shape = !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && b == 16 && Q % 8 == 0 && Q <= 80 && r % 32 == 0;
+  const bool mixu_shape = !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && b == 16 && Q % 8 == 0 && Q <= 80 && r % 32 == 0 && !silu_mul_armed();
   // Narrow input blocks as well (at most 96 columns): the whole call is one launch that forms Y per step of the rank walk in the
   // compute unit and keeps neither Y nor Z in memory (blast_one_kernel).  BLR_BLAST_ONE=0 switches it off.
   static const int one_mode = getenv("BLR_BLAST_ONE") ? atoi(getenv("BLR_BLAST_ONE")) : 1;
@@ -415,6 +473,10 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   g2.C = out; g2.ldc = ldo; g2.sC = Q; g2.cn = 1;
   g2.M = M; g2.N = Q; g2.K = r; g2.batch = b;
   if (!sat8) attach_epilogue(g2);
+  if (g2.pair) {                                    // silu(gate) * up: output blocks i and i + b/2 as the two tiles of a work item
+    if (sat8 || b % 2) { set_error("blast: BLR_ACT_SILU_MUL needs an even number of blocks"); return BLR_ERR_UNSUPPORTED; }
+    g2.batch = b / 2; g2.pair_dA = (int64_t)(b / 2) * g2.sA; g2.pair_dB = (int64_t)(b / 2) * g2.sB; g2.pair_dbias = (int64_t)(b / 2) * Q;
+  }
   if (mixu) {                                       // (Y is in memory: the branch above ran the GEMM and skipped the mix)
     rc = blast_mixu_launch(Y, S, U, out, ldo, g2, M, b, r, Q, si, sj, sr, s_layout, dtype, Z, ybytes, st, mixu_prepared != 0, u_layout == BLR_U_RQ);
     if (rc != 1) return rc;
@@ -434,7 +496,7 @@ int blr_blast_fwd(const void* x, int64_t ldx, const void* U, const void* V, cons
   if (!dtype_ok(dtype) || u_layout < 0 || u_layout > 1 || s_layout < 0 || s_layout > 2) { set_error("blast: bad enum"); return BLR_ERR_BAD_ARG; }
   int rc = check_blast_shape("blast", M, in_f, out_f, b, r);
   if (rc) return rc;
-  if (ldx < in_f || ldo < out_f) { set_error("blast: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  if (ldx < in_f || ldo < (silu_mul_armed() ? out_f / 2 : out_f)) { set_error("blast: leading dimension too small"); return BLR_ERR_BAD_ARG; }
   const int P = in_f / b, Q = out_f / b;
   int a = resolve_algo(algo, M, dtype, z_out || y_out);
   if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
@@ -674,7 +736,7 @@ int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
   if (!x || !A || !B || !out) { set_error("low_rank: null pointer"); return BLR_ERR_BAD_ARG; }
   if (!dtype_ok(dtype)) { set_error("low_rank: bad dtype"); return BLR_ERR_BAD_ARG; }
   if (M <= 0 || in_f <= 0 || out_f <= 0 || r <= 0) { set_error("low_rank: non-positive size"); return BLR_ERR_BAD_ARG; }
-  if (ldx < in_f || ldo < out_f) { set_error("low_rank: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  if (ldx < in_f || ldo < (silu_mul_armed() ? out_f / 2 : out_f)) { set_error("low_rank: leading dimension too small"); return BLR_ERR_BAD_ARG; }
   int a = resolve_algo(algo, M, dtype, z_out != nullptr);
   if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
     if (dtype == BLR_F32 || M > 16 || z_out) { set_error("low_rank: streaming algorithm needs f16/bf16, M <= 16, no intermediates"); return BLR_ERR_UNSUPPORTED; }
@@ -707,6 +769,7 @@ int blr_low_rank_fwd(const void* x, int64_t ldx, const void* A, const void* B,
   g2.A = Z; g2.lda = r; g2.B = B; g2.ldb = out_f; g2.b_kn = 1;
   g2.C = out; g2.ldc = ldo; g2.cn = 1; g2.M = M; g2.N = out_f; g2.K = r; g2.batch = 1;
   attach_epilogue(g2);
+  if (g2.pair) { g2.N = out_f / 2; g2.pair_dA = 0; g2.pair_dB = out_f / 2; g2.pair_dbias = out_f / 2; }   // columns n and n + out_f / 2 of B
   return gemm_launch(g2, dtype, st);
 }
 
@@ -727,7 +790,7 @@ int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t 
   if (!x || !W || !out) { set_error("dense: null pointer"); return BLR_ERR_BAD_ARG; }
   if (!dtype_ok(dtype)) { set_error("dense: bad dtype"); return BLR_ERR_BAD_ARG; }
   if (M <= 0 || in_f <= 0 || out_f <= 0) { set_error("dense: non-positive size"); return BLR_ERR_BAD_ARG; }
-  if (ldx < in_f || ldo < out_f) { set_error("dense: leading dimension too small"); return BLR_ERR_BAD_ARG; }
+  if (ldx < in_f || ldo < (silu_mul_armed() ? out_f / 2 : out_f)) { set_error("dense: leading dimension too small"); return BLR_ERR_BAD_ARG; }
   int a = resolve_algo(algo, M, dtype, false);
   if (a == BLR_ALGO_STREAM || a == BLR_ALGO_STREAM_SPLIT) {
     if (dtype == BLR_F32 || M > 16) { set_error("dense: streaming algorithm needs f16/bf16 and M <= 16"); return BLR_ERR_UNSUPPORTED; }
@@ -750,42 +813,42 @@ int blr_dense_fwd(const void* x, int64_t ldx, const void* W, void* out, int64_t 
   // few output tiles and a long reduction (11008 -> 4096 at 256 rows: 32 tiles): room to cut it along K
   if (ws && gemm_splitk_bytes(M, out_f, in_f, dtype) && ws_bytes >= gemm_splitk_bytes(M, out_f, in_f, dtype)) { g.splitk_ws = ws; g.splitk_bytes = ws_bytes; }
   attach_epilogue(g);
+  if (g.pair) { g.N = out_f / 2; g.pair_dA = 0; g.pair_dB = out_f / 2; g.pair_dbias = out_f / 2; g.splitk_ws = nullptr; g.splitk_bytes = 0; }
   return gemm_launch(g, dtype, st);
 }
 
 // ---- fused output stage: out = act(op(x) + bias) ------------------------------------------------------
+size_t blr_ep_workspace_bytes(int op, int M, int out_f, int b, int dtype, int act) {
+  if (act != BLR_ACT_SILU_MUL || M <= 0 || out_f <= 0 || !dtype_ok(dtype)) return 0;
+  return silu_mul_scratch(op, M, out_f, dtype, b);
+}
+
 int blr_blast_fwd_ep(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
                      void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
                      int dtype, int u_layout, int s_layout, int algo,
                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act) {
-  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
-    return blr_blast_fwd(x, ldx, U, V, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, u_layout, s_layout, algo, ws, ws_bytes, stream);
-  });
+  return blr_blast_fwd_ep2(x, ldx, U, V, S, out, ldo, M, in_f, out_f, b, r, dtype, u_layout, s_layout, algo, ws, ws_bytes, stream, bias, act,
+                           nullptr, 0, 0, nullptr, 0);
 }
 
 int blr_monarch_fwd_ep(const void* x, int64_t ldx, const void* w1, const void* w2,
                        void* out, int64_t ldo, int M, int in_f, int out_f, int b, int rank,
                        int dtype, int w2_layout, int out_order, int algo,
                        void* ws, size_t ws_bytes, void* stream, const void* bias, int act) {
-  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
-    return blr_monarch_fwd(x, ldx, w1, w2, out, ldo, nullptr, M, in_f, out_f, b, rank, dtype, w2_layout, out_order, algo, ws, ws_bytes, stream);
-  });
+  return blr_monarch_fwd_ep2(x, ldx, w1, w2, out, ldo, M, in_f, out_f, b, rank, dtype, w2_layout, out_order, algo, ws, ws_bytes, stream, bias, act,
+                             nullptr, 0, 0, nullptr, 0);
 }
 
 int blr_low_rank_fwd_ep(const void* x, int64_t ldx, const void* A, const void* B,
                         void* out, int64_t ldo, int M, int in_f, int out_f, int r, int dtype, int algo,
                         void* ws, size_t ws_bytes, void* stream, const void* bias, int act) {
-  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
-    return blr_low_rank_fwd(x, ldx, A, B, out, ldo, nullptr, M, in_f, out_f, r, dtype, algo, ws, ws_bytes, stream);
-  });
+  return blr_low_rank_fwd_ep2(x, ldx, A, B, out, ldo, M, in_f, out_f, r, dtype, algo, ws, ws_bytes, stream, bias, act, nullptr, 0, 0, nullptr, 0);
 }
 
 int blr_dense_fwd_ep(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo,
                      int M, int in_f, int out_f, int dtype, int algo,
                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act) {
-  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
-    return blr_dense_fwd(x, ldx, W, out, ldo, M, in_f, out_f, dtype, algo, ws, ws_bytes, stream);
-  });
+  return blr_dense_fwd_ep2(x, ldx, W, out, ldo, M, in_f, out_f, dtype, algo, ws, ws_bytes, stream, bias, act, nullptr, 0, 0, nullptr, 0);
 }
 
 // ---- the same with a gate and a residual: out = resid + gate[row group] * act(op(x) + bias) -------------------------------------
@@ -794,8 +857,8 @@ int blr_blast_fwd_ep2(const void* x, int64_t ldx, const void* U, const void* V, 
                       int dtype, int u_layout, int s_layout, int algo,
                       void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
                       const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid) {
-  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
-    return blr_blast_fwd(x, ldx, U, V, S, out, ldo, nullptr, nullptr, M, in_f, out_f, b, r, dtype, u_layout, s_layout, algo, ws, ws_bytes, stream);
+  return with_epilogue(BLR_OP_BLAST, b, bias, act, out, ldo, M, out_f, dtype, ws, ws_bytes, stream, [&](void* o, int64_t ld, size_t wsb) {
+    return blr_blast_fwd(x, ldx, U, V, S, o, ld, nullptr, nullptr, M, in_f, out_f, b, r, dtype, u_layout, s_layout, algo, ws, wsb, stream);
   }, {gate, gate_rows, ld_gate, resid, ld_resid});
 }
 
@@ -804,8 +867,8 @@ int blr_monarch_fwd_ep2(const void* x, int64_t ldx, const void* w1, const void* 
                         int dtype, int w2_layout, int out_order, int algo,
                         void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
                         const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid) {
-  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
-    return blr_monarch_fwd(x, ldx, w1, w2, out, ldo, nullptr, M, in_f, out_f, b, rank, dtype, w2_layout, out_order, algo, ws, ws_bytes, stream);
+  return with_epilogue(BLR_OP_MONARCH, b, bias, act, out, ldo, M, out_f, dtype, ws, ws_bytes, stream, [&](void* o, int64_t ld, size_t wsb) {
+    return blr_monarch_fwd(x, ldx, w1, w2, o, ld, nullptr, M, in_f, out_f, b, rank, dtype, w2_layout, out_order, algo, ws, wsb, stream);
   }, {gate, gate_rows, ld_gate, resid, ld_resid});
 }
 
@@ -813,8 +876,8 @@ int blr_low_rank_fwd_ep2(const void* x, int64_t ldx, const void* A, const void* 
                          void* out, int64_t ldo, int M, int in_f, int out_f, int r, int dtype, int algo,
                          void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
                          const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid) {
-  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
-    return blr_low_rank_fwd(x, ldx, A, B, out, ldo, nullptr, M, in_f, out_f, r, dtype, algo, ws, ws_bytes, stream);
+  return with_epilogue(BLR_OP_LOW_RANK, 1, bias, act, out, ldo, M, out_f, dtype, ws, ws_bytes, stream, [&](void* o, int64_t ld, size_t wsb) {
+    return blr_low_rank_fwd(x, ldx, A, B, o, ld, nullptr, M, in_f, out_f, r, dtype, algo, ws, wsb, stream);
   }, {gate, gate_rows, ld_gate, resid, ld_resid});
 }
 
@@ -822,8 +885,8 @@ int blr_dense_fwd_ep2(const void* x, int64_t ldx, const void* W, void* out, int6
                       int M, int in_f, int out_f, int dtype, int algo,
                       void* ws, size_t ws_bytes, void* stream, const void* bias, int act,
                       const void* gate, int gate_rows, int64_t ld_gate, const void* resid, int64_t ld_resid) {
-  return with_epilogue(bias, act, out, ldo, M, out_f, dtype, stream, [&] {
-    return blr_dense_fwd(x, ldx, W, out, ldo, M, in_f, out_f, dtype, algo, ws, ws_bytes, stream);
+  return with_epilogue(BLR_OP_DENSE, 1, bias, act, out, ldo, M, out_f, dtype, ws, ws_bytes, stream, [&](void* o, int64_t ld, size_t wsb) {
+    return blr_dense_fwd(x, ldx, W, o, ld, M, in_f, out_f, dtype, algo, ws, wsb, stream);
   }, {gate, gate_rows, ld_gate, resid, ld_resid});
 }
 

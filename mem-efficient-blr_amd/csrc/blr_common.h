@@ -152,6 +152,11 @@ struct GemmArgs {
   int act;          // blr_act applied after the bias
   const void* gate; int gate_rows; int64_t ld_gate;   // optional: after the activation, the value is multiplied by gate[(m / gate_rows) * ld_gate + offset in row]
   const void* resid; int64_t ld_resid;   // optional: and resid[m * ld_resid + offset in row] is added (DiT: x + g * h, reference DiT/models.py:120-121)
+  // pair: every work item computes two tiles one after the other - the same rows and columns of two problems whose operands lie
+  // pair_dA / pair_dB elements apart (BLAST: output blocks i and i + b/2; dense and low rank: the columns n and n + N of a factor
+  // with 2 N columns) - and writes ONE tile of C: silu(first + bias[..]) * (second + bias[.. + pair_dbias]), the gated unit of
+  // Llama's MLP over a fused gate|up projection.  N, batch and C describe one half.  Ring kernels with an output stage only.
+  int pair; int64_t pair_dA, pair_dB, pair_dbias;
   void* splitk_ws;  // optional scratch for splitting the reduction (gemm_splitk_bytes says how much); null: never split
   size_t splitk_bytes;
   int kc;           // set by gemm_launch for the split kernels: k values per slice

@@ -202,6 +202,23 @@ __device__ __forceinline__ typename TypeTraits<T>::vec8 ep_vector(const GemmArgs
   return r;
 }
 
+// Second tile of a pair: (r + bias) rounded to T, times the first tile's result, which the same thread stored at `c` before.
+template <typename T>
+__device__ __forceinline__ typename TypeTraits<T>::vec8 ep_pair_up(const GemmArgs& g, typename TypeTraits<T>::vec8 r, int64_t in_row, const T* c) {
+  using V8 = typename TypeTraits<T>::vec8;
+  V8 bv;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) bv[e] = (T)0.0f;
+  if (g.bias) bv = *reinterpret_cast<const V8*>(reinterpret_cast<const T*>(g.bias) + in_row);
+  const V8 gv = *reinterpret_cast<const V8*>(c);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const T up = TypeTraits<T>::from_f32(TypeTraits<T>::to_f32(r[e]) + TypeTraits<T>::to_f32(bv[e]));
+    r[e] = TypeTraits<T>::from_f32(TypeTraits<T>::to_f32(gv[e]) * TypeTraits<T>::to_f32(up));
+  }
+  return r;
+}
+
 template <typename T, int BM, int BN, bool B_KN, int PD, bool EP = false>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int a_vec, int b_vec, int c_vec,
                                                         int per_xcd, int group_m) {
@@ -454,9 +471,16 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   const int tm_i = strip * group_m + rem % gm_here, tn_i = rem / gm_here;
   const int m0 = tm_i * BM, n0 = tn_i * BN;
 
-  const char* Ab = reinterpret_cast<const char*>(g.A) + (int64_t)bt * g.sA * 2;
-  const char* Bb = reinterpret_cast<const char*>(g.B) + (int64_t)bt * g.sB * 2;
+  const char* Ab0 = reinterpret_cast<const char*>(g.A) + (int64_t)bt * g.sA * 2;
+  const char* Bb0 = reinterpret_cast<const char*>(g.B) + (int64_t)bt * g.sB * 2;
   T* C = reinterpret_cast<T*>(g.C);
+  // A pair of tiles (kernels with an output stage only): the second runs the same code on operands pair_dA / pair_dB further on
+  // (not the 256 x 256 tile on four waves: it has no register left for the loop)
+  constexpr bool PAIRS = EP && !PARTIAL && !(BM == 256 && BN == 256 && NWV == 4);
+  const int halves = (PAIRS && g.pair) ? 2 : 1;
+  for (int hf = 0; hf < halves; ++hf) {
+  const char* Ab = Ab0 + (PAIRS ? (int64_t)hf * g.pair_dA * 2 : 0);
+  const char* Bb = Bb0 + (PAIRS ? (int64_t)hf * g.pair_dB * 2 : 0);
 
   // PARTIAL: the batch index counts slices of the reduction (g.kc values of k each, the last one what is left of g.K)
   const int Kloc = PARTIAL ? min(g.kc, g.K - bt * g.kc) : g.K;
@@ -679,7 +703,12 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
     const int gr = m0 + row, gc = n0 + cvec;
     if (gr < g.M && gc < g.N) {
       V8 v = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
-      if (EP) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc, gr);
+      if (EP) {
+        // (a pair: the first tile leaves silu(. + bias) where the result goes; the second is multiplied onto it by the thread that
+        // stored it - the same element index v in both passes)
+        if (!PAIRS || hf == 0) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc, gr);
+        else v = ep_pair_up<T>(g, v, (int64_t)bt * g.sC + gc + g.pair_dbias, &C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]);
+      }
       if (g.epi == EPI_MONARCH_SCATTER) {            // column c of entry bt -> block c / per, column bt * per + c % per
         const int d = gc / g.per;
         *reinterpret_cast<V8*>(&C[(int64_t)d * g.sL + (int64_t)gr * g.ldc + (int64_t)bt * g.per + (gc - d * g.per)]) = v;
@@ -688,6 +717,8 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
       }
     }
   }
+  if (hf + 1 < halves) __syncthreads();              // the staged tile has been read: the rings may be filled again
+  }  // tiles of a pair
   TRG(4);
 }
 
@@ -932,7 +963,11 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       return BLR_OK;
     }
   }
-  if (ring > 0 && force == 0 && ring_ok(g)) {
+  if (g.pair && (!ring_ok(g) || g.epi != EPI_PLAIN || g.cn != 1 || g.sat8 || g.gate || g.resid || g.pair_dA % 8 || g.pair_dB % 8 || g.pair_dbias % 8 || !aligned(g.C, 16))) {
+    set_error("gemm: a pair of tiles (SiLU-gated halves) needs 16-byte aligned operands, K and the half width multiples of 8, a plain row-major output");
+    return BLR_ERR_UNSUPPORTED;
+  }
+  if ((ring > 0 && force == 0 && ring_ok(g)) || g.pair) {
     int rt = option_value(OPT_GEMM_RING_TILE, 0);
     const int64_t fill = ((int64_t)cus * 9 + 9) / 10;
     const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
@@ -955,12 +990,13 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       else if (g.N <= 128 && g.K <= 1024 && r128 >= fill) rt = 128128;
       else if (t256 >= fill) rt = 256256;
       else if (t128 >= fill) rt = 256128;
-      else if (r128 >= fill || ring > 1) rt = 128128;
+      else if (r128 >= fill || ring > 1 || g.pair) rt = 128128;
     }
-    if (rt > 0 && (ring > 1 || (g.M >= 96 && g.K >= 64))) {
+    if (g.pair && rt <= 0) rt = 128128;
+    if (rt > 0 && (ring > 1 || g.pair || (g.M >= 96 && g.K >= 64))) {
       if (rt == 256256) {
         // eight waves (2 x 4, wave tile 128 x 64, two per SIMD) hide each other's barrier and LDS waits: the default
-        return option_value(OPT_GEMM_RING_WAVES, 8) == 4 ? launch_ring<T, 256, 256>(g, st) : launch_ring<T, 256, 256, false, 8>(g, st);
+        return option_value(OPT_GEMM_RING_WAVES, 8) == 4 && !g.pair ? launch_ring<T, 256, 256>(g, st) : launch_ring<T, 256, 256, false, 8>(g, st);
       }
       if (rt == 256128) {
         if (per_cu != 2 && option_value(OPT_GEMM_RING_WAVES, 4) == 8) return launch_ring<T, 256, 128, false, 8>(g, st);

@@ -9,7 +9,8 @@ exactly as in the reference:
   Monarch "left" in name -> w2 (b, r, s), else (b, s, r); w1 (b, p, r)
 The bias is added as `out += bias.to(x.dtype)` (reference wrappers.py:176-177); with a library kernel
 ("triton" names other than the quantized one) the bias - and an activation the owner of the module asks
-for by setting `fused_act` ("gelu_tanh" or "silu") - is handed to the kernel's output stage instead.
+for by setting `fused_act` ("gelu_tanh", "silu", or "silu_mul": silu(gate) * up over a fused gate|up projection, whose result
+has out_features / 2 columns) - is handed to the kernel's output stage instead.
 Factors are drawn with std 1/sqrt(fan-in of the factor) instead of the reference's std 1, so that
 fp16 activations stay in range at the ranks the networks use.
 """
@@ -40,7 +41,10 @@ class _StructuredLinear(nn.Module):
         else:
             self.register_parameter("bias", None)
         self.fused_act = None          # set by the owner (e.g. an MLP) to have its activation applied by the kernel
-        self.fuses = self.kind == "triton" and not is_compiled and "int8" not in self.func_name and "int4" not in self.func_name
+        # (the *_fp32 verification names return their intermediates and never read an armed output stage: bias and activation
+        # are applied here for them, as for the torch baselines)
+        self.fuses = (self.kind == "triton" and not is_compiled and "int8" not in self.func_name and "int4" not in self.func_name
+                      and "fp32" not in self.func_name)
 
     def _param(self, shape, fan_in):
         return nn.Parameter(torch.randn(shape, device=self.device, dtype=torch.float32).mul_(1.0 / math.sqrt(fan_in)).to(self.dtype))
@@ -56,7 +60,7 @@ class _StructuredLinear(nn.Module):
             return self.func(*args), True
 
     def _finish(self, out, fused=False):
-        if self.kind == "torch" and isinstance(out, tuple):
+        if isinstance(out, tuple):                     # torch baselines and the *_fp32 names: (out, intermediates...)
             out = out[0]
         if fused:
             return out
@@ -66,6 +70,9 @@ class _StructuredLinear(nn.Module):
             out = torch.nn.functional.gelu(out, approximate="tanh")
         elif self.fused_act == "silu":
             out = torch.nn.functional.silu(out)
+        elif self.fused_act == "silu_mul":
+            gate, up = out.chunk(2, dim=-1)
+            out = torch.nn.functional.silu(gate) * up
         return out
 
 
@@ -194,8 +201,8 @@ class LowRankLinear(_StructuredLinear):
 
     def forward(self, x):
         out, fused = self._call(x, self.V, self.U)
-        if self.kind == "triton":                      # the kernel returns (N, out_f): restore the leading dims
-            out = out.reshape(*x.shape[:-1], self.out_features)
+        if self.kind == "triton" and not isinstance(out, tuple):   # the kernel returns (N, out_f): restore the leading dims
+            out = out.reshape(*x.shape[:-1], out.shape[-1])
         return self._finish(out, fused)
 
     def extra_repr(self):
@@ -210,8 +217,8 @@ class DenseLinear(_StructuredLinear):
 
     def forward(self, x):
         out, fused = self._call(x, self.W)
-        if self.kind == "triton":
-            out = out.reshape(*x.shape[:-1], self.out_features)
+        if self.kind == "triton" and not isinstance(out, tuple):
+            out = out.reshape(*x.shape[:-1], out.shape[-1])
         return self._finish(out, fused)
 
     def extra_repr(self):

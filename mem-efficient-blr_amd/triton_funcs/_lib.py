@@ -22,8 +22,9 @@ S_JIR, S_RIJ, S_IJR = 0, 1, 2
 ALGO_AUTO, ALGO_STREAM, ALGO_TILED, ALGO_FUSED, ALGO_STREAM_SPLIT = 0, 1, 2, 3, 4
 W2_SR, W2_RS = 0, 1
 OUT_INTERLEAVED, OUT_BLOCKED = 0, 1
-ACT_NONE, ACT_GELU_TANH, ACT_SILU = 0, 1, 2
-ACTS = {None: ACT_NONE, "none": ACT_NONE, "gelu_tanh": ACT_GELU_TANH, "silu": ACT_SILU}
+ACT_NONE, ACT_GELU_TANH, ACT_SILU, ACT_SILU_MUL = 0, 1, 2, 3
+ACTS = {None: ACT_NONE, "none": ACT_NONE, "gelu_tanh": ACT_GELU_TANH, "silu": ACT_SILU, "silu_mul": ACT_SILU_MUL}
+OP_BLAST, OP_MONARCH, OP_LOW_RANK, OP_DENSE = 0, 1, 2, 3
 
 _c = ctypes
 _vp, _i, _i64, _sz = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_size_t
@@ -53,6 +54,7 @@ _SIGNATURES = {
     "blr_monarch_fwd_ep2": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 9 + [_vp, _sz, _vp, _vp, _i, _vp, _i, _i64, _vp, _i64]),
     "blr_low_rank_fwd_ep2": (_i, [_vp, _i64, _vp, _vp, _vp, _i64] + [_i] * 6 + [_vp, _sz, _vp, _vp, _i, _vp, _i, _i64, _vp, _i64]),
     "blr_dense_fwd_ep2": (_i, [_vp, _i64, _vp, _vp, _i64] + [_i] * 5 + [_vp, _sz, _vp, _vp, _i, _vp, _i, _i64, _vp, _i64]),
+    "blr_ep_workspace_bytes": (_sz, [_i] * 6),
     "blr_workspace_status": (_i, [_vp, _sz, _vp]),
     "blr_set_spin_limit": (None, [_c.c_uint]),
     "blr_set_option": (_i, [_c.c_char_p, _i, _i]),
@@ -248,6 +250,16 @@ class fused_epilogue:
     def __exit__(self, *exc):
         _ep_state.ep = self.prev
         return False
+
+
+def ep_out_features(ep, out_f):
+    """Columns of the result: out_f, or out_f / 2 under the gated activation (silu(gate) * up over a fused gate|up projection)."""
+    return out_f // 2 if ep is not None and ep[1] == ACT_SILU_MUL else out_f
+
+
+def ep_workspace_extra(ep, op, M, out_f, b, dt):
+    """Bytes the *_fwd_ep call wants on top of the operator's own workspace (the full-width result where no kernel fuses the gate)."""
+    return lib().blr_ep_workspace_bytes(op, M, out_f, b, dt, ep[1]) if ep is not None else 0
 
 
 def pending_epilogue(out_f, dtype, device):

@@ -62,16 +62,16 @@ def _blast(name, x, U, V, S, u_layout, s_layout, algo, want_intermediates):
     dt = L.dtype_code(x.dtype)
     x2 = L.rows(x)
     M, in_f, out_f = x2.shape[0], b1 * p, b2 * q
-    out = torch.empty((M, out_f), device=x.device, dtype=x.dtype)
     z = y = None
     if want_intermediates:
         z = torch.empty((b2, M, r), device=x.device, dtype=x.dtype)
         y = torch.empty((b1, M, r), device=x.device, dtype=x.dtype)
         algo = L.ALGO_TILED
     lib = L.lib()
-    need = lib.blr_blast_workspace_bytes(M, in_f, out_f, b1, r, dt, algo)
-    ws = L.workspace(x.device, need, algo, M, dt)
     ep = None if want_intermediates else L.pending_epilogue(out_f, x.dtype, x.device)
+    out = torch.empty((M, L.ep_out_features(ep, out_f)), device=x.device, dtype=x.dtype)
+    need = lib.blr_blast_workspace_bytes(M, in_f, out_f, b1, r, dt, algo) + L.ep_workspace_extra(ep, L.OP_BLAST, M, out_f, b1, dt)
+    ws = L.workspace(x.device, need, algo, M, dt)
     if ep is not None:
         rc = lib.blr_blast_fwd_ep2(x2.data_ptr(), x2.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(),
                                   out.data_ptr(), out.stride(0), M, in_f, out_f, b1, r, dt, u_layout, s_layout, algo,
@@ -85,7 +85,7 @@ def _blast(name, x, U, V, S, u_layout, s_layout, algo, want_intermediates):
     L.check(rc, name, ws)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": b1, "rank": r,
                           "algo": algo, "dtype": str(x.dtype)}
-    return out.reshape(*x.shape[:-1], out_f), z, y
+    return out.reshape(*x.shape[:-1], out.shape[-1]), z, y
 
 
 def _fp16(name, x, U, V, S, config, u_layout, s_layout):

@@ -24,10 +24,10 @@ def _dense(name, x, w, algo):
     x2 = L.rows(x)
     M, in_f = x2.shape
     out_f = w.shape[1]
-    out = torch.empty((M, out_f), device=x.device, dtype=x.dtype)
     lib = L.lib()
-    ws = L.workspace(x.device, lib.blr_dense_workspace_bytes(M, in_f, out_f, dt, algo), algo, M, dt)
     ep = L.pending_epilogue(out_f, x.dtype, x.device)
+    out = torch.empty((M, L.ep_out_features(ep, out_f)), device=x.device, dtype=x.dtype)
+    ws = L.workspace(x.device, lib.blr_dense_workspace_bytes(M, in_f, out_f, dt, algo) + L.ep_workspace_extra(ep, L.OP_DENSE, M, out_f, 1, dt), algo, M, dt)
     if ep is not None:
         rc = lib.blr_dense_fwd_ep2(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
                                   M, in_f, out_f, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1], *ep[3])

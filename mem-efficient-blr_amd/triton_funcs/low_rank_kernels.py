@@ -25,11 +25,11 @@ def _low_rank(name, x, a, b, algo, want_z):
     x2 = L.rows(x)
     M, in_f = x2.shape
     r, out_f = b.shape
-    out = torch.empty((M, out_f), device=x.device, dtype=x.dtype)
     z = torch.empty((M, r), device=x.device, dtype=x.dtype) if want_z else None
     lib = L.lib()
-    ws = L.workspace(x.device, lib.blr_low_rank_workspace_bytes(M, in_f, out_f, r, dt, algo), algo, M, dt)
     ep = None if want_z else L.pending_epilogue(out_f, x.dtype, x.device)
+    out = torch.empty((M, L.ep_out_features(ep, out_f)), device=x.device, dtype=x.dtype)
+    ws = L.workspace(x.device, lib.blr_low_rank_workspace_bytes(M, in_f, out_f, r, dt, algo) + L.ep_workspace_extra(ep, L.OP_LOW_RANK, M, out_f, 1, dt), algo, M, dt)
     if ep is not None:
         rc = lib.blr_low_rank_fwd_ep2(x2.data_ptr(), x2.stride(0), a.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
                                      M, in_f, out_f, r, dt, algo, ws.data_ptr(), ws.numel(), L.stream_ptr(x.device), ep[0], ep[1], *ep[3])

@@ -49,13 +49,13 @@ def _monarch(name, x, w1, w2, w2_layout, out_order, algo, want_out1):
     dt = L.dtype_code(x.dtype)
     x2 = L.rows(x)
     M, in_f, out_f = x2.shape[0], k * p, l * s
-    out = torch.empty((M, out_f), device=x.device, dtype=x.dtype)
     out1 = torch.empty((l, M, r), device=x.device, dtype=x.dtype) if want_out1 else None
     if want_out1:
         algo = L.ALGO_TILED
     lib = L.lib()
-    ws = L.workspace(x.device, lib.blr_monarch_workspace_bytes(M, in_f, out_f, k, q, dt, algo), algo, M, dt)
     ep = None if want_out1 else L.pending_epilogue(out_f, x.dtype, x.device)
+    out = torch.empty((M, L.ep_out_features(ep, out_f)), device=x.device, dtype=x.dtype)
+    ws = L.workspace(x.device, lib.blr_monarch_workspace_bytes(M, in_f, out_f, k, q, dt, algo) + L.ep_workspace_extra(ep, L.OP_MONARCH, M, out_f, k, dt), algo, M, dt)
     if ep is not None:
         rc = lib.blr_monarch_fwd_ep2(x2.data_ptr(), x2.stride(0), w1.data_ptr(), w2.data_ptr(), out.data_ptr(), out.stride(0),
                                     M, in_f, out_f, k, q, dt, w2_layout, out_order, algo,
@@ -67,7 +67,7 @@ def _monarch(name, x, w1, w2, w2_layout, out_order, algo, want_out1):
                                  ws.data_ptr(), ws.numel(), L.stream_ptr(x.device))
     L.check(rc, name, ws)
     _last_config[name] = {"kernel": "libblr", "M": M, "in_f": in_f, "out_f": out_f, "b": k, "rank": q, "algo": algo}
-    return out.reshape(*x.shape[:-1], out_f), out1
+    return out.reshape(*x.shape[:-1], out.shape[-1]), out1
 
 
 def _pre_out1(out1, k):

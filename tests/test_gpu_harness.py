@@ -155,3 +155,20 @@ def test_gpu_profile_traces_a_function_under_rocprofv3(tmp_path):
     rows = [ln for ln in text.splitlines() if "blr" in ln and "command:" not in ln]
     assert rows, text
     assert any(int(ln.split()[-4]) >= 8 for ln in rows), text          # 2 warm-up + 6 timed calls of at least one kernel
+
+
+def test_fp32_verification_names_keep_bias_gate_and_residual():
+    """The *_fp32 names return their intermediates and never read an armed output stage; a wrapper module built on one must
+    apply bias, gate and residual itself (reference DiT/models.py:120-121: x + gate.unsqueeze(1) * f(x))."""
+    import torch
+    from models import wrappers as W
+    from models.dit_xl import _gated
+    torch.manual_seed(0)
+    lin = W.BlastLinear(128, 160, 4, 32, "triton_funcs.blast_kernels.triton_blast_full_fp32", torch.device("cuda"), torch.float32, bias=True)
+    assert lin.fuses is False
+    h = torch.randn(2, 24, 128, device="cuda"); gate = torch.randn(2, 160, device="cuda"); resid = torch.randn(2, 24, 160, device="cuda")
+    with torch.no_grad():
+        plain = lin.func(h, lin.U, lin.V, lin.S)[0] + lin.bias
+        got = _gated(lin, h, gate, resid)
+    want = resid + gate.unsqueeze(1) * plain
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-5)
