@@ -91,19 +91,21 @@ def test_monarch_small_all_algorithms(name, shape, algo, dtype):
 LLAMA_IO = {"qkvo": (4096, 4096), "gate_up": (4096, 22016), "down": (11008, 4096)}
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M", [1, 16, 2048])
 @pytest.mark.parametrize("layer", list(LLAMA_IO))
-def test_monarch_llama7b(layer, M):
-    """BASELINE config 2: nblocks = 4, rank 1024 per block, fp16."""
+def test_monarch_llama7b(layer, M, dtype):
+    """BASELINE config 2: nblocks = 4, rank 1024 per block; fp16 as the config says and bf16 as the reference's kernels compute
+    (reference triton_funcs/monarch_kernels.py:676-677)."""
     in_f, out_f = LLAMA_IO[layer]
     b, rank = 4, 1024
     x, w1_t, w2_t = monarch_inputs(b, in_f // b, rank, out_f // b, (1, M), seed=0)
     rows = list(range(M)) if M <= 16 else [0, 1, 127, 128, 1023, 2047]
-    ref = _ref_monarch(x[:, rows], w1_t, w2_t, torch.float16)[0]
+    ref = _ref_monarch(x[:, rows], w1_t, w2_t, dtype)[0]
     for name in ("triton_monarch_right_fp16", "triton_monarch_right_left_fp16"):
-        say(f"[case] llama7b monarch {layer} {name} M={M}")
-        out = _run_monarch(name, x, w1_t, w2_t, torch.float16)
-        assert_close(out[:, rows], ref, torch.float16, f"monarch {layer} {name} M{M}")
+        say(f"[case] llama7b monarch {layer} {name} M={M} {dtype}")
+        out = _run_monarch(name, x, w1_t, w2_t, dtype)
+        assert_close(out[:, rows], ref, dtype, f"monarch {layer} {name} M{M}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -246,24 +248,26 @@ def test_load_store_probes_move_every_operand_at_hbm_speed(M):
     assert y0.dtype == torch.float32 and not y0.any()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M", [1, 16, 2048])
 @pytest.mark.parametrize("layer", list(LLAMA_IO))
-def test_low_rank_and_dense_llama7b(layer, M):
-    """BASELINE config 2: r = 1024, fp16."""
+def test_low_rank_and_dense_llama7b(layer, M, dtype):
+    """BASELINE config 2: r = 1024; fp16 as the config says and bf16 as the reference's kernels compute
+    (reference triton_funcs/low_rank_kernels.py:286-288, dense_kernels.py:268-269)."""
     from triton_funcs import low_rank_kernels as K, dense_kernels as D
     in_f, out_f = LLAMA_IO[layer]
     x, Vt, Ut = lr_inputs(in_f, 1024, out_f, (1, M), seed=0)
     rows = list(range(M)) if M <= 16 else [0, 1, 127, 128, 1023, 2047]
-    say(f"[case] llama7b low_rank {layer} M={M}")
-    y = K.triton_low_rank_fp16(dev(x, torch.float16), dev(Vt.T, torch.float16), dev(Ut.T, torch.float16))
-    ro = O.low_rank_forward(rounded(x[0, rows], torch.float16), rounded(Vt, torch.float16), rounded(Ut, torch.float16))[0]
-    assert_close(y[rows], ro, torch.float16, f"low_rank {layer} M{M}")
+    say(f"[case] llama7b low_rank {layer} M={M} {dtype}")
+    y = K.triton_low_rank_fp16(dev(x, dtype), dev(Vt.T, dtype), dev(Ut.T, dtype))
+    ro = O.low_rank_forward(rounded(x[0, rows], dtype), rounded(Vt, dtype), rounded(Ut, dtype))[0]
+    assert_close(y[rows], ro, dtype, f"low_rank {layer} M{M}")
     rng = np.random.default_rng(1)
     W = rng.standard_normal((in_f, out_f)).astype(np.float32) / np.sqrt(in_f)
-    say(f"[case] llama7b dense {layer} M={M}")
-    d = D.triton_dense_fp16(dev(x, torch.float16), dev(W, torch.float16))
-    rd = rounded(x[0, rows], torch.float16) @ rounded(W, torch.float16)
-    assert_close(d[rows], rd, torch.float16, f"dense {layer} M{M}")
+    say(f"[case] llama7b dense {layer} M={M} {dtype}")
+    d = D.triton_dense_fp16(dev(x, dtype), dev(W, dtype))
+    rd = rounded(x[0, rows], dtype) @ rounded(W, dtype)
+    assert_close(d[rows], rd, dtype, f"dense {layer} M{M}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -75,11 +75,14 @@ def test_blast_q_vs_oracle_on_dequantized(shape, bits, dtype):
         assert_close(out, ref, dtype, f"blast_q bits={bits} algo={algo}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M", [1, 4, 16])
 @pytest.mark.parametrize("bits", [8, 4])
 @pytest.mark.parametrize("layer", ["gate_up", "down"])
-def test_blast_q_llama7b(layer, bits, M):
-    """BASELINE config 4 at full shape."""
+def test_blast_q_llama7b(layer, bits, M, dtype):
+    """BASELINE config 4 at full shape (activations and S in fp16 as the config says, and in bf16).  The weight quantizer is
+    this build's own definition - the reference has none - so "parity" here means: codes and scales bit-exact against the
+    numpy restatement of that definition, outputs against the fp64 product of the dequantized factors."""
     from triton_funcs import blast_sym_quant_kernels as Q
     p, q, r = {"gate_up": (256, 1376, 1024), "down": (688, 256, 1024)}[layer]
     b = 16
@@ -88,16 +91,16 @@ def test_blast_q_llama7b(layer, bits, M):
     U = (rng.standard_normal((b, q, r)) / np.sqrt(r)).astype(np.float32)
     V = (rng.standard_normal((b, p, r)) / np.sqrt(r)).astype(np.float32)
     S = rng.standard_normal((r, b, b))
-    say(f"[case] blast_q llama7b {layer} bits={bits} M={M}")
+    say(f"[case] blast_q llama7b {layer} bits={bits} M={M} {dtype}")
     Uq, Vq = Q.quantize_blast_factors(torch.from_numpy(U).cuda(), torch.from_numpy(V).cuda(), bits)
     uc, us = O.quantize_sym(U, 2, bits); vc, vs = O.quantize_sym(V, 1, bits)
     got_uc = Uq.codes.cpu().numpy() if bits == 8 else O.unpack_int4(Uq.codes.cpu().numpy())
     np.testing.assert_array_equal(got_uc.transpose(0, 2, 1), uc)      # U codes are stored (b, r, q)
     np.testing.assert_array_equal(Uq.scales.cpu().numpy(), us)
     np.testing.assert_array_equal(Vq.scales.cpu().numpy(), vs)
-    out = Q.triton_blast_bmm_int8_fp16(dev(x, torch.float16), Uq, Vq, dev(S, torch.float16))
-    ref = O.blast_q_forward(rounded(x, torch.float16), uc, us, vc, vs, rounded(S, torch.float16))
-    assert_close(out, ref, torch.float16, f"blast_q {layer} bits={bits} M={M}")
+    out = Q.triton_blast_bmm_int8_fp16(dev(x, dtype), Uq, Vq, dev(S, dtype))
+    ref = O.blast_q_forward(rounded(x, dtype), uc, us, vc, vs, rounded(S, dtype))
+    assert_close(out, ref, dtype, f"blast_q {layer} bits={bits} M={M}")
 
 
 def test_blast_q_rejects_bad_input():
