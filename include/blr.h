@@ -204,6 +204,15 @@ int blr_stream_probe(const void* src, size_t bytes, void* dst, void* stream);
 int blr_load_store_probe(const void* x, size_t x_bytes, const void* w1, size_t w1_bytes, const void* w2, size_t w2_bytes,
                          void* y, size_t y_bytes, void* dst, void* stream);
 
+/* What the matrix cores sustain with nothing in their way (no counterpart in the reference; the role its device.py gives to a
+ * spec-sheet number): one workgroup of eight waves per compute unit, each wave a chain of eight independent 32x32x16 fp16
+ * products per iteration with the operands in registers.  random != 0: pseudo-random operands in [-2, 2) instead of ones (the
+ * power drawn, and with it the clock, depends on the data); lds_reads = 6: every eight products come with the six 1 KiB
+ * fragment reads from LDS that a 128 x 64 wave tile needs (0: none).  dst: at least 4 bytes of device memory.  Time the launch
+ * with events; blr_mfma_probe_flops(iters) is the number of floating-point operations of one launch on the current device.   */
+int blr_mfma_probe(int iters, int random, int lds_reads, void* dst, void* stream);
+double blr_mfma_probe_flops(int iters);
+
 /* ---- fused output stage ---------------------------------------------------------------------
  * out = act(op(x) + bias): what the callers do right after the operator - the bias add of the wrapper
  * modules (reference models/wrappers.py:176-177) and the activation that follows the first MLP linear

@@ -1310,6 +1310,73 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
 
 }  // namespace blr
 
+// ---- matrix-core probe ----------------------------------------------------------------------------------------------
+// What the matrix cores sustain with nothing in their way: one workgroup of eight waves per compute unit, every wave a chain of
+// eight independent 32x32x16 products per iteration, operands in registers.  With `random` the operands are pseudo-random
+// numbers in [-2, 2) instead of ones (the power drawn, and with it the clock, depends on the data); with `lds_reads` every group
+// of eight products is accompanied by that many 1 KiB fragment reads from LDS (6 = what a 128 x 64 wave tile needs).
+namespace blr {
+template <bool RANDOM, int READS>
+__global__ __launch_bounds__(512) void mfma_probe_kernel(unsigned* sink, int iters) {
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[32768];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < 32768 / 4; i += 512) reinterpret_cast<unsigned*>(smem)[i] = i;
+  __syncthreads();
+  f32x16 acc[8];
+#pragma unroll
+  for (int a = 0; a < 8; ++a)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[a][e] = 0.f;
+  f16x8 fa = {1, 1, 1, 1, 1, 1, 1, 1}, fb = fa;
+  if (RANDOM) {
+    unsigned h = (tid * 2654435761u) ^ (blockIdx.x * 40503u) ^ 0x9e3779b9u;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      h ^= h << 13; h ^= h >> 17; h ^= h << 5;
+      fa[e] = (f16)(((int)(h & 0xffff) - 32768) / 16384.0f);
+      h ^= h << 13; h ^= h >> 17; h ^= h << 5;
+      fb[e] = (f16)(((int)(h & 0xffff) - 32768) / 16384.0f);
+    }
+  }
+  u32x4 x = {0, 0, 0, 0};
+  const unsigned char* base = smem + (wave & 3) * 8192 + lane * 16;
+  uint32_t off = 0;
+  for (int it = 0; it < iters; ++it) {
+    asm volatile("" : "+v"(off));                        // (keeps the reads inside the loop)
+    u32x4 v[READS > 0 ? READS : 1];
+#pragma unroll
+    for (int r = 0; r < READS; ++r) v[r] = *reinterpret_cast<const u32x4*>(base + off + r * 1024);
+#pragma unroll
+    for (int a = 0; a < 8; ++a) acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb, acc[a], 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < READS; ++r) x ^= v[r];
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int a = 0; a < 8; ++a) s += acc[a][0];
+  if (s == 12345.f || x[0] == 0xdeadbeefu) sink[0] = x[1];
+}
+}  // namespace blr
+
+extern "C" double blr_mfma_probe_flops(int iters) {
+  const int cus = blr::device_cus() > 0 ? blr::device_cus() : 256;
+  return (double)cus * 8.0 * (double)iters * 8.0 * (2.0 * 32 * 32 * 16);
+}
+
+extern "C" int blr_mfma_probe(int iters, int random, int lds_reads, void* dst, void* stream) {
+  using namespace blr;
+  if (iters <= 0 || !dst || (lds_reads != 0 && lds_reads != 6)) { set_error("mfma_probe: iters > 0, dst, lds_reads 0 or 6"); return BLR_ERR_BAD_ARG; }
+  const int cus = device_cus() > 0 ? device_cus() : 256;
+  hipStream_t st = (hipStream_t)stream;
+  unsigned* sink = reinterpret_cast<unsigned*>(dst);
+  if (random && lds_reads) hipLaunchKernelGGL((mfma_probe_kernel<true, 6>), dim3(cus), dim3(512), 0, st, sink, iters);
+  else if (random) hipLaunchKernelGGL((mfma_probe_kernel<true, 0>), dim3(cus), dim3(512), 0, st, sink, iters);
+  else if (lds_reads) hipLaunchKernelGGL((mfma_probe_kernel<false, 6>), dim3(cus), dim3(512), 0, st, sink, iters);
+  else hipLaunchKernelGGL((mfma_probe_kernel<false, 0>), dim3(cus), dim3(512), 0, st, sink, iters);
+  BLR_CHECK_LAUNCH("mfma_probe");
+  return BLR_OK;
+}
+
 #ifdef BLR_TRACE
 extern "C" int blr_debug_trace_gemm(unsigned long long* host, int n) {
   return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(blr::g_trace_gemm), (size_t)n * 8, 0, hipMemcpyDeviceToHost);

@@ -61,6 +61,8 @@ _SIGNATURES = {
     "blr_blast_fwd_static": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64] + [_i] * 8 + [_vp]),
     "blr_probe_dst_words": (_i, []),
     "blr_stream_probe": (_i, [_vp, _sz, _vp, _vp]),
+    "blr_mfma_probe": (_i, [_i, _i, _i, _vp, _vp]),
+    "blr_mfma_probe_flops": (_c.c_double, [_i]),
     "blr_load_store_probe": (_i, [_vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp]),
 }
 
