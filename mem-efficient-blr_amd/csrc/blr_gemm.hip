@@ -573,8 +573,11 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
     }
   };
   auto mfma_one = [&](int set, int idx) {
+    // the operands are handed over swapped, so that a product comes out transposed: lane l then holds, for row l & 31 of the
+    // 32 x 32 block, four runs of four CONSECUTIVE columns (8 q + 4 (l >> 5) + 0..3, q = 0..3) - the write-out packs a run into
+    // one 8-byte LDS store (one 16-byte store of partial sums) instead of four two-byte ones
     const int i = idx / TN, j = idx % TN;
-    acc[i][j] = TypeTraits<T>::mfma32(af[set][i], bf[set][j], acc[i][j]);
+    acc[i][j] = TypeTraits<T>::mfma32(bf[set][j], af[set][i], acc[i][j]);
   };
 
   // One k tile per step.  During step t the loads of A tile t + NA - 1 and of B tile t + NB - 1 go out (A first), into the
@@ -655,17 +658,19 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
   TRG(2);
   if (PARTIAL) {
-    // fp32 partial sums of this slice, straight from the accumulators: an instruction stores two rows of 32 floats
+    // fp32 partial sums of this slice, straight from the accumulators: 16 bytes per lane (N is a multiple of 8, so a run of
+    // four columns is inside or outside as a whole)
     float* P = reinterpret_cast<float*>(g.C) + (int64_t)bt * g.sC;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const int gc = n0 + wn * WN + j * 32 + (lane & 31);
+        const int gr = m0 + wm * WM + i * 32 + (lane & 31);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int gr = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-          if (gr < g.M && gc < g.N) P[(int64_t)gr * g.ldc + gc] = acc[i][j][e];
+        for (int q = 0; q < 4; ++q) {
+          const int gc = n0 + wn * WN + j * 32 + q * 8 + (lane >> 5) * 4;
+          if (gr < g.M && gc < g.N)
+            *reinterpret_cast<f32x4*>(&P[(int64_t)gr * g.ldc + gc]) = f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
         }
       }
     return;
@@ -678,11 +683,14 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int col = wn * WN + j * 32 + (lane & 31);
+      const int row = wm * WM + i * 32 + (lane & 31);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        cs[row * CLD + col] = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][e]) : acc[i][j][e]);
+      for (int q = 0; q < 4; ++q) {
+        const int col = wn * WN + j * 32 + q * 8 + (lane >> 5) * 4;
+        typename TypeTraits<T>::vec4 v4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v4[e] = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][4 * q + e]) : acc[i][j][4 * q + e]);
+        *reinterpret_cast<typename TypeTraits<T>::vec4*>(&cs[row * CLD + col]) = v4;
       }
     }
   __syncthreads();
