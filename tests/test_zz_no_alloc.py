@@ -103,3 +103,54 @@ def test_oversize_call_is_refused_without_a_launch():
     assert rc == 0, L.lib().blr_last_error().decode()
     torch.cuda.synchronize()
     assert torch.isfinite(out).all()
+
+
+def test_no_device_memory_is_allocated_and_a_graph_can_hold_the_call():
+    """What the entry point is for: after the first call on a device (which resolves the address of the built-in scratch),
+    further calls change neither the driver's free memory nor torch's allocator; and one call captured into a HIP graph
+    replays - several times, with eager calls and synchronisations between the replays - to the bits of the eager result."""
+    from triton_funcs import _lib as L
+    dtype = torch.float16
+    b, p, q, r = 16, 64, 72, 128
+    cases = []
+    for n, M in enumerate((96, 3)):                              # three launches with Y and Z in the scratch; two launches at few rows
+        x, U, V, S, ref = _operands(b, p, q, r, M, dtype, 95 + n)
+        out = torch.empty((M, b * q), device="cuda", dtype=dtype)
+        cases.append((x, U, V, S, ref, out, M))
+
+    def call(c, stream):
+        x, U, V, S, _, out, M = c
+        return L.lib().blr_blast_fwd_static(x.data_ptr(), x.stride(0), U.data_ptr(), V.data_ptr(), S.data_ptr(), out.data_ptr(), out.stride(0),
+                                            M, b * p, b * q, b, r, L.dtype_code(dtype), L.U_RQ, L.S_JIR, stream)
+
+    say("[case] blast_fwd_static allocates nothing; graph capture and replay")
+    for c in cases:                                              # first calls: one-time set-up, outside any measurement
+        assert call(c, L.stream_ptr(c[0].device)) == 0, L.lib().blr_last_error().decode()
+    torch.cuda.synchronize()
+    eager = [c[5].clone() for c in cases]
+    free0, _ = torch.cuda.mem_get_info()
+    alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(5):
+        for c in cases:
+            assert call(c, L.stream_ptr(c[0].device)) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, f"free device memory changed by {free0 - free1} bytes over repeated calls"
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+    for c, e in zip(cases, eager):
+        assert torch.equal(c[5], e)
+        assert_close(c[5], c[4], dtype, "static call against the oracle")
+    for c, e in zip(cases, eager):
+        g = torch.cuda.CUDAGraph()
+        c[5].zero_()
+        with torch.cuda.graph(g):
+            rc = call(c, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, L.lib().blr_last_error().decode()
+        for rep in range(3):
+            c[5].zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(c[5], e), f"replay {rep} of the captured call differs from the eager result"
+            other = cases[1] if c is cases[0] else cases[0]      # an eager call of another shape between the replays
+            assert call(other, L.stream_ptr(other[0].device)) == 0
+            torch.cuda.synchronize()
