@@ -32,6 +32,29 @@ def test_layer_verify_all_match(cfg, tmp_path, monkeypatch):
     assert os.path.exists(f"output/{l.network_name}/{l.layer_name}/triton_blast_bmm_xv_fp16_best_config.pkl")
 
 
+REFERENCE_SWEEP_LAYERS = ["dit_xl.adaln", "gpt2s.c_attn", "gpt2s.mlp_c_proj", "llama1b.down_proj", "llama1b.gate_proj", "llama1b.qo_proj",
+                          "llama1b.up_proj", "vit_b_patch16_224.attn_qkv", "vit_b_patch16_224.mlp_fc1", "vit_b_patch16_224.mlp_fc2",
+                          "vit_b_patch8_224.attn_qkv", "vit_b_patch8_224.mlp_fc1", "vit_b_patch8_224.mlp_fc2"]
+
+
+@pytest.mark.parametrize("num_seq", [1, 48, 300])
+@pytest.mark.parametrize("cfg", REFERENCE_SWEEP_LAYERS)
+def test_reference_sweep_layers_verify(cfg, num_seq, tmp_path, monkeypatch):
+    """The layer files of the reference's own sweeps (configs/layers/*.yaml: 3, 6, 9 and 16 blocks, Monarch with 16 blocks,
+    ranks 128 to 768) through Layer.verify at one row, a few dozen and a few hundred: every function of every family MATCHes."""
+    from layer import Layer
+    from utils import VerificationStatus
+    monkeypatch.chdir(tmp_path)
+    l = Layer(os.path.join(PKG, "configs", "layers", cfg + ".yaml"))
+    l.num_seq = num_seq
+    say(f"[case] Layer.verify {cfg} num_seq={num_seq}")
+    l.verify("all")
+    for fam in ("blast", "monarch", "low_rank", "dense"):
+        if fam == "monarch" and l.monarch is None:
+            continue
+        assert l.status[fam] and all(s == VerificationStatus.MATCH for s in l.status[fam]), (fam, l.status[fam])
+
+
 @pytest.mark.parametrize("M", [1, 40])
 def test_wrappers_on_gpu_vs_oracle(M):
     from models.wrappers import BlastLinear, MonarchLinear, LowRankLinear, DenseLinear, QuantBlastLinear
