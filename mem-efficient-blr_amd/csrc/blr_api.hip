@@ -294,13 +294,24 @@ using namespace blr;
 namespace blr {
 namespace {
 constexpr int kOptUnset = -2147483647 - 1;
-const char* const kOptNames[OPT_COUNT] = {"BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU", "BLR_GEMM_RING_WAVES", "BLR_GEMM_SPLITK"};
+const char* const kOptNames[OPT_COUNT] = {"BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU", "BLR_GEMM_RING_WAVES", "BLR_GEMM_SPLITK",
+                                          "BLR_DECODE2", "BLR_DECODE3", "BLR_DECODE_PAIR", "BLR_DECODE_ROWS", "BLR_DENSE_SLAB", "BLR_DENSE_ROWS",
+                                          "BLR_BLAST_MIXU", "BLR_BLAST_ONE"};
+// what each option may be set to: a range, or (BLR_GEMM_RING_TILE, BLR_GEMM_RING_WAVES) a short list; anything else is refused
+bool opt_value_ok(int id, int v) {
+  switch (id) {
+    case OPT_GEMM_RING: case OPT_GEMM_RING_PER_CU: case OPT_DECODE_PAIR: case OPT_BLAST_MIXU: return v >= 0 && v <= 2;
+    case OPT_GEMM_RING_TILE: return v == 0 || v == 256256 || v == 256128 || v == 128128;
+    case OPT_GEMM_RING_WAVES: return v == 4 || v == 8;
+    default: return v == 0 || v == 1;
+  }
+}
 std::atomic<int> g_opts[OPT_COUNT];
 std::once_flag g_opts_once;
 void opts_init() {
   for (int i = 0; i < OPT_COUNT; ++i) {
     const char* e = getenv(kOptNames[i]);
-    g_opts[i].store(e ? atoi(e) : kOptUnset, std::memory_order_relaxed);
+    g_opts[i].store(e && opt_value_ok(i, atoi(e)) ? atoi(e) : kOptUnset, std::memory_order_relaxed);   // (a value out of range is ignored)
   }
 }
 }  // namespace
@@ -324,6 +335,7 @@ int blr_set_option(const char* name, int value, int unset) {
   std::call_once(blr::g_opts_once, blr::opts_init);
   for (int i = 0; name && i < blr::OPT_COUNT; ++i)
     if (!strcmp(name, blr::kOptNames[i])) {
+      if (!unset && !blr::opt_value_ok(i, value)) { set_error("set_option: %d is not a value of %s", value, name); return BLR_ERR_BAD_ARG; }
       blr::g_opts[i].store(unset ? blr::kOptUnset : value, std::memory_order_relaxed);
       return BLR_OK;
     }
@@ -406,7 +418,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   // others with a long stream each (4096 -> 4096 at 17 rows: 36 us through the tiles, 12 us at 16 rows through the few-row
   // kernels).  Up to 128 rows the three launches of the few-row path run over tiles of 16 rows with the weights held in registers
   // (at 128 rows 32 / 44 / 43 us against 39 / 48 / 56 us through the tiles on the three Llama-7B layers).
-  static const int rows_max_m = getenv("BLR_TILED_ROWS_MAX_M") ? atoi(getenv("BLR_TILED_ROWS_MAX_M")) : 128;
+  constexpr int rows_max_m = 128;
   if (M <= rows_max_m && !y_out && !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && !silu_mul_armed()) {
     StreamBlastArgs s = {};
     s.x = x; s.ldx = ldx; s.U = U; s.V = V; s.S = S; s.out = out; s.ldo = ldo;
@@ -419,17 +431,17 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
   // by itself only for narrow input blocks: the fused kernel re-reads V once per 32 rows, and from about 128 columns per
   // block on that costs more than the round trip of Y it saves (measured at 4096 rows: 1152 -> 1152, r = 288: 64 against
   // 68 us; 4608 -> 1152, r = 576: 154 against 122 us; Llama-7B gate_up at 2048 rows: 201 against 186 us).
-  static const int fuse_max_p = getenv("BLR_BLAST_FUSE_MAX_P") ? atoi(getenv("BLR_BLAST_FUSE_MAX_P")) : 128;
+  constexpr int fuse_max_p = 128;
   // Narrow output blocks (either layout of U: it is re-laid for the kernel anyway): the mix and the product with U run as one launch that reads Y once and
   // never writes Z (blast_mixu_kernel); the first half is then the plain GEMM, which leaves Y.  Measured at 4096 rows against the
   // mix kernel + batched GEMM: 4608 -> 1152, r = 576: 90 against 122 us; against the fused first half + batched GEMM: 1152 -> 1152,
   // r = 288: 47 against 51 us.  BLR_BLAST_MIXU: 0 never, 1 only where the first half would not be fused anyway, 2 (default)
   // wherever the kernel takes the shape.
-  static const int mixu_mode = getenv("BLR_BLAST_MIXU") ? atoi(getenv("BLR_BLAST_MIXU")) : 2;
+  const int mixu_mode = option_value(OPT_BLAST_MIXU, 2);
   const bool mixu_shape = !z_out && !sat8 && fused <= 0 && dtype != BLR_F32 && b == 16 && Q % 8 == 0 && Q <= 80 && r % 32 == 0 && !silu_mul_armed();
   // Narrow input blocks as well (at most 96 columns): the whole call is one launch that forms Y per step of the rank walk in the
   // compute unit and keeps neither Y nor Z in memory (blast_one_kernel).  BLR_BLAST_ONE=0 switches it off.
-  static const int one_mode = getenv("BLR_BLAST_ONE") ? atoi(getenv("BLR_BLAST_ONE")) : 1;
+  const int one_mode = option_value(OPT_BLAST_ONE, 1);
   if (one_mode && mixu_shape && !y_out && P <= 96 && P % 8 == 0) {
     GemmArgs e1 = {};
     attach_epilogue_peek(e1);
@@ -453,8 +465,7 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
     if (mixu) {                                     // the GEMM's launch also re-lays U and S for the kernel that follows, if it can
       GemmArgs e2 = {};
       attach_epilogue_peek(e2);
-      static const int side_on = getenv("BLR_MIXU_SIDE") ? atoi(getenv("BLR_MIXU_SIDE")) : 1;      // 0: a launch of its own
-      if (side_on && blast_mixu_plan(Y, S, U, out, ldo, e2, M, b, r, Q, si, sj, sr, dtype, Z, ybytes, &g1.side, u_layout == BLR_U_RQ)) g1.side_taken = &mixu_prepared;
+      if (blast_mixu_plan(Y, S, U, out, ldo, e2, M, b, r, Q, si, sj, sr, dtype, Z, ybytes, &g1.side, u_layout == BLR_U_RQ)) g1.side_taken = &mixu_prepared;
       else g1.side.items = 0;
     }
     rc = gemm_launch(g1, dtype, st);

@@ -84,8 +84,11 @@ unsigned spin_limit_now();
 // that applies it itself says so with epilogue_taken(), otherwise the entry point finishes with an elementwise launch.
 bool epilogue_pending(const void** bias, int* act);   // (false when a gate or a residual is armed: only the tiled path fuses those)
 void epilogue_taken();
-// Tuning options that tests switch at run time (blr_set_option); each starts from the environment variable of its name, read once.
-enum { OPT_GEMM_RING = 0, OPT_GEMM_RING_TILE, OPT_GEMM_RING_PER_CU, OPT_GEMM_RING_WAVES, OPT_GEMM_SPLITK, OPT_COUNT };
+// Every run-time switch of the library (blr_set_option): each starts from the environment variable of its name, read once, and
+// is range-checked where it is set.  The first five pick the GEMM variant, the rest switch a kernel family off (0) so that the
+// call falls through to the next one that serves it - for A/B measurements and as a way out should a kernel misbehave.
+enum { OPT_GEMM_RING = 0, OPT_GEMM_RING_TILE, OPT_GEMM_RING_PER_CU, OPT_GEMM_RING_WAVES, OPT_GEMM_SPLITK,
+       OPT_DECODE2, OPT_DECODE3, OPT_DECODE_PAIR, OPT_DECODE_ROWS, OPT_DENSE_SLAB, OPT_DENSE_ROWS, OPT_BLAST_MIXU, OPT_BLAST_ONE, OPT_COUNT };
 int option_value(int id, int dflt);             // the option's value, or dflt when it is unset
 // true when p is aligned to `bytes`.
 static inline bool aligned(const void* p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) % bytes) == 0; }

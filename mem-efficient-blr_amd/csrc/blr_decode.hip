@@ -1283,10 +1283,9 @@ size_t decode2_region_bytes() { return (size_t)16 << 20; }
 size_t decode2_plain_bytes() { return (size_t)8 << 20; }
 
 bool decode2_applicable(const StreamBlastArgs& a) {
-  static const int enabled = env_i("BLR_DECODE2", 1);
+  const int enabled = option_value(OPT_DECODE2, 1);
   if (!enabled || a.split) return false;
-  static const int nk_on = env_i("BLR_D2_NK", 1);
-  if (a.u_layout != BLR_U_RQ && !(nk_on && a.u_layout == BLR_U_QR && a.wbits == 16)) return false;
+  if (a.u_layout != BLR_U_RQ && !(a.u_layout == BLR_U_QR && a.wbits == 16)) return false;
   if (a.wbits != 16 && (a.wbits != 8 && a.wbits != 4)) return false;
   if (a.wbits != 16 && (!a.u_scales || !a.v_scales)) return false;
   if (a.dtype != BLR_F16 && a.dtype != BLR_BF16) return false;
@@ -1307,7 +1306,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, un
                          unsigned* err_word, hipStream_t st) {
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
-  static const int rows_min_m = env_i("BLR_DECODE_ROWS_MIN_M", 2);
+  constexpr int rows_min_m = 2;
   if (M >= rows_min_m || a.wbits == 4 || a.rows_only) {   // (4-bit codes at one row too: 15.8 against 16.9 - 20.6 us on the single-row kernels)
     const int rc = decode_rows_launch(a, plain, decode2_plain_bytes(), st);
     if (rc != 1) return rc;
@@ -1326,9 +1325,9 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, un
     rc = decode3_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
     if (rc != 1) return rc;
   }
-  static const int mfma_min_m = env_i("BLR_D2_MFMA_MIN_M", 5);
+  constexpr int mfma_min_m = 5;
   if (M >= mfma_min_m && a.wbits == 16) return decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
-  static const int q_mfma_min_m = env_i("BLR_D2_Q_MFMA_MIN_M", 3);
+  constexpr int q_mfma_min_m = 3;
   if ((M > 4 || M >= q_mfma_min_m) && a.wbits != 16) {   // below that, codes stay with the vector variant
     const int rc = decode2m_blast_launch(a, region, epoch_word, arrive_word, err_word, st);
     if (rc != 1 || M > 4) return rc;                     // a shape it declines at 3 or 4 rows is still the vector variant's
@@ -1383,8 +1382,8 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, un
   } else
   // stage 2: column chunks of 8 * lpr2 outputs; k split so that the slabs cover the resident grid
   {
-    static const int e_lpr = env_i("BLR_D2_LPR2", 16), e_ks = env_i("BLR_D2_KS2", 0), e_ksmax = env_i("BLR_D2_KS2_MAX", 4);
-    int lpr = e_lpr < lpr_cap ? e_lpr : lpr_cap;
+    constexpr int ks_cap = 4;
+    int lpr = 16 < lpr_cap ? 16 : lpr_cap;
     const int vecs = (Q + EPL - 1) / EPL;
     while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
     if (lpr > 64) lpr = 64;
@@ -1393,8 +1392,8 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, un
     const int nch = (vecs + lpr - 1) / lpr;
     const int base = bo * nch;
     if (base > resident) return d2_bail(__LINE__);
-    int ks = e_ks > 0 ? e_ks : resident / base;
-    if (ks > e_ksmax) ks = e_ksmax;
+    int ks = resident / base;
+    if (ks > ks_cap) ks = ks_cap;
     if (ks > resident / base) ks = resident / base;
     if (ks < 1) ks = 1;
     int kc = (R + ks - 1) / ks;
@@ -1412,8 +1411,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, un
   }
   // stage 1: column chunks of EPL * lpr1 ranks; k split only as far as needed to engage the chip
   {
-    static const int e_lpr = env_i("BLR_D2_LPR1", 16), e_ks = env_i("BLR_D2_KS1", 0);
-    int lpr = e_lpr < lpr_cap ? e_lpr : lpr_cap;
+    int lpr = 16 < lpr_cap ? 16 : lpr_cap;
     const int vecs = (R + EPL - 1) / EPL;
     while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
     if (lpr > 64) lpr = 64;
@@ -1425,13 +1423,12 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, un
     if (base > resident) return d2_bail(__LINE__);
     // split k just far enough that a lane's share of a slice is one batch of loads
     const int ks_max = d2_ks1_max(MT);
-    int ks = e_ks > 0 ? e_ks : ((P + rpp - 1) / rpp + d2_unr1(MT) - 1) / d2_unr1(MT);
+    int ks = ((P + rpp - 1) / rpp + d2_unr1(MT) - 1) / d2_unr1(MT);
     if (ks > resident / base) ks = resident / base;
     // A workgroup that owns both a stage-1 item and a slab of U starts streaming its slab only after its stage-1
     // work and ends last: when a slightly coarser k split lets every item have a workgroup of its own, take it
     // (as long as a lane's share of a slice still fits two batches of loads).
-    static const int e_solo = env_i("BLR_D2_SOLO", 1);
-    if (e_solo && e_ks <= 0 && base + p.items2 <= resident && base * ks + p.items2 > resident) {
+    if (base + p.items2 <= resident && base * ks + p.items2 > resident) {
       const int ks_solo = (resident - p.items2) / base;
       if (((P + ks_solo - 1) / ks_solo + rpp - 1) / rpp <= 2 * d2_unr1(MT)) ks = ks_solo;
     }
@@ -1457,8 +1454,7 @@ int decode2_blast_launch(const StreamBlastArgs& a, void* region, void* plain, un
     p.rch_log2 = ilog2(rch);
     p.itemsM = (R + rch - 1) / rch;
     if (p.itemsM > resident) return d2_bail(__LINE__);
-    static const int e_depth = env_i("BLR_D2_PF_DEPTH", 4);
-    p.pf_depth = e_depth;
+    p.pf_depth = 4;
     p.pf_first = 0;
   }
   const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)(p.zrep > 1 ? p.zrep : bo) * M * R * 8, 256);
@@ -1515,10 +1511,9 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
   {
-    static const int e_ks = env_i("BLR_DM_KS1", 0);
     const int nch = (R + 127) / 128, base = b * nch;
     if (base > resident) return d2_bail(__LINE__);
-    int ks = e_ks > 0 ? e_ks : (P + DM_ROWS - 1) / DM_ROWS;       // one batch per slice if the grid allows
+    int ks = (P + DM_ROWS - 1) / DM_ROWS;       // one batch per slice if the grid allows
     if (ks > resident / base) ks = resident / base;
     if (ks > 4) ks = 4;
     if (ks < 1) ks = 1;
@@ -1532,14 +1527,14 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     p.x_vec = aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0 && kc % 8 == 0;
   }
   {
-    static const int e_ks = env_i("BLR_DM_KS2", 0), e_ksmax = env_i("BLR_DM_KS2_MAX", 4);
+    constexpr int ks_cap = 4;
     const int nch = (Q + 127) / 128, base = bo * nch;
     if (base > resident) return d2_bail(__LINE__);
     // BLAST proper (b output blocks): no k split of stage 2 - handing partial outputs of up to 16 rows between workgroups
     // costs more than the shorter slabs save (measured at every M from 5 to 16); low rank and Monarch keep the split
     const bool no_split = bo == b && bo > 1 && a.perm_per == 0;
-    int ks = e_ks > 0 ? e_ks : (no_split ? 1 : resident / base);
-    if (ks > e_ksmax) ks = e_ksmax;
+    int ks = no_split ? 1 : resident / base;
+    if (ks > ks_cap) ks = ks_cap;
     if (ks > 4) ks = 4;
     if (ks > resident / base) ks = resident / base;
     if (ks < 1) ks = 1;
@@ -1564,8 +1559,7 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
     p.rch_log2 = ilog2(rch);
     p.itemsM = ((R + rch - 1) / rch) * ((M + DM_MC - 1) / DM_MC);
     if (p.itemsM > resident) return d2_bail(__LINE__);
-    static const int e_depth = env_i("BLR_DM_PF_DEPTH", 4);
-    p.pf_depth = e_depth;
+    p.pf_depth = 4;
   }
   const size_t ybytes = align_up((size_t)p.ks1 * b * M * R * 8, 256), zbytes = align_up((size_t)(p.zrep > 1 ? p.zrep : bo) * M * (R / 2) * 8, 256);
   const size_t obytes = (size_t)(p.ks2 - 1) * bo * M * Q * 8;
@@ -1590,8 +1584,7 @@ int decode2m_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoc
 // limits K to one slab).  Returns BLR_OK, a negative status, or 1 when the call is not for this kernel.
 int slab_gemm_launch(const void* A, int64_t lda, int64_t sA, const void* B, int64_t ldb, int64_t sB, void* C, int64_t ldc, int64_t sC,
                      int M, int N, int K, int batch, int dtype, float* part, int max_slices, hipStream_t st) {
-  static const int enabled = env_i("BLR_DENSE_SLAB", 1), min_m = env_i("BLR_DENSE_SLAB_MIN_M", 1);
-  if (!enabled || M < min_m || M > 16) return 1;
+  if (!option_value(OPT_DENSE_SLAB, 1) || M < 1 || M > 16) return 1;
   if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
   if (N % 8 || ldb % 8 || sB % 8 || !aligned(B, 16) || (int64_t)K * ldb * 2 >= (1ll << 31)) return d2_bail(__LINE__);   // 16-byte pieces of a row, 32-bit buffer offsets
   if (!part || max_slices < 1) max_slices = 1;
@@ -1600,9 +1593,8 @@ int slab_gemm_launch(const void* A, int64_t lda, int64_t sA, const void* B, int6
   const int64_t base = (int64_t)nch * batch;
   // Slices: one workgroup per compute unit if its slab then fits the four register batches (512 rows: the whole slab is
   // requested at once and the partial sums stay few), otherwise two per compute unit.
-  static const int e_per_cu = env_i("BLR_DENSE_SLAB_WGS_PER_CU", 0);
   int ks = 1, kc = K;
-  for (int per_cu = e_per_cu > 0 ? e_per_cu : 1; per_cu <= (e_per_cu > 0 ? e_per_cu : 2); ++per_cu) {
+  for (int per_cu = 1; per_cu <= 2; ++per_cu) {
     ks = (int)(((int64_t)per_cu * cus + base - 1) / base);   // enough slices to give every compute unit its workgroups
     if (ks > max_slices) ks = max_slices;
     if (ks > (K + DM_ROWS - 1) / DM_ROWS) ks = (K + DM_ROWS - 1) / DM_ROWS;

@@ -582,7 +582,7 @@ double d3_stream_us(double bytes) { return 0.6 + bytes / 35e3; }
 
 int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch_word, unsigned* arrive_word,
                          unsigned* err_word, hipStream_t st) {
-  static const int enabled = env_i("BLR_DECODE3", 1);
+  const int enabled = option_value(OPT_DECODE3, 1);
   if (!enabled) return 1;
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int P = a.in_f / a.b, Q = a.out_f / bo, R = a.r, b = a.b, M = a.M;
@@ -619,7 +619,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   else if (a.s_layout == BLR_S_RIJ) { p.s_sr = (int64_t)b * b; p.s_si = b; p.s_sj = 1; }
   else { p.s_si = (int64_t)b * R; p.s_sj = R; p.s_sr = 1; }
   p.spin_limit = spin_limit_now();
-  { static const int e_xcd = env_i("BLR_XCD_ORDER", 1); p.xcd_order = e_xcd; }
+  p.xcd_order = 1;
   { const void* eb = nullptr; int ea = 0; if (epilogue_pending(&eb, &ea)) { p.ep = 1; p.bias = eb; p.act = ea; } }
   p.x_vec = aligned(a.x, 16) && a.ldx % 8 == 0 && P % 8 == 0;
   p.s_mode = 0;
@@ -644,7 +644,6 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   struct S1 { int lpr, nch, ks, kc, nb, kpad, items, n1s, nchain; double t_chain, extra_slab; };
   const double vbytes = (double)b * P * R * WBITS / 8.0;
   auto plan1 = [&](int nslab, double slab_bytes, S1& s) -> bool {
-    static const int e_ks = env_i("BLR_D3_KS1", 0);
     const int navail = resident - nslab;
     int lpr = 16;
     const int vecs = (R + EPL - 1) / EPL;
@@ -658,7 +657,6 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     {
       const int takers = D3_ITEMS * navail;
       for (int ks = 1; ks <= D3_KS1_MAX; ++ks) {
-        if (e_ks > 0 && ks != e_ks) continue;
         int kc = (int)cdiv(P, ks);
         kc = (int)cdiv(kc, rpp) * rpp;
         if ((int)cdiv(P, kc) != ks) continue;
@@ -688,19 +686,16 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   S1 s1 = {};
   {
     // stage 2 on U (bo, r, q): the cut (lanes per row, k-slices) with the smallest estimated time
-    static const int e_lpr = env_i("BLR_D3_LPR2", 0), e_ks = env_i("BLR_D3_KS2", 0);
     double best = 1e30;
     bool found = false;
     for (int lpr0 = 16; lpr0 >= 4; lpr0 >>= 1) {
-      if (e_lpr > 0 && lpr0 != e_lpr) continue;
-      if (lpr0 == 4 && WBITS == 16 && e_lpr != 4) continue;        // 64-byte pieces of a row only for codes
+      if (lpr0 == 4 && WBITS == 16) continue;        // 64-byte pieces of a row only for codes
       int lpr = lpr0;
       const int vecs = (Q + EPL - 1) / EPL;
       while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
       const int rpp = D3_NT / lpr;
       const int nch = (vecs + lpr - 1) / lpr;
       for (int ks0 = 1; ks0 <= 4; ++ks0) {
-        if (e_ks > 0 && ks0 != e_ks) continue;
         int kc = (int)cdiv(R, ks0);
         kc = (int)cdiv(kc, rpp) * rpp;
         const int ks = (int)cdiv(R, kc);

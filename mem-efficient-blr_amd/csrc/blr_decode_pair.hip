@@ -581,7 +581,7 @@ bool pair_fns(int MT, int wbits, int pfg, bool qr, bool st, int jpg, void** f1, 
 
 // Returns BLR_OK, a negative blr_status, or 1 when the call is not for these kernels.
 int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_bytes, hipStream_t st) {
-  static const int enabled = env_i("BLR_DECODE_PAIR", 1);
+  const int enabled = option_value(OPT_DECODE_PAIR, 1);
   if (!enabled) return 1;
   static const int dbg0 = env_i("BLR_D2_DEBUG", 0);
   auto decline = [&](int line) { if (dbg0) fprintf(stderr, "decode pair: not for this call (line %d)\n", line); return 1; };
@@ -622,7 +622,6 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
 
   // ---- stage 1: 128-rank chunks, k split so that an item is at most eight loads per lane; any number of workgroups ----
   {
-    static const int e_ks = env_i("BLR_DP_KS1", 0);
     int lpr = 16;
     const int vecs = (R + EPL - 1) / EPL;
     while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
@@ -636,7 +635,6 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     // on 4096 -> 4096 and 11008 -> 4096).  An item may take two batches of loads; slices are added only up to half the chip.
     while (ks < ks_max && cdiv(cdiv(P, ks), rpp) > 2 * DP_UNR1) ++ks;
     while (ks < ks_max && (int64_t)b * nch * ks < cus / 2 && cdiv(cdiv(P, ks + 1), rpp) >= 2) ++ks;
-    if (e_ks > 0) ks = e_ks < ks_max ? e_ks : ks_max;
     int kc = (int)cdiv(P, ks);
     kc = (int)cdiv(kc, rpp) * rpp;
     ks = (int)cdiv(P, kc);
@@ -648,7 +646,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     p.lpr1_log2 = ilog2(lpr); p.nch1 = fd_make((uint32_t)nch); p.bdiv = fd_make((uint32_t)b);
     p.ks1 = ks; p.kc1 = kc; p.kpad1_log2 = ilog2(kpad);
   }
-  { static const int e_xcd = env_i("BLR_XCD_ORDER", 1); p.xcd_order = e_xcd; }
+  p.xcd_order = 1;
   { const void* eb = nullptr; int ea = 0; if (epilogue_pending(&eb, &ea)) { p.ep = 1; p.bias = eb; p.act = ea; } }
   const size_t ybytes = ((size_t)p.ks1 * b * M * R * 2 + 255) / 256 * 256;
   const size_t sbytes = s_turn ? (size_t)b * bo * R * 2 : 0;
@@ -662,7 +660,6 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
 
   // ---- mix + stage 2: a slab spans the whole rank; the narrowest column chunk that keeps it within the registers ----
   {
-    static const int e_lpr = env_i("BLR_DP_LPR2", 0);
     const int cus = device_cus() > 0 ? device_cus() : 256;
     int best_lpr = 0, best_pfn = 0;
     double best = 1e30;
@@ -675,8 +672,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
       }
     }
     for (int lpr0 = 16; lpr0 >= 4 && !qr; lpr0 >>= 1) {
-      if (e_lpr > 0 && lpr0 != e_lpr) continue;
-      if (lpr0 == 4 && WBITS == 16 && e_lpr != 4) continue;        // 64-byte pieces of a row only for codes
+      if (lpr0 == 4 && WBITS == 16) continue;        // 64-byte pieces of a row only for codes
       int lpr = lpr0;
       const int vecs = (Q + EPL - 1) / EPL;
       while (lpr > 4 && lpr / 2 >= vecs) lpr /= 2;
@@ -725,8 +721,7 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
   // Monarch 15.8 -> 15.2, low rank 4096 -> 4096 (64 KiB items, four workgroups per slab) 12.4 -> 11.7 (one per slab: 12.8);
   // 4096 -> 4096 (32 KiB items) 9.2 -> 9.4 - 9.6; 4096 -> 22016 (45 MB of U) 16.6 -> 17.1 - 18.3.  Hence: items of at least
   // 60 KB, whole slabs of at most 16 loads, at most 12 MB of U and no more slabs than compute units; as many workgroups per
-  // slab (1, 2 or 4) as keep one's share within three quarters of an item.  BLR_DP_PRE / BLR_DP_PRE_SPLIT override (0: none).
-  static const int e_pre = env_i("BLR_DP_PRE", -1), e_split = env_i("BLR_DP_PRE_SPLIT", 0);
+  // slab (1, 2 or 4) as keep one's share within three quarters of an item.
   p.items1 = grid1; p.grid2 = grid2; p.qr = qr ? 1 : 0;
   {
     const double item_bytes = (double)p.kc1 * (1 << p.lpr1_log2) * 16.0;
@@ -734,10 +729,8 @@ int decode_pair_launch(const StreamBlastArgs& a, void* region, size_t region_byt
     const int cus = device_cus() > 0 ? device_cus() : 256;
     const int pfn8 = (int)cdiv(p.pfn, 8) * 8;
     int pre = (item_bytes >= 60e3 && pfn8 <= 16 && u_bytes <= 12e6 && grid2 <= cus) ? pfn8 : 0;
-    if (e_pre >= 0) { pre = (int)cdiv(e_pre, 8) * 8; if (pre > pfn8) pre = pfn8; }
     int split = 1;
     while (split < 4 && pre * 8192.0 / split > 0.75 * item_bytes && pre % (2 * split) == 0) split *= 2;
-    if ((e_split == 1 || e_split == 2 || e_split == 4) && pre % e_split == 0) split = e_split;
     p.pre_loads = pre; p.pre_split = split;
   }
   const int grid1_all = grid1 + (p.pre_loads > 0 ? (int)cdiv(grid2, 8) * 8 * p.pre_split : 0);

@@ -575,7 +575,6 @@ int rows_plan(RowsParams& p, int batch, int dtype, int wbits, bool nk) {
   if (p.mtiles > 1 && p.rounds > 1) return 1;          // more rows than one tile only with the whole factor slice in registers
   p.kw = (int)cdiv(cdiv(p.K, DR_WAVES * p.rounds), 32) * 32;
   const int cus = device_cus() > 0 ? device_cus() : 256;
-  static const int e_npc = env_i("BLR_DR_NPC", 0);
   if (nk) {
     // column groups of 16 per chunk (at most 8): as many as keep the busiest compute unit's bytes lowest
     int best = 8; double best_t = 1e30;
@@ -586,12 +585,11 @@ int rows_plan(RowsParams& p, int batch, int dtype, int wbits, bool nk) {
     p.npc = best;
     p.nch = fd_make((uint32_t)cdiv(p.N, 16 * p.npc));
   } else {
-    p.npc = e_npc > 0 && e_npc <= 16 ? e_npc : plan_pieces(batch, p.K, p.N, wbits, cus);
+    p.npc = plan_pieces(batch, p.K, p.N, wbits, cus);
     p.nch = fd_make((uint32_t)cdiv(p.N / 8, p.npc));
   }
   if ((int64_t)batch * p.nch.d >= 65536) return 1;
-  static const int e_xcd = env_i("BLR_DR_XCD", 1);
-  p.xcd_span = (e_xcd && (batch * p.nch.d) % 8 == 0) ? (uint32_t)(batch * p.nch.d / 8) : 0u;
+  p.xcd_span = ((batch * p.nch.d) % 8 == 0) ? (uint32_t)(batch * p.nch.d / 8) : 0u;
   return BLR_OK;
 }
 
@@ -606,8 +604,7 @@ int rows_launch(RowsParams p, int batch, int dtype, int wbits, bool nk, hipStrea
 // or the factor is too small to matter.
 RowsPrefetch rows_prefetch_plan(const RowsParams& p, int batch, int wbits, bool nk) {
   RowsPrefetch f = {};
-  static const int enabled = env_i("BLR_DR_PREFETCH", 1);
-  static const int e_kb = env_i("BLR_DR_PREFETCH_KB", 96);
+  static const int enabled = 1;
   if (!enabled) return f;
   const int64_t w_bytes = (int64_t)batch * p.K * p.N * wbits / 8;
   if (w_bytes < (1 << 20)) return f;
@@ -628,7 +625,7 @@ RowsPrefetch rows_prefetch_plan(const RowsParams& p, int batch, int wbits, bool 
   f.nch = p.nch; f.xcd_span = p.xcd_span;
   f.nblocks2 = (uint32_t)batch * p.nch.d;
   // per workgroup: what a compute unit draws during the launch (about 35 GB/s for 2 - 3 us), and an XCD's share within 3 MB of its L2
-  int64_t budget = (int64_t)e_kb * 1024;
+  int64_t budget = (int64_t)96 * 1024;
   const int64_t per_xcd = (int64_t)3 << 20;
   if (budget * ((f.nblocks2 + 7) / 8) > per_xcd) budget = per_xcd / ((f.nblocks2 + 7) / 8);
   f.budget16 = (uint32_t)(budget / 16);
@@ -639,7 +636,7 @@ RowsPrefetch rows_prefetch_plan(const RowsParams& p, int batch, int wbits, bool 
 }  // namespace
 
 int decode_rows_launch(const StreamBlastArgs& a, void* region, size_t region_bytes, hipStream_t st) {
-  static const int enabled = env_i("BLR_DECODE_ROWS", 1);
+  const int enabled = option_value(OPT_DECODE_ROWS, 1);
   if (!enabled) return 1;
   const int bo = a.bo > 0 ? a.bo : a.b;
   const int b = a.b, M = a.M, R = a.r, P = a.in_f / a.b, Q = a.out_f / bo;
@@ -749,7 +746,7 @@ size_t dense_rows_bytes(int M, int in_f, int out_f, int dtype) {
 
 int dense_rows_launch(const void* x, int64_t ldx, const void* W, void* out, int64_t ldo, int M, int in_f, int out_f, int dtype,
                       void* ws, size_t ws_bytes, hipStream_t st) {
-  static const int enabled = env_i("BLR_DENSE_ROWS", 1);
+  const int enabled = option_value(OPT_DENSE_ROWS, 1);
   const int bi = dense_slices(in_f);
   if (!enabled || !dense_rows_wanted(M, out_f) || (dtype != BLR_F16 && dtype != BLR_BF16) || !bi || out_f % 8) return 1;
   if (bi > 1 && (ldo != out_f || !ws || ws_bytes < dense_rows_bytes(M, in_f, out_f, dtype) || !aligned(out, 8))) return 1;

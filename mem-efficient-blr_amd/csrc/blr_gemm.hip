@@ -790,13 +790,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g, int tiles_m) 
 }
 
 template <typename T, int BM, int BN, bool B_KN>
-static void* mfma_kernel_ptr(int pd, bool ep) {
-  if (ep) return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 2, true>;
-  switch (pd) {
-    case 1: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 1>;
-    case 3: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 3>;
-    default: return (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 2>;
-  }
+static void* mfma_kernel_ptr(bool ep) {          // (two k-tiles of global loads in flight: PD = 2)
+  return ep ? (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 2, true> : (void*)gemm_mfma_kernel<T, BM, BN, B_KN, 2>;
 }
 
 template <typename T, int BM, int BN>
@@ -808,10 +803,8 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
   int c_vec = g.epi == EPI_PLAIN && g.cn == 1 && aligned(g.C, 16) && g.ldc % 8 == 0 && g.sC % 8 == 0 && g.N % 8 == 0 &&
               (!g.bias || aligned(g.bias, 16)) && (!g.gate || (aligned(g.gate, 16) && g.ld_gate % 8 == 0)) && (!g.resid || (aligned(g.resid, 16) && g.ld_resid % 8 == 0));
   size_t lds = 2 * sizeof(GemmSmem<T, BM, BN>);
-  // k-tiles of global loads kept in flight (tuning aid: BLR_GEMM_PD = 1, 2 or 3)
-  static const int pd = [] { const char* e = getenv("BLR_GEMM_PD"); return e ? atoi(e) : 2; }();
   const bool ep = g.bias != nullptr || g.act != 0 || g.gate != nullptr || g.resid != nullptr;
-  void* fn = g.b_kn ? mfma_kernel_ptr<T, BM, BN, true>(pd, ep) : mfma_kernel_ptr<T, BM, BN, false>(pd, ep);
+  void* fn = g.b_kn ? mfma_kernel_ptr<T, BM, BN, true>(ep) : mfma_kernel_ptr<T, BM, BN, false>(ep);
   static std::mutex mu;
   static std::set<void*> raised;
   {
@@ -822,13 +815,10 @@ static int launch_mfma(const GemmArgs& g, hipStream_t st) {
       raised.insert(fn);
     }
   }
-  // tuning aids: BLR_GEMM_XCD=0 keeps the linear tile order, BLR_GEMM_GM sets the strip height in tiles
-  static const int xcd_on = [] { const char* e = getenv("BLR_GEMM_XCD"); return e ? atoi(e) : 1; }();
-  static const int gm_env = [] { const char* e = getenv("BLR_GEMM_GM"); return e ? atoi(e) : 4; }();
   const int64_t total = (int64_t)tiles_m * tiles_n * g.batch;
   if (total > (1ll << 30)) { set_error("gemm: too many tiles"); return BLR_ERR_UNSUPPORTED; }
-  int per_xcd = xcd_on ? (int)cdiv(total, 8) : 0;
-  int group_m = gm_env < 1 ? 1 : gm_env;
+  int per_xcd = (int)cdiv(total, 8);
+  int group_m = 4;
   dim3 grid((unsigned)(per_xcd > 0 ? per_xcd * 8 : total));
   GemmArgs ga = g;
   void* args[] = {&ga, &tiles_m, &tiles_n, &a_vec, &b_vec, &c_vec, &per_xcd, &group_m};
@@ -920,12 +910,10 @@ static int launch_ring(const GemmArgs& g, hipStream_t st) {
       raised.insert(fn);
     }
   }
-  static const int xcd_on = [] { const char* e = getenv("BLR_GEMM_XCD"); return e ? atoi(e) : 1; }();
-  static const int gm_env = [] { const char* e = getenv("BLR_GEMM_GM"); return e ? atoi(e) : 4; }();
   const int64_t total = (int64_t)tiles_m * tiles_n * g.batch;
   if (total > (1ll << 30)) { set_error("gemm: too many tiles"); return BLR_ERR_UNSUPPORTED; }
-  int per_xcd = xcd_on ? (int)cdiv(total, 8) : 0;
-  int group_m = gm_env < 1 ? 1 : gm_env;
+  int per_xcd = (int)cdiv(total, 8);
+  int group_m = 4;
   // a side job: one thread per item, in workgroups ahead of the tiles (a multiple of eight of them, so that tile u stays on XCD u % 8)
   int side_wgs = 0;
   if (!PARTIAL && g.side.items > 0 && g.side_taken) side_wgs = (int)(cdiv(cdiv(g.side.items, NWV * 64), 8) * 8);
@@ -943,7 +931,6 @@ template <typename T>
 static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   // Bigger tiles do more MFMA work per LDS byte (the 2x2 wave grid reads 0.5 fragments per MFMA at
   // 256x256, 0.75 at 256x128, 1 at 128x128) but need enough tiles to fill the 256 CUs.
-  static const int force = [] { const char* e = getenv("BLR_GEMM_TILE"); return e ? atoi(e) : 0; }();
   const int cus = device_cus() > 0 ? device_cus() : 256;
   int64_t t256 = cdiv(g.M, 256) * cdiv(g.N, 256) * g.batch;
   int64_t t128 = cdiv(g.M, 256) * cdiv(g.N, 128) * g.batch;
@@ -953,7 +940,7 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   // BLR_GEMM_RING_WAVES = 4 or 8 the workgroup size of the two larger ones - options that tests switch with
   // blr_set_option).
   const int ring = option_value(OPT_GEMM_RING, 1);
-  if (ring > 0 && force == 0 && ring_ok(g) && g.epi == EPI_PLAIN && g.splitk_ws && g.batch == 1 && g.cn == 1 && !g.sat8 && !g.bias && !g.act && !g.gate && !g.resid) {
+  if (ring > 0 && ring_ok(g) && g.epi == EPI_PLAIN && g.splitk_ws && g.batch == 1 && g.cn == 1 && !g.sat8 && !g.bias && !g.act && !g.gate && !g.resid) {
     // few tiles, long reduction: slices of K as the batch of the partial-sum kernel, then one pass that adds them up
     int kc = 0;
     const int splits = option_value(OPT_GEMM_SPLITK, 1) == 0 ? 1 : splitk_plan(g.M, g.N, g.K, &kc);
@@ -975,7 +962,7 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     set_error("gemm: a pair of tiles (SiLU-gated halves) needs 16-byte aligned operands, K and the half width multiples of 8, a plain row-major output");
     return BLR_ERR_UNSUPPORTED;
   }
-  if ((ring > 0 && force == 0 && ring_ok(g)) || g.pair) {
+  if ((ring > 0 && ring_ok(g)) || g.pair) {
     int rt = option_value(OPT_GEMM_RING_TILE, 0);
     const int64_t fill = ((int64_t)cus * 9 + 9) / 10;
     const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
@@ -1014,11 +1001,8 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       return per_cu == 2 ? launch_ring<T, 128, 128, true>(g, st) : launch_ring<T, 128, 128>(g, st);
     }
   }
-  // the register-staged kernel at 256x256 needs more registers than there are and spills: only on request (BLR_GEMM_TILE=256)
-  if (force == 256 && t256 > 0) return launch_mfma<T, 256, 256>(g, st);
   // short reductions are dominated by filling and draining a tile: two smaller workgroups per CU overlap those
-  static const int small_k = [] { const char* e = getenv("BLR_GEMM_SMALL_K"); return e ? atoi(e) : 1024; }();
-  if (force == 128256 || (force == 0 && g.M >= 256 && t128 >= cus && g.K > small_k)) return launch_mfma<T, 256, 128>(g, st);
+  if (g.M >= 256 && t128 >= cus && g.K > 1024) return launch_mfma<T, 256, 128>(g, st);
   return launch_mfma<T, 128, 128>(g, st);
 }
 
@@ -1280,16 +1264,12 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
   int r_chunks = (int)cdiv(R, 64);
   if (dtype != BLR_F32 && b <= 16 && R % 8 == 0 && aligned(Y, 16) && aligned(Z, 16)) {
     size_t lds = (size_t)b * b * MIX_LDR * 2;
-    static const int mpw_env = [] { const char* e = getenv("BLR_MIX_MPW"); return e ? atoi(e) : 0; }();
     // S may be fetched in 16-byte pieces if every piece starts on a 16-byte boundary
     const int s_vec = aligned(S, 16) && ((s_sr == 1 && s_si % 8 == 0 && s_sj % 8 == 0) ||
                                          (s_sj == 1 && s_si % 8 == 0 && s_sr % 8 == 0));
-    static const bool h2 = [] { const char* e = getenv("BLR_MIX_H2"); return e ? atoi(e) != 0 : true; }();
-    static const int mb_env = [] { const char* e = getenv("BLR_MIX_MB"); return e ? atoi(e) : 2; }();
-    const bool use_h2 = dtype == BLR_F16 && h2 && !sat8;
-    const int mb = use_h2 && mb_env == 2 && M >= 64 ? 2 : 1;
+    const bool use_h2 = dtype == BLR_F16 && !sat8;
+    const int mb = use_h2 && M >= 64 ? 2 : 1;
     int m_per_wg = 32 * mb;                        // one pass of the 32 row slots: more, smaller workgroups measured fastest
-    if (mpw_env > 0) m_per_wg = mpw_env;
     dim3 grid(r_chunks, (unsigned)cdiv(M, m_per_wg));
     if (use_h2 && mb == 2)
       if (b == 16) hipLaunchKernelGGL((blast_mix_h2_kernel<true, 2>), grid, dim3(256), lds, st, (const f16*)Y, (const f16*)S, (f16*)Z, M, b, R, s_si, s_sj, s_sr, m_per_wg, s_vec);

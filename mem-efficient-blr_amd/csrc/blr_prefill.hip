@@ -302,14 +302,13 @@ int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, 
   // 12 pieces = 384 (1.5 rounds) 34.8 us, 9 = 512 (2 rounds) 36.2 us.
   const int pieces = R / 8;
   const int cus = device_cus() > 0 ? device_cus() : 256;
-  static const int e_npc = env_i("BLR_YM_NPC", 0);
   int best_npc = 16; double best_cost = -1.0;
   for (int npc = 16; npc >= 4; --npc) {
     const double x = (double)(cdiv(pieces, npc) * cdiv(M, YM_BM)) / cus;
     const double cost = 0.5 * (std::ceil(x) + x) * (12 + npc);
     if (best_cost < 0 || cost < best_cost - 1e-9) { best_cost = cost; best_npc = npc; }
   }
-  p.npc = e_npc > 0 && e_npc <= 16 ? e_npc : best_npc;
+  p.npc = best_npc;
   const int nrt = (int)cdiv(pieces, p.npc), nmt = (int)cdiv(M, YM_BM);
   if ((int64_t)nrt * nmt >= 65536 || nmt >= 65536) return 1;
   p.nmt = fd_make((uint32_t)nmt);
@@ -327,8 +326,7 @@ int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, 
   const int BR = p.npc * 8;
   const size_t lds_y = (size_t)(b / 2) * (YM_BM * (BR + 4) + 16) * 4;
   const size_t lds_z = (size_t)b * 16 * (BR / 2 + 4) * 4;                 // the rows of one product group on their way out
-  static const int e_stage = env_i("BLR_YM_STAGE", 1);
-  const bool stage = e_stage && lds_y + lds_z <= 160 * 1024;
+  const bool stage = lds_y + lds_z <= 160 * 1024;
   const size_t lds = lds_y + (stage ? lds_z : 0);
   const int fi = (dtype == BLR_F16 ? 0 : 2) + (stage ? 1 : 0);
   void* const fns[4] = {(void*)blast_ymix_kernel<f16, false>, (void*)blast_ymix_kernel<f16, true>,
@@ -624,7 +622,7 @@ int blast_mixu_launch(const void* Y, const void* S, const void* U, void* out, in
   p.bias = ep.bias; p.act = ep.act; p.gate = ep.gate; p.gate_rows = ep.gate ? ep.gate_rows : 1; p.ld_gate = ep.ld_gate;
   p.resid = ep.resid; p.ld_resid = ep.ld_resid;
   p.Ut = job.Ut; p.Sp = job.Sp;
-  { static const int e_rot = env_i("BLR_MIXU_ROTATE", 1); p.rotate = e_rot; }
+  p.rotate = 1;
   if (!prepared) {
     const unsigned tg = (unsigned)cdiv(job.items, 256);
     if (dtype == BLR_F16) hipLaunchKernelGGL(mixu_prep_kernel<f16>, dim3(tg), dim3(256), 0, st, job);

@@ -981,8 +981,8 @@ int env_int(const char* name, int dflt) {
   const char* e = getenv(name);
   return e ? atoi(e) : dflt;
 }
-// Workgroups kept resident per CU (tuning aid: BLR_STREAM_WGS_PER_CU).
-int wgs_per_cu() { static int v = env_int("BLR_STREAM_WGS_PER_CU", 2); return v < 1 ? 1 : v; }
+// Workgroups kept resident per CU.
+int wgs_per_cu() { return 2; }
 // Largest M for which the BLAST mix is recomputed inside the last phase instead of run as its own phase.
 int mix_inline_max_m() { return 0; }
 // Largest M for which BLAST stage 1 adds its S-weighted result straight into Z with float atomics
@@ -1017,8 +1017,8 @@ size_t lds_bytes_for(const StreamParams& p) {
 int mt_for(int M) { return M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16))); }
 
 // Choose the KN tiling: lanes per row, k-chunk and split count, aiming at `target` work items.
-// Smallest M served by the matrix-core KN variant (tuning aid: BLR_KN_MFMA_MIN_M).
-int kn_mfma_min_m() { static int v = env_int("BLR_KN_MFMA_MIN_M", 5); return v; }
+// Smallest M served by the matrix-core KN variant.
+int kn_mfma_min_m() { return 5; }
 
 bool plan_kn(PhaseDesc& d, int MT, int target, int M = 0) {
   const int vecs = (d.N + 7) / 8;
@@ -1313,7 +1313,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
   }
   if (a.op == 1) {                             // low rank: z = x A (in, r); out = z B (r, out)
     WsLayout w = ws_carve(a.ws, (size_t)a.M * a.r);
-    static const int rows_min_m = env_int("BLR_LOWRANK_ROWS_MIN_M", 2);
+    constexpr int rows_min_m = 2;
     if (!a.split && a.M >= rows_min_m) {
       // From two rows up: the three-launch matrix-core path, low rank being BLAST with the input cut into 16 (or 8, 4, 2) slices of
       // rows of A, one output block and S = 1 (the mix is the sum over the slices).
@@ -1329,7 +1329,7 @@ int stream_generic_launch(const StreamGenericArgs& a, hipStream_t st) {
         if (rc != 1) return rc;
       }
     }
-    static const int slab_min_m = env_int("BLR_LOWRANK_SLAB_MIN_M", 5);
+    constexpr int slab_min_m = 5;
     if (!a.split && a.M >= slab_min_m && a.r % 8 == 0 && a.out_f % 8 == 0) {
       // From a handful of rows up, two launches of the slab kernel, each followed by the sum of its k-slices: z = x A goes
       // to the first staging buffer as T, then out = z B.  Four launches, 19-29 us whatever M is; the single launch below

@@ -83,3 +83,23 @@ def test_no_cpu_fallback():
     x = torch.zeros(1, 1, 4); U = torch.zeros(2, 2, 2); V = torch.zeros(2, 2, 2); S = torch.zeros(2, 2, 2)
     with pytest.raises(_lib.BlrError):
         K.triton_blast_full_fp32(x, U, V, S)
+
+
+def test_run_time_options_are_named_and_range_checked():
+    """blr_set_option knows every switch of the library by name and refuses values outside its range (no kernel launch is
+    involved: the table lives on the host)."""
+    from triton_funcs import _lib
+    lib = _lib.lib()
+    ok = {"BLR_GEMM_RING": (0, 1, 2), "BLR_GEMM_RING_TILE": (0, 256256, 256128, 128128), "BLR_GEMM_RING_PER_CU": (0, 1, 2),
+          "BLR_GEMM_RING_WAVES": (4, 8), "BLR_GEMM_SPLITK": (0, 1), "BLR_DECODE2": (0, 1), "BLR_DECODE3": (0, 1),
+          "BLR_DECODE_PAIR": (0, 1, 2), "BLR_DECODE_ROWS": (0, 1), "BLR_DENSE_SLAB": (0, 1), "BLR_DENSE_ROWS": (0, 1),
+          "BLR_BLAST_MIXU": (0, 1, 2), "BLR_BLAST_ONE": (0, 1)}
+    for name, values in ok.items():
+        for v in values:
+            assert lib.blr_set_option(name.encode(), v, 0) == 0, (name, v)
+        for bad in (-1, 3, 100, 12345):
+            if bad not in values:
+                assert lib.blr_set_option(name.encode(), bad, 0) == -1, (name, bad)
+                assert name.encode() in lib.blr_last_error()
+        assert lib.blr_set_option(name.encode(), 0, 1) == 0            # back to "not set"
+    assert lib.blr_set_option(b"BLR_NO_SUCH_SWITCH", 1, 0) == -1

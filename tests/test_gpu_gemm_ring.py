@@ -22,8 +22,9 @@ def ring_forced(request):
     """Selects the kernel for every legal problem, with one of its variants: tile shape / ring depth (1 deep rings, 2
     shallow ones and more workgroups per compute unit) / waves per workgroup (256x256 only)."""
     from triton_funcs import _lib as L
-    parts = (request.param.split("/") + ["1", "4"])[:3]
-    with L.options(BLR_GEMM_RING=2, BLR_GEMM_RING_TILE=parts[0], BLR_GEMM_RING_PER_CU=parts[1], BLR_GEMM_RING_WAVES=parts[2]):
+    parts = request.param.split("/")
+    per_cu, waves = (parts[1] if len(parts) > 1 else "1"), (parts[2] if len(parts) > 2 else "4")
+    with L.options(BLR_GEMM_RING=2, BLR_GEMM_RING_TILE=parts[0], BLR_GEMM_RING_PER_CU=per_cu, BLR_GEMM_RING_WAVES=waves):
         yield request.param
 
 
