@@ -47,11 +47,13 @@ typedef enum { BLR_U_RQ = 0, BLR_U_QR = 1 } blr_u_layout;
  * (b2=i, b1=j, r) for the torch baseline layout (reference layer.py:193-200).               */
 typedef enum { BLR_S_JIR = 0, BLR_S_RIJ = 1, BLR_S_IJR = 2 } blr_s_layout;
 
-/* Which kernel family serves a call.  AUTO picks STREAM for M <= 16 (HBM-bound) and TILED above. */
+/* Which kernel family serves a call.  AUTO picks STREAM for M <= 16 of f16 / bf16 (HBM-bound) and TILED otherwise. */
 typedef enum {
   BLR_ALGO_AUTO = 0,
-  BLR_ALGO_STREAM = 1,        /* persistent streaming kernel, one launch, M <= 16, f16/bf16 */
-  BLR_ALGO_TILED = 2,         /* MFMA tiled GEMMs; the rank-space intermediates go through HBM unless the fused first half pays */
+  BLR_ALGO_STREAM = 1,        /* the few-row kernels, M <= 16, f16/bf16: one to three launches chosen by row count and shape (one or two
+                                 at M = 1, three on the matrix cores at 2..16 rows; a single persistent launch for what those decline) */
+  BLR_ALGO_TILED = 2,         /* up to 128 rows: the three-launch few-row kernels over tiles of 16 rows; above: MFMA tiled GEMMs with the
+                                 rank-space intermediates in the workspace (narrow blocks: fused launches that keep Y and / or Z on chip) */
   BLR_ALGO_FUSED = 3,         /* BLAST: x V and the mix in one launch, Y = x V only ever in LDS; then the batched GEMM with U.
                                  Needs f16/bf16, 4 | b <= 16, 8 | in_f / b, 8 | r, y_out == NULL; else BLR_ERR_UNSUPPORTED */
   BLR_ALGO_STREAM_SPLIT = 4   /* the STREAM phases as separate launches (no grid barrier)   */
@@ -98,9 +100,12 @@ typedef enum { BLR_OP_BLAST = 0, BLR_OP_MONARCH = 1, BLR_OP_LOW_RANK = 2, BLR_OP
  * (4,000,000, about a second).  Meant for tests of the give-up path.                          */
 int blr_workspace_status(void* ws, size_t ws_bytes, void* stream);
 void blr_set_spin_limit(unsigned polls);
-/* Tuning options the tests switch at run time (no counterpart in the reference): BLR_GEMM_RING, BLR_GEMM_RING_TILE,
- * BLR_GEMM_RING_PER_CU, BLR_GEMM_RING_WAVES, BLR_GEMM_SPLITK.  Each starts from the environment variable of its name
- * (read once); unset != 0 returns it to "not set".  Returns BLR_ERR_BAD_ARG for an unknown name.                  */
+/* The run-time switches of the library (no counterpart in the reference), all of them: the GEMM variant - BLR_GEMM_RING
+ * (0..2), BLR_GEMM_RING_TILE (0, 256256, 256128, 128128), BLR_GEMM_RING_PER_CU (0..2), BLR_GEMM_RING_WAVES (4, 8),
+ * BLR_GEMM_SPLITK (0, 1) - and kernel families on / off - BLR_DECODE2, BLR_DECODE3, BLR_DECODE_ROWS, BLR_DENSE_SLAB,
+ * BLR_DENSE_ROWS, BLR_BLAST_ONE (0, 1), BLR_DECODE_PAIR, BLR_BLAST_MIXU (0..2); a family that is off hands its calls to the
+ * next one that serves them.  Each starts from the environment variable of its name (read once; a value out of range is
+ * ignored); unset != 0 returns it to "not set".  Returns BLR_ERR_BAD_ARG for an unknown name or a value out of range.  */
 int blr_set_option(const char* name, int value, int unset);
 
 const char* blr_last_error(void);
@@ -140,8 +145,10 @@ int blr_blast_i8act_fwd(const void* x, int64_t ldx, const void* U, const void* V
  * and fp16 per-output-channel scales.  Both factors are stored (k, n)-ordered, the order in which
  * the kernels stream them: U codes (b, r, q[/2]) + u_scales (b, q); V codes (b, p, r[/2]) +
  * v_scales (b, r); S (r, i, j) of dtype.  Served behind the name triton_blast_bmm_int8_fp16
- * (reference triton_funcs/blast_sym_quant_kernels.py:558-580).  r % 32 == 0 and q % 8 == 0.
- * M <= 16 streams the codes; larger M expands them to dtype in the workspace first.           */
+ * (reference triton_funcs/blast_sym_quant_kernels.py:558-580).  r % 8 == 0 and (out_f / b) % 8 == 0.
+ * Up to 128 rows the kernels stream the codes and widen them in registers; larger M expands them to dtype in the
+ * workspace first and runs the tiled kernels.  The quantizer and its code layout are this library's own: the reference
+ * has no weight quantizer.                                                                                          */
 size_t blr_blast_q_workspace_bytes(int M, int in_f, int out_f, int b, int r, int bits);
 int blr_blast_q_fwd(const void* x, int64_t ldx,
                     const void* u_codes, const void* u_scales,
@@ -217,10 +224,11 @@ double blr_mfma_probe_flops(int iters);
  * out = act(op(x) + bias): what the callers do right after the operator - the bias add of the wrapper
  * modules (reference models/wrappers.py:176-177) and the activation that follows the first MLP linear
  * (GELU-tanh in DiT, reference DiT/models.py:111-112; SiLU in Llama).  bias: out_f values of dtype or NULL;
- * act: blr_act.  The other arguments are those of the entry point without the suffix.  On the tiled path
- * (M > 16) bias and activation are applied while the last GEMM writes its tile out (to the result rounded
- * to dtype, as the callers' separate kernels would), so the M x out_f round trip of those kernels
- * disappears; on the streaming path (M <= 16) a small elementwise launch follows the operator.   */
+ * act: blr_act.  The other arguments are those of the entry point without the suffix.  Above 128 rows bias and
+ * activation are applied while the last GEMM writes its tile out (to the result rounded to dtype, as the callers'
+ * separate kernels would), so the M x out_f round trip of those kernels disappears; below, BLAST and Monarch apply them
+ * in the output stage of their last few-row kernel (dense: at 17..128 rows with one slice), and what no kernel fuses is
+ * finished by a small elementwise launch after the operator.                                                        */
 int blr_blast_fwd_ep(const void* x, int64_t ldx, const void* U, const void* V, const void* S,
                      void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
                      int dtype, int u_layout, int s_layout, int algo,
