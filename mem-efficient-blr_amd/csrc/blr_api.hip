@@ -301,7 +301,7 @@ const char* const kOptNames[OPT_COUNT] = {"BLR_GEMM_RING", "BLR_GEMM_RING_TILE",
 bool opt_value_ok(int id, int v) {
   switch (id) {
     case OPT_GEMM_RING: case OPT_GEMM_RING_PER_CU: case OPT_DECODE_PAIR: case OPT_BLAST_MIXU: return v >= 0 && v <= 2;
-    case OPT_GEMM_RING_TILE: return v == 0 || v == 256256 || v == 256128 || v == 128128;
+    case OPT_GEMM_RING_TILE: return v == 0 || v == 256256 || v == 256128 || v == 256096 || v == 128128;
     case OPT_GEMM_RING_WAVES: return v == 4 || v == 8;
     default: return v == 0 || v == 1;
   }

@@ -433,12 +433,16 @@ __device__ unsigned long long g_trace_gemm[4096 * 8];
 #define TRG(i) do {} while (0)
 #endif
 
-template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false, int NWV = 4, bool PARTIAL = false>
+// BNC: the columns of a tile that are computed and written.  Below BN (96 of 128) the stages keep their 128-column layout and the
+// four waves sit above each other, 64 rows x 96 columns each: for output widths like 288 that 128-column tiles cover with a
+// quarter of their matrix instructions wasted.
+template <typename T, bool B_KN, int BM, int BN, bool EP = false, bool SHALLOW = false, int NWV = 4, bool PARTIAL = false, int BNC = BN>
 __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m, int side_wgs) {
   constexpr int NA = ring_na<SHALLOW>(), NB = ring_nb<SHALLOW>();
   constexpr int ASTG = BM * 64, BSTG = BN * 64, BRING = NA * ASTG;   // stage sizes, start of the B ring
-  constexpr int WGN = (NWV == 8 && BN == 256) ? 4 : 2, WGM = NWV / WGN;   // waves: 2 x 2, or 2 x 4 / 4 x 2 (two per SIMD)
-  constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+  static_assert(BNC == BN || (BNC == 96 && BN == 128 && NWV == 4), "narrow tiles: 96 of 128 columns on four waves");
+  constexpr int WGN = BNC != BN ? 1 : (NWV == 8 && BN == 256) ? 4 : 2, WGM = NWV / WGN;   // waves: 2 x 2, or 2 x 4 / 4 x 2 (two per SIMD), or 4 x 1
+  constexpr int WM = BM / WGM, WN = BNC / WGN, TM = WM / 32, TN = WN / 32;
   constexpr int LA = BM / (16 * NWV), LB = BN / (16 * NWV);   // 1 KiB direct loads per wave and k tile
   constexpr int LT = LA + LB;
   constexpr int RB = BN * 2, CPR = BN / 8, RPI = 1024 / RB;
@@ -469,7 +473,7 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   const int rem = ut - strip * group_m * tiles_n;
   const int gm_here = min(group_m, tiles_m - strip * group_m);
   const int tm_i = strip * group_m + rem % gm_here, tn_i = rem / gm_here;
-  const int m0 = tm_i * BM, n0 = tn_i * BN;
+  const int m0 = tm_i * BM, n0 = tn_i * BNC;
 
   const char* Ab0 = reinterpret_cast<const char*>(g.A) + (int64_t)bt * g.sA * 2;
   const char* Bb0 = reinterpret_cast<const char*>(g.B) + (int64_t)bt * g.sB * 2;
@@ -698,14 +702,14 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
   if (g.cn != 1) {
     // interleaved columns (column n of batch bt is element n * cn + bt of the row): two-byte stores, lanes along n, so
     // that an instruction touches cn * 128 contiguous bytes; the other batches fill the gaps
-    for (int v = tid; v < BM * BN; v += NWV * 64) {
-      const int row = v / BN, col = v - row * BN;
+    for (int v = tid; v < BM * BNC; v += NWV * 64) {
+      const int row = v / BNC, col = v - row * BNC;
       const int gr = m0 + row, gc = n0 + col;
       if (gr < g.M && gc < g.N) C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + (int64_t)gc * g.cn] = cs[row * CLD + col];
     }
     return;
   }
-  constexpr int VPR = BN / 8;
+  constexpr int VPR = BNC / 8;
   for (int v = tid; v < BM * VPR; v += NWV * 64) {
     const int row = v / VPR, cvec = (v - row * VPR) * 8;
     const int gr = m0 + row, gc = n0 + cvec;
@@ -889,17 +893,17 @@ static bool ring_ok(const GemmArgs& g) {
   return true;
 }
 
-template <typename T, int BM, int BN, bool SHALLOW = false, int NWV = 4, bool PARTIAL = false>
+template <typename T, int BM, int BN, bool SHALLOW = false, int NWV = 4, bool PARTIAL = false, int BNC = BN>
 static int launch_ring(const GemmArgs& g, hipStream_t st) {
-  int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
+  int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BNC);
   const size_t lds = ring_lds_bytes<BM, BN, SHALLOW>();
   const bool ep = g.bias != nullptr || g.act != 0 || g.gate != nullptr || g.resid != nullptr;
   void* fn;
   if constexpr (PARTIAL)
     fn = g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW, NWV, true> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW, NWV, true>;
   else
-    fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true, SHALLOW, NWV> : (void*)gemm_ring_kernel<T, false, BM, BN, true, SHALLOW, NWV>)
-            : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW, NWV> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW, NWV>);
+    fn = ep ? (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, true, SHALLOW, NWV, false, BNC> : (void*)gemm_ring_kernel<T, false, BM, BN, true, SHALLOW, NWV, false, BNC>)
+            : (g.b_kn ? (void*)gemm_ring_kernel<T, true, BM, BN, false, SHALLOW, NWV, false, BNC> : (void*)gemm_ring_kernel<T, false, BM, BN, false, SHALLOW, NWV, false, BNC>);
   static std::mutex mu;
   static std::set<void*> raised;
   {
@@ -964,6 +968,8 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   }
   if ((ring > 0 && ring_ok(g)) || g.pair) {
     int rt = option_value(OPT_GEMM_RING_TILE, 0);
+    const bool auto_tile = rt == 0, narrow = rt == 256096;
+    if (narrow) rt = 256128;
     const int64_t fill = ((int64_t)cus * 9 + 9) / 10;
     const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
     int per_cu = option_value(OPT_GEMM_RING_PER_CU, 0);
@@ -995,6 +1001,10 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       }
       if (rt == 256128) {
         if (per_cu != 2 && option_value(OPT_GEMM_RING_WAVES, 4) == 8) return launch_ring<T, 256, 128, false, 8>(g, st);
+        // 96-column tiles where they cover the width with at most 4/5 of what 128-column tiles compute (288 = 3 x 96 against 3 x 128)
+        // (BLR_GEMM_RING_TILE = 256096 asks for them, 256128 keeps them away)
+        if (g.cn == 1 && (narrow || (auto_tile && per_cu == 2 && cdiv(g.N, 96) * 96 * 5 <= cdiv(g.N, 128) * 128 * 4)))
+          return launch_ring<T, 256, 128, true, 4, false, 96>(g, st);
         return per_cu == 2 ? launch_ring<T, 256, 128, true>(g, st) : launch_ring<T, 256, 128>(g, st);
       }
       if (!per_cu) per_cu = r128 >= 2 * (int64_t)cus ? 2 : 1;     // three shallow workgroups per compute unit, or two deep ones

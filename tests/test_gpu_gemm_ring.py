@@ -17,7 +17,7 @@ from gpu_util import assert_close, back, blast_inputs, dev, rounded, say
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["256256", "256256/1/8", "256128", "256128/1/8", "256128/2", "128128", "128128/2"])
+@pytest.fixture(params=["256256", "256256/1/8", "256128", "256128/1/8", "256128/2", "256096", "128128", "128128/2"])
 def ring_forced(request):
     """Selects the kernel for every legal problem, with one of its variants: tile shape / ring depth (1 deep rings, 2
     shallow ones and more workgroups per compute unit) / waves per workgroup (256x256 only)."""
