@@ -294,7 +294,7 @@ using namespace blr;
 namespace blr {
 namespace {
 constexpr int kOptUnset = -2147483647 - 1;
-const char* const kOptNames[OPT_COUNT] = {"BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU", "BLR_GEMM_RING_WAVES", "BLR_GEMM_SPLITK",
+const char* const kOptNames[OPT_COUNT] = {"BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU", "BLR_GEMM_RING_WAVES", "BLR_GEMM_RING_BK", "BLR_GEMM_SPLITK",
                                           "BLR_DECODE2", "BLR_DECODE3", "BLR_DECODE_PAIR", "BLR_DECODE_ROWS", "BLR_DENSE_SLAB", "BLR_DENSE_ROWS",
                                           "BLR_BLAST_MIXU", "BLR_BLAST_ONE"};
 // what each option may be set to: a range, or (BLR_GEMM_RING_TILE, BLR_GEMM_RING_WAVES) a short list; anything else is refused
@@ -303,6 +303,7 @@ bool opt_value_ok(int id, int v) {
     case OPT_GEMM_RING: case OPT_GEMM_RING_PER_CU: case OPT_DECODE_PAIR: case OPT_BLAST_MIXU: return v >= 0 && v <= 2;
     case OPT_GEMM_RING_TILE: return v == 0 || v == 256256 || v == 256128 || v == 256096 || v == 128128;
     case OPT_GEMM_RING_WAVES: return v == 4 || v == 8;
+    case OPT_GEMM_RING_BK: return v == 32 || v == 64;
     default: return v == 0 || v == 1;
   }
 }

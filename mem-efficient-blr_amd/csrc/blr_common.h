@@ -85,9 +85,9 @@ unsigned spin_limit_now();
 bool epilogue_pending(const void** bias, int* act);   // (false when a gate or a residual is armed: only the tiled path fuses those)
 void epilogue_taken();
 // Every run-time switch of the library (blr_set_option): each starts from the environment variable of its name, read once, and
-// is range-checked where it is set.  The first five pick the GEMM variant, the rest switch a kernel family off (0) so that the
+// is range-checked where it is set.  The first six pick the GEMM variant, the rest switch a kernel family off (0) so that the
 // call falls through to the next one that serves it - for A/B measurements and as a way out should a kernel misbehave.
-enum { OPT_GEMM_RING = 0, OPT_GEMM_RING_TILE, OPT_GEMM_RING_PER_CU, OPT_GEMM_RING_WAVES, OPT_GEMM_SPLITK,
+enum { OPT_GEMM_RING = 0, OPT_GEMM_RING_TILE, OPT_GEMM_RING_PER_CU, OPT_GEMM_RING_WAVES, OPT_GEMM_RING_BK, OPT_GEMM_SPLITK,
        OPT_DECODE2, OPT_DECODE3, OPT_DECODE_PAIR, OPT_DECODE_ROWS, OPT_DENSE_SLAB, OPT_DENSE_ROWS, OPT_BLAST_MIXU, OPT_BLAST_ONE, OPT_COUNT };
 int option_value(int id, int dflt);             // the option's value, or dflt when it is unset
 // true when p is aligned to `bytes`.

@@ -433,6 +433,66 @@ __device__ unsigned long long g_trace_gemm[4096 * 8];
 #define TRG(i) do {} while (0)
 #endif
 
+// The tile's way out of a ring kernel: accumulators -> LDS (as T, the stages are done with) -> whole rows to memory, through the
+// output stage where there is one.  acc[i][j][4 q + e] is row (lane & 31), column 8 q + 4 (lane >> 5) + e of the 32 x 32 block
+// (i, j) of the wave's WM x WN part (the products were formed transposed).  hf: which tile of a pair this is.
+template <typename T, int BM, int BN, int BNC, int NWV, int WM, int WN, int TM, int TN, bool EP, bool PAIRS>
+__device__ __forceinline__ void ring_write_out(const GemmArgs& g, f32x16 (&acc)[TM][TN], unsigned char* smem, T* C, int m0, int n0, int wm, int wn,
+                                               int bt, int hf) {
+  using V8 = typename TypeTraits<T>::vec8;
+  const int tid = threadIdx.x, lane = tid & 63;
+  __syncthreads();                                                   // the epilogue reuses the tile memory
+
+  constexpr int CLD = BN + 8;
+  T* cs = reinterpret_cast<T*>(smem);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int row = wm * WM + i * 32 + (lane & 31);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int col = wn * WN + j * 32 + q * 8 + (lane >> 5) * 4;
+        typename TypeTraits<T>::vec4 v4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v4[e] = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][4 * q + e]) : acc[i][j][4 * q + e]);
+        *reinterpret_cast<typename TypeTraits<T>::vec4*>(&cs[row * CLD + col]) = v4;
+      }
+    }
+  __syncthreads();
+  TRG(3);
+  if (g.cn != 1) {
+    // interleaved columns (column n of batch bt is element n * cn + bt of the row): two-byte stores, lanes along n, so
+    // that an instruction touches cn * 128 contiguous bytes; the other batches fill the gaps
+    for (int v = tid; v < BM * BNC; v += NWV * 64) {
+      const int row = v / BNC, col = v - row * BNC;
+      const int gr = m0 + row, gc = n0 + col;
+      if (gr < g.M && gc < g.N) C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + (int64_t)gc * g.cn] = cs[row * CLD + col];
+    }
+    return;
+  }
+  constexpr int VPR = BNC / 8;
+  for (int v = tid; v < BM * VPR; v += NWV * 64) {
+    const int row = v / VPR, cvec = (v - row * VPR) * 8;
+    const int gr = m0 + row, gc = n0 + cvec;
+    if (gr < g.M && gc < g.N) {
+      V8 v = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
+      if (EP) {
+        // (a pair: the first tile leaves silu(. + bias) where the result goes; the second is multiplied onto it by the thread that
+        // stored it - the same element index v in both passes)
+        if (!PAIRS || hf == 0) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc, gr);
+        else v = ep_pair_up<T>(g, v, (int64_t)bt * g.sC + gc + g.pair_dbias, &C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]);
+      }
+      if (g.epi == EPI_MONARCH_SCATTER) {            // column c of entry bt -> block c / per, column bt * per + c % per
+        const int d = gc / g.per;
+        *reinterpret_cast<V8*>(&C[(int64_t)d * g.sL + (int64_t)gr * g.ldc + (int64_t)bt * g.per + (gc - d * g.per)]) = v;
+      } else {
+        *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = v;
+      }
+    }
+  }
+}
+
 // BNC: the columns of a tile that are computed and written.  Below BN (96 of 128) the stages keep their 128-column layout and the
 // four waves sit above each other, 64 rows x 96 columns each: for output widths like 288 that 128-column tiles cover with a
 // quarter of their matrix instructions wasted.
@@ -679,61 +739,284 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
       }
     return;
   }
-  __syncthreads();                                                   // the epilogue reuses the tile memory
-
-  constexpr int CLD = BN + 8;
-  T* cs = reinterpret_cast<T*>(smem);
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int row = wm * WM + i * 32 + (lane & 31);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int col = wn * WN + j * 32 + q * 8 + (lane >> 5) * 4;
-        typename TypeTraits<T>::vec4 v4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v4[e] = TypeTraits<T>::from_f32(g.sat8 ? sat8_rne(acc[i][j][4 * q + e]) : acc[i][j][4 * q + e]);
-        *reinterpret_cast<typename TypeTraits<T>::vec4*>(&cs[row * CLD + col]) = v4;
-      }
-    }
-  __syncthreads();
-  TRG(3);
-  if (g.cn != 1) {
-    // interleaved columns (column n of batch bt is element n * cn + bt of the row): two-byte stores, lanes along n, so
-    // that an instruction touches cn * 128 contiguous bytes; the other batches fill the gaps
-    for (int v = tid; v < BM * BNC; v += NWV * 64) {
-      const int row = v / BNC, col = v - row * BNC;
-      const int gr = m0 + row, gc = n0 + col;
-      if (gr < g.M && gc < g.N) C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + (int64_t)gc * g.cn] = cs[row * CLD + col];
-    }
-    return;
-  }
-  constexpr int VPR = BNC / 8;
-  for (int v = tid; v < BM * VPR; v += NWV * 64) {
-    const int row = v / VPR, cvec = (v - row * VPR) * 8;
-    const int gr = m0 + row, gc = n0 + cvec;
-    if (gr < g.M && gc < g.N) {
-      V8 v = *reinterpret_cast<const V8*>(&cs[row * CLD + cvec]);
-      if (EP) {
-        // (a pair: the first tile leaves silu(. + bias) where the result goes; the second is multiplied onto it by the thread that
-        // stored it - the same element index v in both passes)
-        if (!PAIRS || hf == 0) v = ep_vector<T>(g, v, (int64_t)bt * g.sC + gc, gr);
-        else v = ep_pair_up<T>(g, v, (int64_t)bt * g.sC + gc + g.pair_dbias, &C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]);
-      }
-      if (g.epi == EPI_MONARCH_SCATTER) {            // column c of entry bt -> block c / per, column bt * per + c % per
-        const int d = gc / g.per;
-        *reinterpret_cast<V8*>(&C[(int64_t)d * g.sL + (int64_t)gr * g.ldc + (int64_t)bt * g.per + (gc - d * g.per)]) = v;
-      } else {
-        *reinterpret_cast<V8*>(&C[(int64_t)bt * g.sC + (int64_t)gr * g.ldc + gc]) = v;
-      }
-    }
-  }
+  ring_write_out<T, BM, BN, BNC, NWV, WM, WN, TM, TN, EP, PAIRS>(g, acc, smem, C, m0, n0, wm, wn, bt, hf);
   if (hf + 1 < halves) __syncthreads();              // the staged tile has been read: the rings may be filled again
   }  // tiles of a pair
   TRG(4);
 }
 
+
+// ---- the same kernel with operand stages of 64 k ---------------------------------------------------------------------------
+// The vector memory path moves whole 128-byte lines from the L2: a load instruction that takes 64 bytes from each of 16 rows of
+// a K-contiguous operand (a stage of 32 k) gets half of what it could - measured with every workgroup of the chip reading from
+// an L2-resident buffer: 18-20 TB/s for 16 rows x 64 bytes per instruction against 35-37 TB/s for 8 rows x 128 bytes.  Here a
+// stage is 64 k: an instruction takes the 128 bytes (eight 16-byte chunks) of each of 8 rows, lanes 8 r .. 8 r + 7 on row r, and
+// lane (r, s) fetches chunk s ^ r, so that chunk c of row r lies at position c ^ (r & 7) of the row's 128 bytes in LDS: the
+// fragment reads of eight consecutive rows (same chunk) then cover all banks.  A (k, n) operand stage is 64 rows of BN n, laid out
+// as above.  NST stages (two or three) of both operands form one ring with one barrier per step of 64 k; a step is four sub-steps
+// of 16 k (one fragment of each 32-row block).
+// What the loop is made of, per step of a 256 x 256 tile on eight waves (two per SIMD): 64 matrix instructions per SIMD (2048
+// cycles of its matrix pipe), 192 KiB of fragment reads and 64 KiB of operand loads into LDS - the LDS is as busy as the matrix
+// pipe.  In-kernel cycle counts: 2890 cycles per step with the fragment reads of a sub-step issued as one burst ahead of its
+// products and the barrier at the end of the step, 2570 with one read or load between two products and the barrier between the
+// third and the fourth sub-step (behind it a wave still holds a sub-step of products in registers, under which the first fragments
+// of the next stage arrive).  The clock drops as the pipe fills up (1.35 -> 1.27 GHz under the board's power limit with random
+// operands), so the second gain in cycles is worth 4 % in time.
+template <int BM, int BN, int NST>
+constexpr size_t ring64_lds_bytes() {
+  size_t st = (size_t)NST * (BM + BN) * 128, ep = (size_t)BM * (BN + 8) * 2;
+  return st > ep ? st : ep;
+}
+
+template <typename T, bool B_KN, int BM, int BN, bool EP, int NWV, int NST, int PER_CU>
+__global__ __launch_bounds__(NWV * 64, (NWV / 4) * PER_CU) void gemm_ring64_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m, int side_wgs) {
+  constexpr int ASTG = BM * 128, BSTG = BN * 128, BRING = NST * ASTG;
+  constexpr int WGN = (NWV == 8 && BN == 256) ? 4 : 2, WGM = NWV / WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+  constexpr int LA = BM / (8 * NWV), LB = BN / (8 * NWV), LT = LA + LB;     // 1 KiB loads per wave and stage
+  constexpr int RB = BN * 2, CPR = BN / 8, RPI = 1024 / RB;                 // (k, n) operand: bytes per k row, chunks per row, rows per load
+  constexpr int NMF = TM * TN;
+  constexpr int SLOTS = NMF;                                                // matrix instructions between which a step's loads go out
+  static_assert(NMF >= TM + TN, "a sub-step has a gap for every fragment read");
+  static_assert(LA >= 1 && LB >= 1 && NST >= 2, "tile too small for the workgroup");
+  using V8 = typename TypeTraits<T>::vec8;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int tiles = tiles_m * tiles_n;
+  TRG(0);
+  int u = blockIdx.x;
+  if (side_wgs > 0) {
+    if (u < side_wgs) {
+      for (int64_t idx = (int64_t)u * (NWV * 64) + tid; idx < g.side.items; idx += (int64_t)side_wgs * (NWV * 64)) side_prep_item<T>(g.side, idx);
+      return;
+    }
+    u -= side_wgs;
+  }
+  if (per_xcd > 0) u = (u & 7) * per_xcd + (u >> 3);
+  if (u >= tiles * g.batch) return;
+  const int bt = u / tiles;
+  const int ut = u - bt * tiles;
+  const int strip = ut / (group_m * tiles_n);
+  const int rem = ut - strip * group_m * tiles_n;
+  const int gm_here = min(group_m, tiles_m - strip * group_m);
+  const int tm_i = strip * group_m + rem % gm_here, tn_i = rem / gm_here;
+  const int m0 = tm_i * BM, n0 = tn_i * BN;
+
+  const char* Ab0 = reinterpret_cast<const char*>(g.A) + (int64_t)bt * g.sA * 2;
+  const char* Bb0 = reinterpret_cast<const char*>(g.B) + (int64_t)bt * g.sB * 2;
+  T* C = reinterpret_cast<T*>(g.C);
+  constexpr bool PAIRS = EP && !(BM == 256 && BN == 256 && NWV == 4);
+  const int halves = (PAIRS && g.pair) ? 2 : 1;
+  for (int hf = 0; hf < halves; ++hf) {
+  const char* Ab = Ab0 + (PAIRS ? (int64_t)hf * g.pair_dA * 2 : 0);
+  const char* Bb = Bb0 + (PAIRS ? (int64_t)hf * g.pair_dB * 2 : 0);
+
+  const int KT = (g.K + 63) >> 6;
+  const int ktail = g.K & 63;                         // valid k of the last stage when it is partial: a multiple of 8
+
+  // lane (r8, s8) of a K-contiguous load: row r8 of the instruction's eight, LDS position s8 of its 128 bytes, global chunk s8 ^ r8
+  const int r8 = lane >> 3, s8 = lane & 7, c8 = s8 ^ r8;
+  uint32_t a_off[LA], b_off[LB];
+#pragma unroll
+  for (int i = 0; i < LA; ++i) a_off[i] = (uint32_t)(min(m0 + (i * NWV + wave) * 8 + r8, g.M - 1) * g.lda * 2 + c8 * 16);
+#pragma unroll
+  for (int i = 0; i < LB; ++i) {
+    if (B_KN) {
+      const int krow = (i * NWV + wave) * RPI + lane / CPR;
+      const int chunk = (lane % CPR) ^ ((krow & 3) << 1);
+      b_off[i] = (uint32_t)(krow * g.ldb * 2 + min(n0 + chunk * 8, g.N - 8) * 2);
+    } else {
+      b_off[i] = (uint32_t)(min(n0 + (i * NWV + wave) * 8 + r8, g.N - 1) * g.ldb * 2 + c8 * 16);
+    }
+  }
+  // a partial last stage: chunks (rows of a (k, n) stage) past ktail are replaced by valid ones; what lands there meets zeros
+  const int cmax = max((ktail >> 3) - 1, 0), rmax = max(ktail - 1, 0);
+  const uint32_t tail_kc = (uint32_t)((c8 - min(c8, cmax)) * 16);
+  uint32_t tail_kn[LB];
+#pragma unroll
+  for (int i = 0; i < LB; ++i) {
+    const int krow = (i * NWV + wave) * RPI + lane / CPR;
+    tail_kn[i] = B_KN ? (uint32_t)((krow - min(krow, rmax)) * g.ldb * 2) : tail_kc;
+  }
+  const uint32_t lds0 = ring_lds_addr(smem + wave * 1024);
+  auto issue = [&](int li, int tile, int stg, bool partial) {       // load li (A first, then B) of stage `tile` into ring slot stg
+    if (li < LA) {
+      ring_load_lds(Ab + (int64_t)tile * 128, a_off[li] - (partial ? tail_kc : 0u), lds0 + stg * ASTG + li * (NWV * 1024));
+    } else {
+      const int lb = li - LA;
+      const char* Bp = B_KN ? Bb + (int64_t)tile * 64 * g.ldb * 2 : Bb + (int64_t)tile * 128;
+      ring_load_lds(Bp, b_off[lb] - (partial ? tail_kn[lb] : 0u), lds0 + BRING + stg * BSTG + lb * (NWV * 1024));
+    }
+  };
+
+  // fragment addresses: row rl of a K-contiguous stage starts at (rl >> 3) KiB + (rl & 7) * 128; sub-step q, lane half h wants
+  // chunk 2 q + h, which lies at position (2 q + h) ^ (rl & 7), and rl & 7 = lane & 7
+  const int half = lane >> 5;
+  uint32_t rowA[TM], rowB[TN], xo[4];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int rl = wm * WM + i * 32 + (lane & 31);
+    rowA[i] = (uint32_t)(((rl >> 3) << 10) + ((rl & 7) << 7));
+  }
+  const int g4 = lane >> 4, i16 = lane & 15;
+  if (B_KN) {
+    const int chunk0 = wn * WN / 8 + (g4 & 1) * 2 + ((i16 & 3) >> 1);
+    const int swz = (i16 >> 2) << 1;
+    const uint32_t kn_base = (uint32_t)(((g4 >> 1) * 8 + (i16 >> 2)) * RB + (i16 & 1) * 8);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) rowB[j] = kn_base + (uint32_t)(((chunk0 + 4 * j) ^ swz) << 4);
+  } else {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int rl = wn * WN + j * 32 + (lane & 31);
+      rowB[j] = (uint32_t)(((rl >> 3) << 10) + ((rl & 7) << 7));
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) xo[q] = (uint32_t)(((2 * q + half) ^ (lane & 7)) << 4);
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  V8 af[2][TM], bf[2][TN];
+  auto frags = [&](int stg, int q, int set) {
+    const unsigned char* sta = smem + stg * ASTG;
+    const unsigned char* st = smem + BRING + stg * BSTG;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[set][i] = *reinterpret_cast<const V8*>(sta + rowA[i] + xo[q]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      if (B_KN) {
+        union { V8 v; s16x4 h[2]; } w;
+        w.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(st + rowB[j] + (q * 16) * RB));
+        w.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(st + rowB[j] + (q * 16 + 4) * RB));
+        bf[set][j] = w.v;
+      } else {
+        bf[set][j] = *reinterpret_cast<const V8*>(st + rowB[j] + xo[q]);
+      }
+    }
+  };
+  // fragment number idx of a sub-step, in the order the products want them: A 0, all of B, the rest of A
+  auto frag_one = [&](int stg, int q, int set, int idx) {
+    const unsigned char* sta = smem + stg * ASTG;
+    const unsigned char* st = smem + BRING + stg * BSTG;
+    if (idx == 0 || idx > TN) {
+      const int i = idx == 0 ? 0 : idx - TN;
+      af[set][i] = *reinterpret_cast<const V8*>(sta + rowA[i] + xo[q]);
+    } else {
+      const int j = idx - 1;
+      if (B_KN) {
+        union { V8 v; s16x4 h[2]; } w;
+        w.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(st + rowB[j] + (q * 16) * RB));
+        w.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(st + rowB[j] + (q * 16 + 4) * RB));
+        bf[set][j] = w.v;
+      } else {
+        bf[set][j] = *reinterpret_cast<const V8*>(st + rowB[j] + xo[q]);
+      }
+    }
+  };
+  auto mfma_one = [&](int set, int idx) {              // (operands swapped: the product comes out transposed, see the kernel above)
+    const int i = idx / TN, j = idx % TN;
+    acc[i][j] = TypeTraits<T>::mfma32(bf[set][j], af[set][i], acc[i][j]);
+  };
+  auto zero_tail = [&](int set, int q) {               // a partial last stage: the A fragment of chunk 2 q + half is past ktail
+    if ((2 * q + half) * 8 >= ktail) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) af[set][i][e] = (T)0.0f;
+    }
+  };
+
+  // All NST stages go out before the loop.  Step t: sub-steps 0, 1 and 2 run while the fragments of sub-steps 1, 2 and 3 are read;
+  // once those are in registers nobody needs stage t in LDS any more, and that is where the step's one barrier stands.  The loads
+  // of stage t + NST go out behind it, into the slot of stage t, between the products of sub-step 3.
+#pragma unroll
+  for (int s = 0; s < NST; ++s) {
+    const int tc = min(s, KT - 1);
+    const bool partial = ktail && tc == KT - 1;
+#pragma unroll
+    for (int li = 0; li < LT; ++li) issue(li, tc, s, partial);
+  }
+  __builtin_amdgcn_s_waitcnt(ring_vmcnt((NST - 1) * LT));
+  __builtin_amdgcn_s_barrier();
+  TRG(1);
+  frags(0, 0, 0);
+#ifdef BLR_TRACE
+  uint64_t trw_v = 0, trw_b = 0;
+  const uint64_t trw_0 = __builtin_amdgcn_s_memtime();
+#endif
+  int cs = 0;                                         // ring slot of stage t
+  for (int t = 0; t < KT; ++t) {
+    const int tn = min(t + NST, KT - 1);
+    const bool pn = ktail && tn == KT - 1;
+    const bool last_partial = ktail && t == KT - 1;
+    const int nq = last_partial ? (ktail + 15) >> 4 : 4;             // sub-steps with anything to add
+    const int nx = cs + 1 == NST ? 0 : cs + 1;
+    auto slot = [&](int sidx) {
+      if (sidx < SLOTS && (sidx * LT) / SLOTS != ((sidx + 1) * LT) / SLOTS) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int li = (sidx * LT) / SLOTS; li < ((sidx + 1) * LT) / SLOTS; ++li) issue(li, tn, cs, pn);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // A sub-step: its products, between them - one per gap - the fragment reads of the next sub-step (a wave cannot issue a
+    // product while it issues something else, and a burst of reads or loads leaves the matrix pipe idle when the SIMD's other wave
+    // is in the same burst), and in the last sub-step the loads of stage t + NST.
+    auto substep = [&](int set, bool live, int stg_next, int q_next, bool loads) {
+#pragma unroll
+      for (int m = 0; m < NMF; ++m) {
+        if (live) mfma_one(set, m);
+        if (m < TM + TN) frag_one(stg_next, q_next, set ^ 1, m);
+        if (loads) slot(m);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    if (last_partial) zero_tail(0, 0);
+    substep(0, true, cs, 1, false);
+    if (last_partial) zero_tail(1, 1);
+    substep(1, nq > 1, cs, 2, false);
+    if (last_partial) zero_tail(0, 2);
+    substep(0, nq > 2, cs, 3, false);
+    // the step's barrier: stage t is in registers, stage t + 1 has landed
+#ifdef BLR_TRACE
+    const uint64_t tw0 = __builtin_amdgcn_s_memtime();
+#endif
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(ring_vmcnt((NST - 2) * LT));   // (later stages may still be out)
+#ifdef BLR_TRACE
+    const uint64_t tw1 = __builtin_amdgcn_s_memtime();
+#endif
+    __builtin_amdgcn_s_barrier();
+#ifdef BLR_TRACE
+    const uint64_t tw2 = __builtin_amdgcn_s_memtime();
+    trw_v += tw1 - tw0; trw_b += tw2 - tw1;
+#endif
+    __builtin_amdgcn_sched_barrier(0);
+    if (last_partial) zero_tail(1, 3);
+    substep(1, nq > 3, nx, 0, true);
+    cs = nx;
+  }
+  __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
+  TRG(2);
+#ifdef BLR_TRACE
+  if (tid == 0 && blockIdx.x < 4096) {               // wave 0: cycles waiting for its loads, at the barrier, and in the whole loop
+    g_trace_gemm[blockIdx.x * 8 + 5] = trw_v; g_trace_gemm[blockIdx.x * 8 + 6] = trw_b; g_trace_gemm[blockIdx.x * 8 + 7] = __builtin_amdgcn_s_memtime() - trw_0;
+  }
+#endif
+  ring_write_out<T, BM, BN, BN, NWV, WM, WN, TM, TN, EP, PAIRS>(g, acc, smem, C, m0, n0, wm, wn, bt, hf);
+  if (hf + 1 < halves) __syncthreads();
+  }  // tiles of a pair
+  TRG(4);
+}
 
 // ---- fp32 verification GEMM: 64x64 tile, 16x16 threads, 4x4 outputs per thread ---------------
 template <bool B_KN>
@@ -931,6 +1214,39 @@ static int launch_ring(const GemmArgs& g, hipStream_t st) {
   return BLR_OK;
 }
 
+template <typename T, int BM, int BN, int NWV, int NST, int PER_CU>
+static int launch_ring64(const GemmArgs& g, hipStream_t st) {
+  int tiles_m = (int)cdiv(g.M, BM), tiles_n = (int)cdiv(g.N, BN);
+  const size_t lds = ring64_lds_bytes<BM, BN, NST>();
+  const bool ep = g.bias != nullptr || g.act != 0 || g.gate != nullptr || g.resid != nullptr;
+  void* fn = ep ? (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, true, NWV, NST, PER_CU> : (void*)gemm_ring64_kernel<T, false, BM, BN, true, NWV, NST, PER_CU>)
+                : (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, false, NWV, NST, PER_CU> : (void*)gemm_ring64_kernel<T, false, BM, BN, false, NWV, NST, PER_CU>);
+  static std::mutex mu;
+  static std::set<void*> raised;
+  {
+    std::lock_guard<std::mutex> lk(mu);
+    if (!raised.count(fn)) {
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) { set_error("gemm: cannot raise LDS limit: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+      raised.insert(fn);
+    }
+  }
+  const int64_t total = (int64_t)tiles_m * tiles_n * g.batch;
+  if (total > (1ll << 30)) { set_error("gemm: too many tiles"); return BLR_ERR_UNSUPPORTED; }
+  int per_xcd = (int)cdiv(total, 8);
+  int group_m = 4;
+  int side_wgs = 0;
+  if (g.side.items > 0 && g.side_taken) side_wgs = (int)(cdiv(cdiv(g.side.items, NWV * 64), 8) * 8);
+  if (side_wgs > 4096) side_wgs = 4096;
+  dim3 grid((unsigned)(per_xcd * 8 + side_wgs));
+  GemmArgs ga = g;
+  void* args[] = {&ga, &tiles_m, &tiles_n, &per_xcd, &group_m, &side_wgs};
+  hipError_t e = hipLaunchKernel(fn, grid, dim3(NWV * 64), args, lds, st);
+  if (e != hipSuccess) { set_error("gemm_ring64: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  if (side_wgs > 0) *g.side_taken = 1;
+  return BLR_OK;
+}
+
 template <typename T>
 static int pick_mfma(const GemmArgs& g, hipStream_t st) {
   // Bigger tiles do more MFMA work per LDS byte (the 2x2 wave grid reads 0.5 fragments per MFMA at
@@ -995,6 +1311,17 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     }
     if (g.pair && rt <= 0) rt = 128128;
     if (rt > 0 && (ring > 1 || g.pair || (g.M >= 96 && g.K >= 64))) {
+      // Stages of 64 k (plain row-major output only): by default for single products with a reduction of a thousand or more - the
+      // batched products of BLAST have short reductions and live on two workgroups per compute unit overlapping each other's tile
+      // start-up and write-out, which the larger stages leave no LDS for (2048 rows: dense 4096 -> 22016 355 -> 335 us,
+      // 11008 -> 4096 207 -> 174 us; BLAST 4096 -> 22016 186 -> 201 us; DiT-XL/2 with dense layers 11.67 -> 11.04 ms, with BLAST
+      // layers 11.76 -> 12.25 ms).  BLR_GEMM_RING_BK = 32 / 64 decides for every problem.
+      if (option_value(OPT_GEMM_RING_BK, g.batch == 1 && g.K >= 1024 ? 64 : 32) == 64 && g.cn == 1) {
+        const bool w8 = option_value(OPT_GEMM_RING_WAVES, 8) == 8;
+        if (rt == 256256) return !w8 && !g.pair ? launch_ring64<T, 256, 256, 4, 2, 1>(g, st) : launch_ring64<T, 256, 256, 8, 2, 1>(g, st);
+        if (rt == 256128) return w8 ? launch_ring64<T, 256, 128, 8, 3, 1>(g, st) : launch_ring64<T, 256, 128, 4, 3, 1>(g, st);
+        return per_cu == 1 ? launch_ring64<T, 128, 128, 4, 3, 1>(g, st) : launch_ring64<T, 128, 128, 4, 2, 2>(g, st);
+      }
       if (rt == 256256) {
         // eight waves (2 x 4, wave tile 128 x 64, two per SIMD) hide each other's barrier and LDS waits: the default
         return option_value(OPT_GEMM_RING_WAVES, 8) == 4 && !g.pair ? launch_ring<T, 256, 256>(g, st) : launch_ring<T, 256, 256, false, 8>(g, st);

@@ -17,14 +17,16 @@ from gpu_util import assert_close, back, blast_inputs, dev, rounded, say
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["256256", "256256/1/8", "256128", "256128/1/8", "256128/2", "256096", "128128", "128128/2"])
+@pytest.fixture(params=["256256", "256256/1/8", "256128", "256128/1/8", "256128/2", "256096", "128128", "128128/2",
+                        "256256/1/8/64", "256128/1/8/64", "256128/1/4/64", "128128/1/4/64", "128128/2/4/64"])
 def ring_forced(request):
     """Selects the kernel for every legal problem, with one of its variants: tile shape / ring depth (1 deep rings, 2
-    shallow ones and more workgroups per compute unit) / waves per workgroup (256x256 only)."""
+    shallow ones and more workgroups per compute unit) / waves per workgroup / k per operand stage (32, or 64: the
+    kernel whose loads take whole 128-byte lines)."""
     from triton_funcs import _lib as L
     parts = request.param.split("/")
-    per_cu, waves = (parts[1] if len(parts) > 1 else "1"), (parts[2] if len(parts) > 2 else "4")
-    with L.options(BLR_GEMM_RING=2, BLR_GEMM_RING_TILE=parts[0], BLR_GEMM_RING_PER_CU=per_cu, BLR_GEMM_RING_WAVES=waves):
+    per_cu, waves, bk = (parts[1] if len(parts) > 1 else "1"), (parts[2] if len(parts) > 2 else "4"), (parts[3] if len(parts) > 3 else "32")
+    with L.options(BLR_GEMM_RING=2, BLR_GEMM_RING_TILE=parts[0], BLR_GEMM_RING_PER_CU=per_cu, BLR_GEMM_RING_WAVES=waves, BLR_GEMM_RING_BK=bk):
         yield request.param
 
 
