@@ -296,7 +296,7 @@ def main():
     g_dn = graph_of([dn[i % 3][0] for i in range(12)])
     dn_us = time_graph(g_dn, 12)
     dn_flops = 2.0 * 2048 * i_f * o_f
-    roofline_prefill = {"bound": "mfma", "kernel": "gemm_ring_kernel<f16, 256x256> (dense gate_up 4096->22016, M=2048: one launch)",
+    roofline_prefill = {"bound": "mfma", "kernel": "gemm_ring64_kernel<f16, 256x256, 8 waves, stages of 64 k> (dense gate_up 4096->22016, M=2048: one launch)",
                         "achieved": round(dn_flops / (dn_us * 1e-6) / 1e12, 1), "peak": MFMA_PEAK / 1e12, "unit": "TFLOP/s",
                         "frac": round(dn_flops / (dn_us * 1e-6) / MFMA_PEAK, 4), "us_per_launch": round(dn_us, 2),
                         "algorithmic_flops": dn_flops, "traffic": None}
