@@ -292,14 +292,17 @@ def main():
 
     # second roofline object: the dominant kernel at M = 2048, the ring GEMM (one launch = the dense gate_up layer), MFMA bound
     i_f, o_f, _ = LAYERS["gate_up"]
-    dn = [mk_dense(2048, i_f, o_f) for _ in range(3)]
-    g_dn = graph_of([dn[i % 3][0] for i in range(12)])
-    dn_us = time_graph(g_dn, 12)
+    # (48 launches per replay over four copies, as in the layer table: the card takes some milliseconds of matrix work to settle
+    # on the clock its power limit allows, and a replay of a dozen launches read 6 % slower than the table's row of the same kernel)
+    dn = [mk_dense(2048, i_f, o_f) for _ in range(4)]
+    g_dn = graph_of([dn[i % 4][0] for i in range(48)])
+    dn_us = time_graph(g_dn, 48)
     dn_flops = 2.0 * 2048 * i_f * o_f
     roofline_prefill = {"bound": "mfma", "kernel": "gemm_ring64_kernel<f16, 256x256, 8 waves, stages of 64 k> (dense gate_up 4096->22016, M=2048: one launch)",
                         "achieved": round(dn_flops / (dn_us * 1e-6) / 1e12, 1), "peak": MFMA_PEAK / 1e12, "unit": "TFLOP/s",
                         "frac": round(dn_flops / (dn_us * 1e-6) / MFMA_PEAK, 4), "us_per_launch": round(dn_us, 2),
-                        "algorithmic_flops": dn_flops, "traffic": None}
+                        "algorithmic_flops": dn_flops, "algorithmic_bytes": 2 * (2048 * i_f + i_f * o_f + 2048 * o_f),
+                        "traffic": traffic_from_profile(PREFILL_PROFILE, "dense_traffic_bytes_per_launch"), "traffic_source": PREFILL_PROFILE}
     del g_dn, dn
     torch.cuda.empty_cache()
 
@@ -307,9 +310,9 @@ def main():
     # rank-space mix, GEMM Z U), its algorithmic flops over the event time of the whole call; traffic = HBM bytes of the three
     # launches from the committed counter summary, against the algorithmic bytes of the call
     i_f, o_f, r_gu = LAYERS["gate_up"]
-    bp = [mk_blast(2048, i_f, o_f, r_gu, L.U_RQ, L.S_JIR) for _ in range(3)]
-    g_bp = graph_of([bp[i % 3][0] for i in range(12)])
-    bp_us = time_graph(g_bp, 12)
+    bp = [mk_blast(2048, i_f, o_f, r_gu, L.U_RQ, L.S_JIR) for _ in range(4)]
+    g_bp = graph_of([bp[i % 4][0] for i in range(48)])
+    bp_us = time_graph(g_bp, 48)
     bp_bytes, bp_flops = blast_bytes_flops(2048, i_f, r_gu, o_f)
     roofline_blast_prefill = {"bound": "mfma", "kernel": "BLAST gate_up 4096->22016 r=1024 b=16, M=2048: gemm_ring_kernel (x V) + blast_mix_h2_kernel + gemm_ring_kernel (Z U)",
                               "achieved": round(bp_flops / (bp_us * 1e-6) / 1e12, 1), "peak": MFMA_PEAK / 1e12, "unit": "TFLOP/s",
