@@ -233,7 +233,8 @@ int blr_blast_fwd_ep(const void* x, int64_t ldx, const void* U, const void* V, c
                      void* out, int64_t ldo, int M, int in_f, int out_f, int b, int r,
                      int dtype, int u_layout, int s_layout, int algo,
                      void* ws, size_t ws_bytes, void* stream, const void* bias, int act);
-/* BLR_ACT_SILU_MUL (no reference kernel: SURVEY of the callers' step after the path - Llama's act(gate) * up): above 128 rows
+/* BLR_ACT_SILU_MUL (no reference kernel: it is the step Llama's MLP takes right after this path, act(gate) * up, on the
+ * fused gate_up layer that reference configs/layers/llama7b.gate_up_proj.yaml:1-8 names): above 128 rows
  * of f16 / bf16, BLAST (even b), low rank and dense compute the tiles of the gate half and of the up half of an output position
  * in one work item of the last GEMM and write only the product, so the (M, out_f) intermediate never exists; everything else
  * (few rows, Monarch, fp32) computes the full-width result into the TAIL of the workspace and finishes with one elementwise
