@@ -75,6 +75,32 @@ def test_blast_through_ring_kernel(b, p, q, r, M, name, dtype, ring_forced):
     assert_close(out, back(other), dtype, "ring vs register-staged kernel", scale=0.5)
 
 
+def test_seeded_random_shapes_through_every_variant(ring_forced):
+    """Shapes nobody chose: per kernel variant a seeded draw of dense problems ((k, n)-ordered weights) and of BLAST calls through
+    the bmm names (U K-contiguous, two or three blocks, so that the second product has a reduction of r) - row counts
+    that end inside a tile, widths and reductions that are any multiple of 8, reductions on either side of a stage (32 / 64 k)
+    and of the ring depth."""
+    from triton_funcs import blast_kernels as KB
+    from triton_funcs import dense_kernels as KD
+    rng = np.random.default_rng(sum(ord(c) for c in ring_forced))
+    for n in range(10):
+        M, in_f, out_f = int(rng.integers(17, 640)), 8 * int(rng.integers(1, 140)), 8 * int(rng.integers(1, 80))
+        x = rng.standard_normal((M, in_f)); w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)
+        say(f"[case] ring random dense {n}: M={M} in={in_f} out={out_f} tile {ring_forced}")
+        out = KD.triton_dense_fp16(dev(x, torch.float16), dev(w, torch.float16), TILED)
+        assert_close(out, rounded(x, torch.float16) @ rounded(w, torch.float16), torch.float16, f"dense M={M} in={in_f} out={out_f}")
+    for n in range(8):
+        b = int(rng.integers(2, 4))
+        p, q, r, M = 8 * int(rng.integers(1, 30)), 8 * int(rng.integers(1, 40)), 8 * int(rng.integers(1, 150)), int(rng.integers(130, 520))
+        x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=1000 + n)
+        Uk, Vk, Sk = O.blast_to_bmm_layout(U, Vt, S)
+        say(f"[case] ring random bmm {n}: b={b} p={p} q={q} r={r} M={M} tile {ring_forced}")
+        dt = torch.bfloat16 if n % 2 else torch.float16
+        out = KB.triton_blast_bmm_fp16(dev(x, dt), dev(Uk, dt), dev(Vk, dt), dev(Sk, dt), TILED)
+        ref = O.blast_forward(rounded(x, dt), rounded(U, dt), rounded(Vt, dt), rounded(S, dt))[0]
+        assert_close(out, ref, dt, f"bmm b={b} p={p} q={q} r={r} M={M}")
+
+
 def test_int8_intermediates_through_ring_kernel(ring_forced):
     """The round-and-saturate epilogue of the ring kernel: integer inputs are exact."""
     from triton_funcs import blast_sym_quant_kernels as Q
