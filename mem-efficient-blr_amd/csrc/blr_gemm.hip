@@ -1311,12 +1311,15 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     }
     if (g.pair && rt <= 0) rt = 128128;
     if (rt > 0 && (ring > 1 || g.pair || (g.M >= 96 && g.K >= 64))) {
-      // Stages of 64 k (plain row-major output only): by default for single products with a reduction of a thousand or more - the
-      // batched products of BLAST have short reductions and live on two workgroups per compute unit overlapping each other's tile
-      // start-up and write-out, which the larger stages leave no LDS for (2048 rows: dense 4096 -> 22016 355 -> 335 us,
-      // 11008 -> 4096 207 -> 174 us; BLAST 4096 -> 22016 186 -> 201 us; DiT-XL/2 with dense layers 11.67 -> 11.04 ms, with BLAST
-      // layers 11.76 -> 12.25 ms).  BLR_GEMM_RING_BK = 32 / 64 decides for every problem.
-      if (option_value(OPT_GEMM_RING_BK, g.batch == 1 && g.K >= 1024 ? 64 : 32) == 64 && g.cn == 1) {
+      // Stages of 64 k (plain row-major output only): by default for reductions of a thousand or more - single products, and
+      // batched ones that give a compute unit at most two 256 x 128 tiles.  Batched products with many tiles per compute unit or
+      // short reductions (most of BLAST's) live on two workgroups per compute unit overlapping each other's tile start-up and
+      // write-out, which the larger stages leave no LDS for (2048 rows: dense 4096 -> 22016 355 -> 335 us, 11008 -> 4096
+      // 207 -> 174 us; BLAST 4096 -> 22016 186 -> 201 us with every product on 64-k stages, 186 -> 190 with only Z U (K = 1024,
+      // 1408 tiles), while 11008 -> 4096, whose Z U has 256 tiles, gains: 138 -> 132 us; Monarch 4096 -> 4096 / 11008 -> 4096
+      // 65.8 -> 60.3 / 96.4 -> 85.7 us; DiT-XL/2 with dense layers 11.67 -> 11.04 ms, with BLAST layers 11.76 -> 12.25 ms when
+      // forced).  BLR_GEMM_RING_BK = 32 / 64 decides for every problem.
+      if (option_value(OPT_GEMM_RING_BK, g.K >= 1024 && (g.batch == 1 || t128 <= 2 * (int64_t)cus) ? 64 : 32) == 64 && g.cn == 1) {
         const bool w8 = option_value(OPT_GEMM_RING_WAVES, 8) == 8;
         if (rt == 256256) return !w8 && !g.pair ? launch_ring64<T, 256, 256, 4, 2, 1>(g, st) : launch_ring64<T, 256, 256, 8, 2, 1>(g, st);
         if (rt == 256128) return w8 ? launch_ring64<T, 256, 128, 8, 3, 1>(g, st) : launch_ring64<T, 256, 128, 4, 3, 1>(g, st);
