@@ -1316,8 +1316,8 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       // short reductions (most of BLAST's) live on two workgroups per compute unit overlapping each other's tile start-up and
       // write-out, which the larger stages leave no LDS for (2048 rows: dense 4096 -> 22016 355 -> 335 us, 11008 -> 4096
       // 207 -> 174 us; BLAST 4096 -> 22016 186 -> 201 us with every product on 64-k stages, 186 -> 190 with only Z U (K = 1024,
-      // 1408 tiles), while 11008 -> 4096, whose Z U has 256 tiles, gains: 138 -> 132 us; Monarch 4096 -> 4096 / 11008 -> 4096
-      // 65.8 -> 60.3 / 96.4 -> 85.7 us; DiT-XL/2 with dense layers 11.67 -> 11.04 ms, with BLAST layers 11.76 -> 12.25 ms when
+      // 1408 tiles), while 11008 -> 4096, whose Z U has 256 tiles, gains: 139.3 -> 134.8 us; Monarch 4096 -> 4096 / 11008 -> 4096
+      // 64.9 -> 61.8 / 96.3 -> 88.8 us, side by side on one box; DiT-XL/2 with dense layers 11.67 -> 11.04 ms, with BLAST layers 11.76 -> 12.25 ms when
       // forced).  BLR_GEMM_RING_BK = 32 / 64 decides for every problem.
       if (option_value(OPT_GEMM_RING_BK, g.K >= 1024 && (g.batch == 1 || t128 <= 2 * (int64_t)cus) ? 64 : 32) == 64 && g.cn == 1) {
         const bool w8 = option_value(OPT_GEMM_RING_WAVES, 8) == 8;
