@@ -1,6 +1,6 @@
-"""Build libblr.so (the HIP kernels and their C ABI) for gfx950, in-tree.
+"""Build libblr.so (the HIP kernels and their C ABI) for gfx950, in-tree, and the stand-alone probes under probes/.
 
-    python build.py            # -> lib/libblr.so next to this file
+    python build.py            # -> lib/libblr.so next to this file, probes/<name> next to probes/<name>.hip
 
 Plain hipcc, no build system.  Objects are compiled in parallel, then linked.
 """
@@ -48,6 +48,13 @@ def build(verbose=True):
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", so])
     if verbose:
         print(f"built {so}")
+    # the stand-alone probes (not part of the library): built next to their sources so that they compile as long as the tree does
+    probes = [n[:-4] for n in sorted(os.listdir(os.path.join(HERE, "probes"))) if n.endswith(".hip")]
+    with ThreadPoolExecutor(max_workers=max(1, len(probes))) as ex:
+        list(ex.map(lambda n: _run([hipcc, *[f for f in FLAGS if f != "-fPIC"], os.path.join(HERE, "probes", n + ".hip"), "-o",
+                                    os.path.join(HERE, "probes", n)]), probes))
+    if verbose and probes:
+        print("built probes:", ", ".join(probes))
     return so
 
 
