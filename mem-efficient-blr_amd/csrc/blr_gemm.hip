@@ -960,32 +960,43 @@ __global__ __launch_bounds__(NWV * 64, (NWV / 4) * PER_CU) void gemm_ring64_kern
     const bool last_partial = ktail && t == KT - 1;
     const int nq = last_partial ? (ktail + 15) >> 4 : 4;             // sub-steps with anything to add
     const int nx = cs + 1 == NST ? 0 : cs + 1;
-    auto slot = [&](int sidx) {
-      if (sidx < SLOTS && (sidx * LT) / SLOTS != ((sidx + 1) * LT) / SLOTS) {
+    // With three stages the slot that the barrier of step t frees is needed only at the barrier of step t + 2, so its loads go out
+    // over four sub-steps (part 0 in sub-step 3 of step t, parts 1..3 in sub-steps 0..2 of step t + 1) instead of queueing in the
+    // compute unit's address path all at once; with two stages they must all go at once (part 0).
+    constexpr int PARTS = NST >= 3 ? 4 : 1;
+    const int tp = min(t - 1 + NST, KT - 1);                 // the stage whose later parts go out in this step, and its slot
+    const bool pp = ktail && tp == KT - 1;
+    const int sp = cs == 0 ? NST - 1 : cs - 1;
+    auto slot = [&](int sidx, int part) {
+      const int s2 = part * SLOTS + sidx;
+      if (part < PARTS && (s2 * LT) / (PARTS * SLOTS) != ((s2 + 1) * LT) / (PARTS * SLOTS)) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int li = (sidx * LT) / SLOTS; li < ((sidx + 1) * LT) / SLOTS; ++li) issue(li, tn, cs, pn);
+        for (int li = (s2 * LT) / (PARTS * SLOTS); li < ((s2 + 1) * LT) / (PARTS * SLOTS); ++li) {
+          if (part == 0) issue(li, tn, cs, pn);
+          else issue(li, tp, sp, pp);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     };
     // A sub-step: its products, between them - one per gap - the fragment reads of the next sub-step (a wave cannot issue a
     // product while it issues something else, and a burst of reads or loads leaves the matrix pipe idle when the SIMD's other wave
     // is in the same burst), and in the last sub-step the loads of stage t + NST.
-    auto substep = [&](int set, bool live, int stg_next, int q_next, bool loads) {
+    auto substep = [&](int set, bool live, int stg_next, int q_next, int part) {      // part: which part of a stage's loads goes with it
 #pragma unroll
       for (int m = 0; m < NMF; ++m) {
         if (live) mfma_one(set, m);
         if (m < TM + TN) frag_one(stg_next, q_next, set ^ 1, m);
-        if (loads) slot(m);
+        slot(m, part);
         __builtin_amdgcn_sched_barrier(0);
       }
     };
     if (last_partial) zero_tail(0, 0);
-    substep(0, true, cs, 1, false);
+    substep(0, true, cs, 1, 1);       // (in step 0 parts 1..3 repeat loads of the last stage the prologue asked for, into the same slot)
     if (last_partial) zero_tail(1, 1);
-    substep(1, nq > 1, cs, 2, false);
+    substep(1, nq > 1, cs, 2, 2);
     if (last_partial) zero_tail(0, 2);
-    substep(0, nq > 2, cs, 3, false);
+    substep(0, nq > 2, cs, 3, 3);
     // the step's barrier: stage t is in registers, stage t + 1 has landed
 #ifdef BLR_TRACE
     const uint64_t tw0 = __builtin_amdgcn_s_memtime();
@@ -1002,7 +1013,7 @@ __global__ __launch_bounds__(NWV * 64, (NWV / 4) * PER_CU) void gemm_ring64_kern
 #endif
     __builtin_amdgcn_sched_barrier(0);
     if (last_partial) zero_tail(1, 3);
-    substep(1, nq > 3, nx, 0, true);
+    substep(1, nq > 3, nx, 0, 0);
     cs = nx;
   }
   __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
