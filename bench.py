@@ -167,8 +167,14 @@ def main():
                 go(st)
         return g
 
-    def time_graph(g, n_launches, reps=5):
+    def time_graph(g, n_launches, reps=5, warm_ms=60.0):
+        # replays for at least warm_ms before the timed ones: from idle the card needs some tens of milliseconds of work to settle
+        # on its clocks, and a matrix-bound call timed right after a pause read up to 10 % slower than in steady state (the dense
+        # 4096 -> 4096 GEMM at 2048 rows: 75.6 us as the first thing measured, 67.5 after 60 ms of replays); decode rows do not move
         g.replay(); torch.cuda.synchronize()
+        t_w = time.perf_counter()
+        while (time.perf_counter() - t_w) * 1e3 < warm_ms:
+            g.replay(); torch.cuda.synchronize()
         best = []
         for _ in range(reps):
             e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
