@@ -756,8 +756,8 @@ __global__ __launch_bounds__(NWV * 64, (SHALLOW ? 2 : 1)) void gemm_ring_kernel(
 // as above.  NST stages (two or three) of both operands form one ring with one barrier per step of 64 k; a step is four sub-steps
 // of 16 k (one fragment of each 32-row block).
 // What the loop is made of, per step of a 256 x 256 tile on eight waves (two per SIMD): 64 matrix instructions per SIMD (2048
-// cycles of its matrix pipe), 192 KiB of fragment reads and 64 KiB of operand loads into LDS - the LDS is as busy as the matrix
-// pipe.  In-kernel cycle counts: 2890 cycles per step with the fragment reads of a sub-step issued as one burst ahead of its
+// cycles of its matrix pipe), 192 KiB of fragment reads (about 770 cycles of the LDS), 64 KiB of operand loads into LDS in 64 load
+// instructions that queue in the compute unit's one address path.  In-kernel cycle counts: 2890 cycles per step with the fragment reads of a sub-step issued as one burst ahead of its
 // products and the barrier at the end of the step, 2570 with one read or load between two products and the barrier between the
 // third and the fourth sub-step (behind it a wave still holds a sub-step of products in registers, under which the first fragments
 // of the next stage arrive).  The clock drops as the pipe fills up (1.35 -> 1.27 GHz under the board's power limit with random
