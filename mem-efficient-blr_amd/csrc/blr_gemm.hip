@@ -768,7 +768,7 @@ constexpr size_t ring64_lds_bytes() {
   return st > ep ? st : ep;
 }
 
-template <typename T, bool B_KN, int BM, int BN, bool EP, int NWV, int NST, int PER_CU>
+template <typename T, bool B_KN, int BM, int BN, bool EP, int NWV, int NST, int PER_CU, bool HALF = false>
 __global__ __launch_bounds__(NWV * 64, (NWV / 4) * PER_CU) void gemm_ring64_kernel(GemmArgs g, int tiles_m, int tiles_n, int per_xcd, int group_m, int side_wgs) {
   constexpr int ASTG = BM * 128, BSTG = BN * 128, BRING = NST * ASTG;
   constexpr int WGN = (NWV == 8 && BN == 256) ? 4 : 2, WGM = NWV / WGN;
@@ -841,13 +841,25 @@ __global__ __launch_bounds__(NWV * 64, (NWV / 4) * PER_CU) void gemm_ring64_kern
     tail_kn[i] = B_KN ? (uint32_t)((krow - min(krow, rmax)) * g.ldb * 2) : tail_kc;
   }
   const uint32_t lds0 = ring_lds_addr(smem + wave * 1024);
+  // HALF (eight waves, two stages, every tile inside the matrices, no partial stage: the launcher checks): a stage's loads cannot
+  // be spread over the step here, and every wave that issues one waits in the compute unit's address path while its SIMD's other
+  // wave may be waiting there too.  Waves 0..3 - one per SIMD - therefore issue the loads of waves 4..7 as well: those rows lie
+  // NWV / 2 load instructions further down, a wave-uniform offset, so the same per-lane offsets serve (nothing is clamped).
+  static_assert(!HALF || (NWV == 8 && NST == 2), "the one configuration this is for");
+  constexpr int ISS = HALF ? 2 : 1;
+  const bool issuer = !HALF || wave < NWV / 2;
+  const int64_t dA = (int64_t)(NWV / 2) * 8 * g.lda * 2;
+  const int64_t dB = B_KN ? (int64_t)(NWV / 2) * RPI * g.ldb * 2 : (int64_t)(NWV / 2) * 8 * g.ldb * 2;
   auto issue = [&](int li, int tile, int stg, bool partial) {       // load li (A first, then B) of stage `tile` into ring slot stg
+    if (HALF && !issuer) return;                                     // (wave-uniform)
     if (li < LA) {
       ring_load_lds(Ab + (int64_t)tile * 128, a_off[li] - (partial ? tail_kc : 0u), lds0 + stg * ASTG + li * (NWV * 1024));
+      if (HALF) ring_load_lds(Ab + (int64_t)tile * 128 + dA, a_off[li] - (partial ? tail_kc : 0u), lds0 + stg * ASTG + li * (NWV * 1024) + (NWV / 2) * 1024);
     } else {
       const int lb = li - LA;
       const char* Bp = B_KN ? Bb + (int64_t)tile * 64 * g.ldb * 2 : Bb + (int64_t)tile * 128;
       ring_load_lds(Bp, b_off[lb] - (partial ? tail_kn[lb] : 0u), lds0 + BRING + stg * BSTG + lb * (NWV * 1024));
+      if (HALF) ring_load_lds(Bp + dB, b_off[lb] - (partial ? tail_kn[lb] : 0u), lds0 + BRING + stg * BSTG + lb * (NWV * 1024) + (NWV / 2) * 1024);
     }
   };
 
@@ -945,7 +957,7 @@ __global__ __launch_bounds__(NWV * 64, (NWV / 4) * PER_CU) void gemm_ring64_kern
 #pragma unroll
     for (int li = 0; li < LT; ++li) issue(li, tc, s, partial);
   }
-  __builtin_amdgcn_s_waitcnt(ring_vmcnt((NST - 1) * LT));
+  __builtin_amdgcn_s_waitcnt(ring_vmcnt((NST - 1) * LT * ISS));
   __builtin_amdgcn_s_barrier();
   TRG(1);
   frags(0, 0, 0);
@@ -1002,7 +1014,7 @@ __global__ __launch_bounds__(NWV * 64, (NWV / 4) * PER_CU) void gemm_ring64_kern
     const uint64_t tw0 = __builtin_amdgcn_s_memtime();
 #endif
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(ring_vmcnt((NST - 2) * LT));   // (later stages may still be out)
+    __builtin_amdgcn_s_waitcnt(ring_vmcnt((NST - 2) * LT * ISS));   // (later stages may still be out)
 #ifdef BLR_TRACE
     const uint64_t tw1 = __builtin_amdgcn_s_memtime();
 #endif
@@ -1232,6 +1244,12 @@ static int launch_ring64(const GemmArgs& g, hipStream_t st) {
   const bool ep = g.bias != nullptr || g.act != 0 || g.gate != nullptr || g.resid != nullptr;
   void* fn = ep ? (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, true, NWV, NST, PER_CU> : (void*)gemm_ring64_kernel<T, false, BM, BN, true, NWV, NST, PER_CU>)
                 : (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, false, NWV, NST, PER_CU> : (void*)gemm_ring64_kernel<T, false, BM, BN, false, NWV, NST, PER_CU>);
+  if constexpr (NWV == 8 && NST == 2) {
+    // no tile with a clamped row or column and no partial stage: four of the eight waves issue all loads (see the kernel)
+    if (g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0)
+      fn = ep ? (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, true, NWV, NST, PER_CU, true> : (void*)gemm_ring64_kernel<T, false, BM, BN, true, NWV, NST, PER_CU, true>)
+              : (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, false, NWV, NST, PER_CU, true> : (void*)gemm_ring64_kernel<T, false, BM, BN, false, NWV, NST, PER_CU, true>);
+  }
   static std::mutex mu;
   static std::set<void*> raised;
   {

@@ -101,6 +101,37 @@ def test_seeded_random_shapes_through_every_variant(ring_forced):
         assert_close(out, ref, dt, f"bmm b={b} p={p} q={q} r={r} M={M}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_whole_tiles_of_the_two_stage_kernel(dtype):
+    """Problems made of whole 256 x 256 tiles and whole 64-k stages take a variant of the eight-wave, two-stage kernel in which
+    four waves issue every load (the others' rows at a wave-uniform offset): plain, with bias + SiLU-gated pairs of tiles, and
+    with a K-contiguous second operand (U of the bmm layout), each against the oracle; one more k stage, one more row and one
+    more column group leave that variant again and must give the same kind of answer."""
+    from triton_funcs import _lib as L, blast_kernels as KB, dense_kernels as KD
+    rng = np.random.default_rng(11)
+    with L.options(BLR_GEMM_RING=2, BLR_GEMM_RING_TILE="256256", BLR_GEMM_RING_PER_CU="1", BLR_GEMM_RING_WAVES="8", BLR_GEMM_RING_BK="64"):
+        for M, in_f, out_f in [(512, 1088, 768), (256, 64, 256), (512, 1096, 768), (513, 1088, 768), (512, 1088, 776)]:
+            x = rng.standard_normal((M, in_f)); w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)
+            say(f"[case] whole tiles dense M={M} in={in_f} out={out_f} {dtype}")
+            out = KD.triton_dense_fp16(dev(x, dtype), dev(w, dtype), TILED)
+            assert_close(out, rounded(x, dtype) @ rounded(w, dtype), dtype, f"dense M={M} in={in_f} out={out_f}")
+        M, in_f, out_f = 512, 320, 1024                              # gate | up of 512 columns each: two column tiles per half
+        x = rng.standard_normal((M, in_f)); w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f); bias = rng.standard_normal(out_f)
+        say(f"[case] whole tiles dense silu_mul {dtype}")
+        with L.fused_epilogue(dev(bias, dtype), "silu_mul"):
+            out = KD.triton_dense_fp16(dev(x, dtype), dev(w, dtype), TILED)
+        v = rounded(x, dtype) @ rounded(w, dtype) + rounded(bias, dtype)
+        g, u = v[:, :out_f // 2], v[:, out_f // 2:]
+        assert_close(out, g / (1.0 + np.exp(-g)) * u, dtype, "dense silu_mul", scale=2.0)
+        b, p, q, r = 2, 64, 256, 128
+        xb, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=5)
+        Uk, Vk, Sk = O.blast_to_bmm_layout(U, Vt, S)
+        say(f"[case] whole tiles blast bmm {dtype}")
+        out = KB.triton_blast_bmm_fp16(dev(xb, dtype), dev(Uk, dtype), dev(Vk, dtype), dev(Sk, dtype), TILED)
+        ref = O.blast_forward(rounded(xb, dtype), rounded(U, dtype), rounded(Vt, dtype), rounded(S, dtype))[0]
+        assert_close(out, ref, dtype, "blast bmm")
+
+
 def test_int8_intermediates_through_ring_kernel(ring_forced):
     """The round-and-saturate epilogue of the ring kernel: integer inputs are exact."""
     from triton_funcs import blast_sym_quant_kernels as Q
