@@ -1318,6 +1318,7 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     const int64_t fill = ((int64_t)cus * 9 + 9) / 10;
     const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
     int per_cu = option_value(OPT_GEMM_RING_PER_CU, 0);
+    bool wide64 = false;                       // a 256 x 256 tile chosen together with stages of 64 k
     // interleaved columns are bound by their two-byte stores: only worth it with several tiles per compute unit
     if (rt == 0 && g.cn != 1 && ring < 2 && t128 < 2 * (int64_t)cus) rt = -1;
     if (rt == 0) {
@@ -1329,6 +1330,10 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       // traffic per matrix instruction beats the overlap of two smaller workgroups (2048 x 22016 x 1024: 164.7 -> 154.1 us for
       // the whole low-rank call; four batches of 2048 x 5504 x 1024: Monarch 184.6 -> 176.8 us)
       else if (g.K >= 1024 && g.K <= 2048 && g.N >= 2048 && t256 >= 2 * (int64_t)cus) rt = 256256;
+      // the same for batched products from a reduction of eight stages of 64 k, where 256-column tiles waste at most an eighth of
+      // their columns: per-kernel times at 2048 rows, 16 batches: 1376 columns, K = 1024 (Z U of BLAST 4096 -> 22016) 118.0 -> 112.4 us,
+      // 1024 columns, K = 688 (x V of 11008 -> 4096) 75.1 -> 66.8 us
+      else if (g.cn == 1 && g.K >= 512 && g.K <= 2048 && g.N >= 1024 && cdiv(g.N, 256) * 256 * 8 <= (int64_t)g.N * 9 && t256 >= 2 * (int64_t)cus) { rt = 256256; wide64 = true; }
       else if (g.K <= 2048 && t128 >= 2 * (int64_t)cus) { rt = 256128; if (!per_cu) per_cu = 2; }
       else if (g.K <= 512 && r128 >= fill) rt = 128128;
       // a narrow output (one 128-column tile, mostly empty at 256): more, smaller tiles (4096 x 72 x 576 in 16 batches:
@@ -1341,14 +1346,15 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     if (g.pair && rt <= 0) rt = 128128;
     if (rt > 0 && (ring > 1 || g.pair || (g.M >= 96 && g.K >= 64))) {
       // Stages of 64 k (plain row-major output only): by default for reductions of a thousand or more - single products, and
-      // batched ones that give a compute unit at most two 256 x 128 tiles.  Batched products with many tiles per compute unit or
-      // short reductions (most of BLAST's) live on two workgroups per compute unit overlapping each other's tile start-up and
-      // write-out, which the larger stages leave no LDS for (2048 rows: dense 4096 -> 22016 355 -> 335 us, 11008 -> 4096
-      // 207 -> 174 us; BLAST 4096 -> 22016 186 -> 201 us with every product on 64-k stages, 186 -> 190 with only Z U (K = 1024,
-      // 1408 tiles), while 11008 -> 4096, whose Z U has 256 tiles, gains: 139.3 -> 134.8 us; Monarch 4096 -> 4096 / 11008 -> 4096
+      // batched ones that give a compute unit at most two 256 x 128 tiles - and for the wide batched products that the rule above
+      // gave 256 x 256 tiles.  Other batched products with many tiles per compute unit or short reductions (most of BLAST's) live
+      // on two workgroups of 256 x 128 per compute unit overlapping each other's tile start-up and write-out, which the larger
+      // stages leave no LDS for (2048 rows: dense 4096 -> 22016 355 -> 335 us, 11008 -> 4096 207 -> 174 us; BLAST 4096 -> 22016
+      // 186 -> 201 us with every product on 64-k stages of 256 x 128 tiles, 186 -> 190 with only Z U (K = 1024, 1408 tiles), while
+      // 11008 -> 4096, whose Z U has 256 tiles, gains: 139.3 -> 134.8 us; Monarch 4096 -> 4096 / 11008 -> 4096
       // 64.9 -> 61.8 / 96.3 -> 88.8 us, side by side on one box; DiT-XL/2 with dense layers 11.67 -> 11.04 ms, with BLAST layers 11.76 -> 12.25 ms when
       // forced).  BLR_GEMM_RING_BK = 32 / 64 decides for every problem.
-      if (option_value(OPT_GEMM_RING_BK, g.K >= 1024 && (g.batch == 1 || t128 <= 2 * (int64_t)cus) ? 64 : 32) == 64 && g.cn == 1) {
+      if (option_value(OPT_GEMM_RING_BK, wide64 || (g.K >= 1024 && (g.batch == 1 || t128 <= 2 * (int64_t)cus)) ? 64 : 32) == 64 && g.cn == 1) {
         const bool w8 = option_value(OPT_GEMM_RING_WAVES, 8) == 8;
         if (rt == 256256) return !w8 && !g.pair ? launch_ring64<T, 256, 256, 4, 2, 1>(g, st) : launch_ring64<T, 256, 256, 8, 2, 1>(g, st);
         if (rt == 256128) return w8 ? launch_ring64<T, 256, 128, 8, 3, 1>(g, st) : launch_ring64<T, 256, 128, 4, 3, 1>(g, st);
