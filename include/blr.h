@@ -103,7 +103,7 @@ void blr_set_spin_limit(unsigned polls);
 /* The run-time switches of the library (no counterpart in the reference), all of them: the GEMM variant - BLR_GEMM_RING
  * (0..2), BLR_GEMM_RING_TILE (0, 256256, 256128, 256096, 128128), BLR_GEMM_RING_PER_CU (0..2), BLR_GEMM_RING_WAVES (4, 8),
  * BLR_GEMM_RING_BK (32, 64: k per operand stage), BLR_GEMM_SPLITK (0, 1) - and kernel families on / off - BLR_DECODE2, BLR_DECODE3, BLR_DECODE_ROWS, BLR_DENSE_SLAB,
- * BLR_DENSE_ROWS, BLR_BLAST_ONE (0, 1), BLR_DECODE_PAIR, BLR_BLAST_MIXU (0..2); a family that is off hands its calls to the
+ * BLR_DENSE_ROWS, BLR_BLAST_ONE, BLR_BLAST_YMIXW (0, 1), BLR_DECODE_PAIR, BLR_BLAST_MIXU (0..2); a family that is off hands its calls to the
  * next one that serves them.  Each starts from the environment variable of its name (read once; a value out of range is
  * ignored); unset != 0 returns it to "not set".  Returns BLR_ERR_BAD_ARG for an unknown name or a value out of range.  */
 int blr_set_option(const char* name, int value, int unset);

@@ -296,7 +296,7 @@ namespace {
 constexpr int kOptUnset = -2147483647 - 1;
 const char* const kOptNames[OPT_COUNT] = {"BLR_GEMM_RING", "BLR_GEMM_RING_TILE", "BLR_GEMM_RING_PER_CU", "BLR_GEMM_RING_WAVES", "BLR_GEMM_RING_BK", "BLR_GEMM_SPLITK",
                                           "BLR_DECODE2", "BLR_DECODE3", "BLR_DECODE_PAIR", "BLR_DECODE_ROWS", "BLR_DENSE_SLAB", "BLR_DENSE_ROWS",
-                                          "BLR_BLAST_MIXU", "BLR_BLAST_ONE"};
+                                          "BLR_BLAST_MIXU", "BLR_BLAST_ONE", "BLR_BLAST_YMIXW"};
 // what each option may be set to: a range, or (BLR_GEMM_RING_TILE, BLR_GEMM_RING_WAVES) a short list; anything else is refused
 bool opt_value_ok(int id, int v) {
   switch (id) {
@@ -452,7 +452,17 @@ static int blast_tiled(const void* x, int64_t ldx, const void* U, const void* V,
     rc = 1;
   }
   const bool mixu = mixu_shape && (mixu_mode >= 2 || (mixu_mode == 1 && (P > fuse_max_p || fused < 0)));
-  if (!mixu && !y_out && !sat8 && fused >= 0 && (fused == 1 || P <= fuse_max_p))
+  // Wide input blocks (16 of them, a multiple of 64 columns each, rank a multiple of 64): x V as one GEMM whose 64 x 64 tile keeps Y
+  // of all 16 blocks in registers, then the mix, in one launch (blast_ymixw_kernel) - by itself from half a round of tiles on
+  // (whole calls, before -> after: 4096 -> 4096, r = 512 at 1024 / 2048 / 4096 rows 47.1 -> 46.1 / 65.7 -> 56.3 / 101.9 -> 96.2 us,
+  // at 512 rows 40.1 -> 44.3; 4096 -> 22016, r = 1024 at 512 / 1024 / 2048 / 4096 rows 78.6 -> 77.7 / 114.4 -> 104.3 / 179.5 -> 174.0 /
+  // 350.6 -> 344.2 us, at 256 rows 55.2 -> 59.3).  BLR_BLAST_YMIXW=0 switches it off; BLR_ALGO_FUSED asks for it at any row count.
+  const int cus_now = device_cus() > 0 ? device_cus() : 256;
+  const bool ymixw_fill = cdiv(M, 64) * (int64_t)(r / 64) * 2 >= cus_now;
+  if (!mixu && !y_out && !sat8 && fused >= 0 && P > fuse_max_p && option_value(OPT_BLAST_YMIXW, 1) && (fused == 1 || ymixw_fill))
+    rc = blast_ymixw_launch(x, ldx, V, S, Z, M, in_f, b, r, si, sj, sr, s_layout, dtype, Y, ybytes, st);
+  if (rc < 0) return rc;
+  if (rc == 1 && !mixu && !y_out && !sat8 && fused >= 0 && (fused == 1 || P <= fuse_max_p))
     rc = blast_ymix_launch(x, ldx, V, S, Z, M, in_f, b, r, si, sj, sr, s_layout, dtype, Y, ybytes, st);   // (the unused room of Y holds S transposed)
   if (rc < 0) return rc;
   if (rc == 1 && fused == 1) { set_error("blast: the fused kernel does not take this shape (b even and <= 16, block width and rank multiples of 8, f16/bf16)"); return BLR_ERR_UNSUPPORTED; }

@@ -88,7 +88,7 @@ void epilogue_taken();
 // is range-checked where it is set.  The first six pick the GEMM variant, the rest switch a kernel family off (0) so that the
 // call falls through to the next one that serves it - for A/B measurements and as a way out should a kernel misbehave.
 enum { OPT_GEMM_RING = 0, OPT_GEMM_RING_TILE, OPT_GEMM_RING_PER_CU, OPT_GEMM_RING_WAVES, OPT_GEMM_RING_BK, OPT_GEMM_SPLITK,
-       OPT_DECODE2, OPT_DECODE3, OPT_DECODE_PAIR, OPT_DECODE_ROWS, OPT_DENSE_SLAB, OPT_DENSE_ROWS, OPT_BLAST_MIXU, OPT_BLAST_ONE, OPT_COUNT };
+       OPT_DECODE2, OPT_DECODE3, OPT_DECODE_PAIR, OPT_DECODE_ROWS, OPT_DENSE_SLAB, OPT_DENSE_ROWS, OPT_BLAST_MIXU, OPT_BLAST_ONE, OPT_BLAST_YMIXW, OPT_COUNT };
 int option_value(int id, int dflt);             // the option's value, or dflt when it is unset
 // true when p is aligned to `bytes`.
 static inline bool aligned(const void* p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) % bytes) == 0; }
@@ -182,6 +182,9 @@ int blast_mix_launch(const void* Y, const void* S, void* Z, int M, int b, int R,
 // Z (b, M, R) of dtype.  Returns BLR_OK, a negative blr_status, or 1 when the shape is not for the kernel.
 // scratch: b * b * R elements for S in (r, i, j) order (not touched when S already has that layout).
 int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, void* Z, int M, int in_f, int b, int R,
+                      int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
+                      hipStream_t st);
+int blast_ymixw_launch(const void* x, int64_t ldx, const void* V, const void* S, void* Z, int M, int in_f, int b, int R,
                       int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
                       hipStream_t st);
 // Second half for output blocks of at most 80 columns: out_i = mix(S, Y)_i U_i with U (b, Q, R) (u_rq: (b, R, Q)), in one launch and without Z;

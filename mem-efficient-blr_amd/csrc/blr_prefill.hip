@@ -22,6 +22,7 @@
 #include <type_traits>
 #include "blr_common.h"
 #include "blr_decode_dev.h"
+#include "blr_ring_dev.h"
 
 namespace blr {
 
@@ -340,6 +341,256 @@ int blast_ymix_launch(const void* x, int64_t ldx, const void* V, const void* S, 
   void* args[] = {&p};
   hipError_t e = hipLaunchKernel(fns[fi], dim3((unsigned)(nrt * nmt)), dim3(YM_NT), args, lds, st);
   if (e != hipSuccess) { set_error("blast_ymix: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+  return BLR_OK;
+}
+
+
+// ---- the same first half for wide input blocks: x V as one GEMM over all of x's columns, Y held in registers -------------------
+//
+// blast_ymix_kernel reads V once per 32 rows, straight into registers; from about 128 columns per input block on that costs more
+// than the round trip of Y through memory that it saves.  Here a workgroup of four waves (one per SIMD, so a lane may hold some
+// 250 registers) owns 64 rows x 64 ranks for all 16 input blocks.  x is (M, 16 P) and V (16 P, R), both contiguous over the
+// blocks, so Y_0 .. Y_15 of the tile are one GEMM with a reduction over all 16 P columns whose accumulator is packed away and
+// cleared every P columns: stages of 64 k of both operands go global -> LDS directly (whole 128-byte lines; the stage layouts
+// and fragment reads of gemm_ring64_kernel), YW_NST stages deep, one barrier per stage; a wave's 32 x 32 block of Y_j leaves the
+// accumulator as 8 dwords (two ranks each), 128 dwords for the sixteen blocks.  When the reduction is done the ring is no longer
+// needed: Y goes to LDS as dwords (Y_2jp, Y_2jp+1) [jp][row][rank ^ f(row, jp)], and the mix runs as in blast_ymix_kernel (one
+// 16 x 16 x 16 matrix instruction per rank and 16 rows), its rows of Z staged through LDS and stored as whole 128-byte lines.
+namespace {
+constexpr int YW_NT = 256, YW_NST = 8, YW_STG = 8192;      // threads; ring depth; bytes of a stage of one operand (64 x 64 elements)
+constexpr size_t YW_LDS = 160 * 1024;                      // ring: 2 x 8 x 8 KiB + the tile's slice of S 32 KiB; afterwards Y 128 KiB + staged rows of Z 32 KiB
+}
+
+struct YmixwParams {
+  const void* x; int64_t ldx;
+  const void* V; const void* St; void* Z;
+  int M, R, KT;                 // KT: stages of 64 k per input block (P / 64)
+  FastDiv nrt;                  // rank tiles
+  int s_stage;                  // 0: St is S as (r, i, j), read straight into the mix's operands; 1: S has the rank contiguous
+  int64_t s_si, s_sj;           //    (strides of i and j in elements): the tile's slice goes through LDS
+};
+
+template <typename T>
+__global__ __launch_bounds__(YW_NT, 1) void blast_ymixw_kernel(YmixwParams p) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char yw_lds[];
+  constexpr int NWV = 4, NST = YW_NST, BRING = NST * YW_STG, LT = 4, RB = 128;
+  using V8 = typename TypeTraits<T>::vec8;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int M = p.M, R = p.R;
+  // a run of items per XCD, rank tiles fastest: the workgroups of an XCD at any time share two tiles of rows of x in its L2
+  const uint32_t item = xcd_item(blockIdx.x, gridDim.x);
+  const uint32_t mt = fd_div(item, p.nrt), rt = item - mt * p.nrt.d;
+  const int m0 = (int)mt * 64, r0 = (int)rt * 64;
+  TR6(0);
+  const int n = lane & 15, g = lane >> 4, rw = wave * 16;
+  // ---------------------------------------------- phase 1: Y of the tile, in registers --------------------------------------
+  // stage s covers columns 64 s .. 64 s + 63 of x and rows 64 s .. of V (all blocks).  K-contiguous stage (x): a load takes eight
+  // 16-byte chunks of each of 8 rows, lane (r8, s8) chunk s8 ^ r8; (k, n) stage (V): a load takes 8 rows of 64 ranks, chunk c of
+  // row k stored at c ^ ((k & 3) << 1).
+  const int r8 = lane >> 3, s8 = lane & 7, c8 = s8 ^ r8;
+  uint32_t a_off[2], b_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    a_off[i] = (uint32_t)(min(m0 + (i * NWV + wave) * 8 + r8, M - 1) * p.ldx * 2 + c8 * 16);
+    const int krow = (i * NWV + wave) * 8 + r8;
+    b_off[i] = (uint32_t)((krow * R + r0 + (s8 ^ ((krow & 3) << 1)) * 8) * 2);
+  }
+  const uint32_t lds0 = ring_lds_addr(yw_lds + wave * 1024);
+  const char* Ab = reinterpret_cast<const char*>(p.x);
+  const char* Bb = reinterpret_cast<const char*>(p.V);
+  auto issue = [&](int s, int slot) {
+    const char* ap = Ab + (int64_t)s * 128;
+    const char* bp = Bb + (int64_t)s * 64 * R * 2;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) ring_load_lds(ap, a_off[i], lds0 + slot * YW_STG + i * (NWV * 1024));
+#pragma unroll
+    for (int i = 0; i < 2; ++i) ring_load_lds(bp, b_off[i], lds0 + BRING + slot * YW_STG + i * (NWV * 1024));
+  };
+  const int half = lane >> 5;
+  const int rl = wm * 32 + (lane & 31);
+  const uint32_t rowA = (uint32_t)(((rl >> 3) << 10) + ((rl & 7) << 7));
+  uint32_t xo[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) xo[q] = (uint32_t)(((2 * q + half) ^ (lane & 7)) << 4);
+  const int i16 = lane & 15;
+  const int chunk0 = wn * 4 + (g & 1) * 2 + ((i16 & 3) >> 1);
+  const uint32_t rowB = (uint32_t)(((g >> 1) * 8 + (i16 >> 2)) * RB + (i16 & 1) * 8 + ((chunk0 ^ ((i16 >> 2) << 1)) << 4));
+
+  // Stage t lives in slot t % NST; NST - 1 stages are in flight.  The loop is bound by how many bytes a compute unit has in flight
+  // over the latency of its loads, so the ring takes all of the LDS.  (Asking for every line a first time twenty stages early, by
+  // a 4-byte load per line into a dump area, made it slower: 18.5 -> 28.9 us per tile at P = 256, R = 512 - an instruction that
+  // touches 32 lines costs the address path as much as four that fetch them.)
+  const int s_total = 16 * p.KT;
+#pragma unroll
+  for (int s = 0; s < NST - 1; ++s) issue(min(s, s_total - 1), s);
+  TR6(1);
+  // S with the rank contiguous ((j, i, r) or (i, j, r)): the 256 rows (j, i) x 64 ranks of this tile go to LDS behind the ring,
+  // where nothing else lives until the mix stages its rows of Z - by then the operands are in registers
+  T* const s_t = reinterpret_cast<T*>(yw_lds + 2 * YW_NST * YW_STG);
+  if (p.s_stage) {
+    const T* Sg = reinterpret_cast<const T*>(p.St);
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int idx = it * YW_NT + tid, ji = idx >> 3, c = (idx & 7) * 8;
+      *reinterpret_cast<V8*>(&s_t[ji * 64 + c]) = *reinterpret_cast<const V8*>(&Sg[(int64_t)(ji & 15) * p.s_si + (int64_t)(ji >> 4) * p.s_sj + r0 + c]);
+    }
+  }
+
+  f32x16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+  uint32_t yreg[16][8];
+  int s = 0, slot = 0;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    for (int kt = 0; kt < p.KT; ++kt, ++s) {
+      __builtin_amdgcn_s_waitcnt(ring_vmcnt((NST - 2) * LT));   // this wave's part of stage s has landed
+      __builtin_amdgcn_s_barrier();                             // everybody's has, and nobody reads stage s - 1 any more
+      issue(min(s + NST - 1, s_total - 1), slot == 0 ? NST - 1 : slot - 1);   // (past the end: the last stage again, never read)
+      const unsigned char* sta = yw_lds + slot * YW_STG;
+      const unsigned char* stb = yw_lds + BRING + slot * YW_STG;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const V8 af = *reinterpret_cast<const V8*>(sta + rowA + xo[q]);
+        union { V8 v; s16x4 h[2]; } w;
+        w.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(stb + rowB + (q * 16) * RB));
+        w.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(stb + rowB + (q * 16 + 4) * RB));
+        acc = TypeTraits<T>::mfma32(w.v, af, acc);             // (ranks as rows: the product comes out transposed)
+      }
+      slot = slot + 1 == NST ? 0 : slot + 1;
+    }
+    // acc[4 q + e] is Y_j at row wm 32 + (lane & 31), rank wn 32 + 8 q + 4 half + e
+#pragma unroll
+    for (int d = 0; d < 8; ++d) yreg[j][d] = ym_pack<T>(acc[2 * d], acc[2 * d + 1]);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+  }
+  TR6(2);
+  __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));                    // the repeats of the last stage have landed too: the ring is free
+  __builtin_amdgcn_s_barrier();
+  // the mix's S operands, asked for now (the loop had no registers to spare) and used after Y has gone to LDS.  Lane (n, g) of
+  // wave w: S_r(i = n, j = 4 g .. 4 g + 3), r = r0 + 16 w ..
+  u32x2 sa[16];
+  if (p.s_stage) {                                              // (the barrier above is behind every wave's stores of the slice)
+    const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s_t);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      uint32_t v[4];
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) v[jj] = s16[((4 * g + jj) * 16 + n) * 64 + rw + q];
+      sa[q] = u32x2{v[0] | (v[1] << 16), v[2] | (v[3] << 16)};
+    }
+  } else {
+    const __amdgpu_buffer_rsrc_t sbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.St), 0, (uint32_t)((int64_t)256 * R * 2), 0x00020000);
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+      sa[q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(sbuf, (uint32_t)(((r0 + rw + q) * 16 + n) * 16 + 4 * g) * 2u, 0, 0));
+  }
+
+  // Y -> LDS: dword (Y_2jp, Y_2jp+1) of (row m, rank r) at [jp][m][r ^ ((m & 15) + 16 (jp >> 1))] - the 64 lanes of a mix read
+  // (16 rows x 4 pairs of planes, one rank) then hit 64 different banks.  Dword d of a block holds ranks ra, ra + 1 (ra even):
+  // neighbours in LDS, in the order the row's parity gives.
+  uint32_t* const y_s = reinterpret_cast<uint32_t*>(yw_lds);
+  {
+    const int m = wm * 32 + (lane & 31);
+#pragma unroll
+    for (int jp = 0; jp < 8; ++jp)
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        const uint32_t h0 = yreg[2 * jp][d], h1 = yreg[2 * jp + 1][d];
+        const uint32_t da = __builtin_amdgcn_perm(h1, h0, 0x05040100u), db = __builtin_amdgcn_perm(h1, h0, 0x07060302u);
+        const int ra = wn * 32 + 8 * (d >> 1) + 4 * half + 2 * (d & 1);
+        const int col = (ra ^ ((m & 15) + 16 * (jp >> 1))) & ~1;
+        *reinterpret_cast<u32x2*>(&y_s[jp * 4096 + m * 64 + col]) = (m & 1) ? u32x2{db, da} : u32x2{da, db};
+        if (d == 7) __builtin_amdgcn_sched_barrier(0);          // (one pair of blocks at a time: nothing to gain from more in flight)
+      }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  TR6(3); TR6(4);
+
+  // ---------------------------------------------- phase 2: the mix --------------------------------------------------------
+  // lane (n, g): operand A = S_r(i = n, j = 4 g .. 4 g + 3), operand B = Y_r(j = 4 g .. 4 g + 3, m = 16 mg + n); the product's lane
+  // holds Z_r(i = 4 g + t, m = 16 mg + n).  The 256 rows (i, m) of a group of 16 rows of the tile go through LDS (128 bytes each,
+  // 16-byte slots XOR-ed with the row's low bits) and leave as whole lines.
+  uint32_t* const z_st = y_s + 8 * 4096;
+#pragma unroll 1
+  for (int mg = 0; mg < 4; ++mg) {
+    if (mg) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // the previous group's rows have been read
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      f32x4 d[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const int rr = rw + 8 * h + q;
+        const uint32_t* src = &y_s[(2 * g) * 4096 + (16 * mg + n) * 64 + (rr ^ (n + 16 * g))];
+        const u32x2 yb = {src[0], src[4096]};
+        d[q] = YmDot<T>::mfma16(sa[8 * h + q], yb, f32x4{0.f, 0.f, 0.f, 0.f});
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        u32x4 o;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) o[q] = ym_pack<T>(d[2 * q][t], d[2 * q + 1][t]);
+        const int row = (4 * g + t) * 16 + n;
+        *reinterpret_cast<u32x4*>(&z_st[row * 32 + (((wave * 2 + h) ^ (row & 7)) << 2)]) = o;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    {
+      const int pc = tid & 7, rr = tid >> 3;               // 16-byte piece of a row; rows rr, rr + 32, ...
+      u32x4 v[8];
+#pragma unroll
+      for (int it = 0; it < 8; ++it) v[it] = *reinterpret_cast<const u32x4*>(&z_st[(rr + 32 * it) * 32 + ((pc ^ (rr & 7)) << 2)]);
+      const int m = m0 + 16 * mg + (rr & 15);
+      if (m < M) {
+#pragma unroll
+        for (int it = 0; it < 8; ++it)
+          *reinterpret_cast<u32x4*>(reinterpret_cast<T*>(p.Z) + ((int64_t)(2 * it + (rr >> 4)) * M + m) * R + r0 + pc * 8) = v[it];
+      }
+    }
+  }
+  TR6(14);
+}
+
+// Z (16, M, R) of dtype = mix(S, x V) for 16 input blocks of a multiple of 64 columns and a rank that is a multiple of 64.
+// scratch: room for S transposed to (r, i, j), used unless S already has that layout.  Returns BLR_OK, a negative blr_status, or
+// 1 when the shape is not for this kernel.
+int blast_ymixw_launch(const void* x, int64_t ldx, const void* V, const void* S, void* Z, int M, int in_f, int b, int R,
+                       int64_t s_si, int64_t s_sj, int64_t s_sr, int s_layout, int dtype, void* scratch, size_t scratch_bytes,
+                       hipStream_t st) {
+  if (dtype != BLR_F16 && dtype != BLR_BF16) return 1;
+  if (b != 16 || in_f % 16) return 1;
+  const int P = in_f / 16;
+  if (P % 64 || R % 64 || ldx % 8 || !aligned(x, 16) || !aligned(V, 16) || !aligned(Z, 16)) return 1;
+  if (((int64_t)(M - 1) * ldx + in_f) * 2 >= ((int64_t)1 << 31) || (int64_t)64 * R * 2 >= ((int64_t)1 << 31) || (int64_t)256 * R * 2 >= ((int64_t)1 << 31)) return 1;
+  const int nmt = (int)cdiv(M, 64), nrt = R / 64;
+  if ((int64_t)nmt * nrt >= 65536) return 1;
+  YmixwParams p = {};
+  p.x = x; p.ldx = ldx; p.V = V; p.Z = Z; p.M = M; p.R = R; p.KT = P / 64;
+  p.nrt = fd_make((uint32_t)nrt);
+  if (s_layout == BLR_S_RIJ && aligned(S, 8)) {
+    p.St = S;
+  } else if (s_sr == 1 && s_si % 8 == 0 && s_sj % 8 == 0 && aligned(S, 16)) {
+    p.St = S; p.s_stage = 1; p.s_si = s_si; p.s_sj = s_sj;
+  } else {
+    if (!scratch || scratch_bytes < (size_t)256 * R * 2 || !aligned(scratch, 8)) return 1;
+    const unsigned tg = (unsigned)cdiv((int64_t)16 * R, 256);
+    if (dtype == BLR_F16) hipLaunchKernelGGL(ym_s_transpose_kernel<f16>, dim3(tg), dim3(256), 0, st, (const f16*)S, (f16*)scratch, 16, R, s_si, s_sj, s_sr);
+    else hipLaunchKernelGGL(ym_s_transpose_kernel<bf16>, dim3(tg), dim3(256), 0, st, (const bf16*)S, (bf16*)scratch, 16, R, s_si, s_sj, s_sr);
+    BLR_CHECK_LAUNCH("ym_s_transpose");
+    p.St = scratch;
+  }
+  void* const fn = dtype == BLR_F16 ? (void*)blast_ymixw_kernel<f16> : (void*)blast_ymixw_kernel<bf16>;
+  static bool attr_set[2] = {false, false};
+  if (!attr_set[dtype == BLR_F16 ? 0 : 1]) {
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)YW_LDS);
+    if (e != hipSuccess) { set_error("blast_ymixw: cannot raise the LDS limit: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
+    attr_set[dtype == BLR_F16 ? 0 : 1] = true;
+  }
+  void* args[] = {&p};
+  hipError_t e = hipLaunchKernel(fn, dim3((unsigned)(nmt * nrt)), dim3(YW_NT), args, YW_LDS, st);
+  if (e != hipSuccess) { set_error("blast_ymixw: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
   return BLR_OK;
 }
 

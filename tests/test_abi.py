@@ -93,7 +93,7 @@ def test_run_time_options_are_named_and_range_checked():
     ok = {"BLR_GEMM_RING": (0, 1, 2), "BLR_GEMM_RING_TILE": (0, 256256, 256128, 256096, 128128), "BLR_GEMM_RING_PER_CU": (0, 1, 2),
           "BLR_GEMM_RING_WAVES": (4, 8), "BLR_GEMM_RING_BK": (32, 64), "BLR_GEMM_SPLITK": (0, 1), "BLR_DECODE2": (0, 1), "BLR_DECODE3": (0, 1),
           "BLR_DECODE_PAIR": (0, 1, 2), "BLR_DECODE_ROWS": (0, 1), "BLR_DENSE_SLAB": (0, 1), "BLR_DENSE_ROWS": (0, 1),
-          "BLR_BLAST_MIXU": (0, 1, 2), "BLR_BLAST_ONE": (0, 1)}
+          "BLR_BLAST_MIXU": (0, 1, 2), "BLR_BLAST_ONE": (0, 1), "BLR_BLAST_YMIXW": (0, 1)}
     for name, values in ok.items():
         for v in values:
             assert lib.blr_set_option(name.encode(), v, 0) == 0, (name, v)

@@ -93,7 +93,9 @@ LLAMA = {"qkvo": (256, 256, 512), "gate_up": (256, 1376, 1024), "down": (688, 25
 
 
 FUSED_SHAPES = [(16, 64, 72, 128, (96,)), (16, 72, 216, 288, (2, 75)), (4, 48, 24, 96, (37,)), (8, 256, 64, 200, (300,)),
-                (16, 688, 256, 1024, (64,)), (12, 16, 8, 40, (33,))]
+                (16, 688, 256, 1024, (64,)), (12, 16, 8, 40, (33,)),
+                # 16 input blocks of a multiple of 64 columns, above 128, rank a multiple of 64: the kernel that runs x V as one GEMM
+                (16, 256, 88, 128, (300,)), (16, 192, 256, 64, (2, 75)), (16, 256, 256, 512, (257,)), (16, 320, 24, 192, (64,))]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -111,6 +113,27 @@ def test_blast_fused_algorithm(name, shape, dtype):
     assert_close(out, ref.reshape(tuple(out.shape)), dtype, f"fused {name}")
     tiled = _run_blast(name, x, U, Vt, S, dtype, "tiled")
     assert_close(out, back(tiled), dtype, f"fused against tiled {name}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("name", ["triton_blast_full_fp16", "triton_blast_bmm_fp16"])
+@pytest.mark.parametrize("shape", [(16, 256, 256, 512, (1100,)), (16, 192, 88, 256, (8, 130))])
+def test_blast_wide_input_blocks_first_half_on_and_off(name, shape, dtype):
+    """Row counts that fill half the chip with 64 x 64 tiles take x V and the mix as one launch by default (16 input blocks of
+    a multiple of 64 columns, Y in registers); BLR_BLAST_YMIXW=0 sends the same call through the batched GEMM and the mix
+    kernel.  Both against the oracle and against each other, S in both layouts (the (j, i, r) one is staged through LDS inside
+    the kernel); row counts that end inside a tile."""
+    from triton_funcs import _lib as L
+    b, p, q, r, lead = shape
+    say(f"[case] wide input blocks {name} b={b} p={p} q={q} r={r} lead={lead} {dtype}")
+    x, U, Vt, S = blast_inputs(b, p, q, r, lead, seed=33)
+    out = _run_blast(name, x, U, Vt, S, dtype, "auto")
+    ref = _ref(x, U, Vt, S, dtype)[0]
+    assert_close(out, ref.reshape(tuple(out.shape)), dtype, f"one launch {name}")
+    with L.options(BLR_BLAST_YMIXW=0):
+        off = _run_blast(name, x, U, Vt, S, dtype, "auto")
+    assert_close(off, ref.reshape(tuple(out.shape)), dtype, f"GEMM + mix {name}")
+    assert_close(out, back(off), dtype, f"one launch against GEMM + mix {name}")
 
 
 NARROW_OUT = [(16, 288, 72, 576, (300,)), (16, 136, 40, 64, (129,)), (16, 200, 80, 96, (4, 50)), (16, 256, 8, 32, (131,)),
