@@ -417,10 +417,14 @@ __global__ __launch_bounds__(YW_NT, 1) void blast_ymixw_kernel(YmixwParams p) {
   const int chunk0 = wn * 4 + (g & 1) * 2 + ((i16 & 3) >> 1);
   const uint32_t rowB = (uint32_t)(((g >> 1) * 8 + (i16 >> 2)) * RB + (i16 & 1) * 8 + ((chunk0 ^ ((i16 >> 2) << 1)) << 4));
 
-  // Stage t lives in slot t % NST; NST - 1 stages are in flight.  The loop is bound by how many bytes a compute unit has in flight
-  // over the latency of its loads, so the ring takes all of the LDS.  (Asking for every line a first time twenty stages early, by
-  // a 4-byte load per line into a dump area, made it slower: 18.5 -> 28.9 us per tile at P = 256, R = 512 - an instruction that
-  // touches 32 lines costs the address path as much as four that fetch them.)
+  // Stage t lives in slot t % NST; NST - 1 stages are in flight.  A stage takes about 620 cycles here whatever the order of the
+  // loop: the same with every workgroup of the launch on one and the same tile (all loads L2 hits), with a ring of ten stages,
+  // with two accumulators taking the sub-steps in turn and with the fragments of stage s + 1 read under the products of stage s
+  // (the blocks of Y pinned to accumulation registers to make room) - in-kernel cycle counts then show 29 % of a wave's loop in
+  // the issue of its four loads: the compute unit's sixteen load instructions and 48 KiB of LDS traffic per stage are what a
+  // 64 x 64 tile costs, and the tile cannot grow because Y of sixteen blocks has to stay in registers.  (Asking for every line a
+  // first time twenty stages early, by a 4-byte load per line into a dump area, made it slower: 18.5 -> 28.9 us per tile at
+  // P = 256, R = 512 - an instruction that touches 32 lines costs the address path as much as four that fetch them.)
   const int s_total = 16 * p.KT;
 #pragma unroll
   for (int s = 0; s < NST - 1; ++s) issue(min(s, s_total - 1), s);
@@ -564,6 +568,9 @@ int blast_ymixw_launch(const void* x, int64_t ldx, const void* V, const void* S,
   const int P = in_f / 16;
   if (P % 64 || R % 64 || ldx % 8 || !aligned(x, 16) || !aligned(V, 16) || !aligned(Z, 16)) return 1;
   if (((int64_t)(M - 1) * ldx + in_f) * 2 >= ((int64_t)1 << 31) || (int64_t)64 * R * 2 >= ((int64_t)1 << 31) || (int64_t)256 * R * 2 >= ((int64_t)1 << 31)) return 1;
+  // (A variant with 64 rows x 128 ranks on eight waves - two per SIMD, three quarters of the operand bytes per product, the tile's
+  // two halves of 64 ranks mixed one after the other - passed the same tests and measured slower: a stage of its loop took 575 ns
+  // against 270 ns, 4096 -> 22016 at 2048 rows 177 against 173 us for the call.)
   const int nmt = (int)cdiv(M, 64), nrt = R / 64;
   if ((int64_t)nmt * nrt >= 65536) return 1;
   YmixwParams p = {};
