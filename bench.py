@@ -320,7 +320,7 @@ def main():
     g_bp = graph_of([bp[i % 4][0] for i in range(48)])
     bp_us = time_graph(g_bp, 48)
     bp_bytes, bp_flops = blast_bytes_flops(2048, i_f, r_gu, o_f)
-    roofline_blast_prefill = {"bound": "mfma", "kernel": "BLAST gate_up 4096->22016 r=1024 b=16, M=2048: gemm_ring_kernel (x V) + blast_mix_h2_kernel + gemm_ring64_kernel (Z U)",
+    roofline_blast_prefill = {"bound": "mfma", "kernel": "BLAST gate_up 4096->22016 r=1024 b=16, M=2048: blast_ymixw_kernel (x V and the mix) + gemm_ring64_kernel (Z U)",
                               "achieved": round(bp_flops / (bp_us * 1e-6) / 1e12, 1), "peak": MFMA_PEAK / 1e12, "unit": "TFLOP/s",
                               "frac": round(bp_flops / (bp_us * 1e-6) / MFMA_PEAK, 4), "us_per_call": round(bp_us, 2),
                               "algorithmic_flops": bp_flops, "algorithmic_bytes": bp_bytes,
