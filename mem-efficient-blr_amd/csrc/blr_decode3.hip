@@ -316,7 +316,14 @@ __global__ __launch_bounds__(D3_NT) void decode3_kernel(Decode3Params p) {
       }
     }
     TR3(2);
-    if (!mixer) return;
+    // The call's epoch is closed by the last chain workgroup, as soon as it has nothing left to do (every workgroup checks in
+    // before its first wait, so all of them have read the previous epoch by the time the count is complete) - at the end of a
+    // slab workgroup the round trip of that count was the last thing the launch waited for.
+    const bool closer = c == p.nchain - 1;
+    if (!mixer) {
+      if (closer) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, p.spin_limit);
+      return;
+    }
 
     // ---- mix: z[i][m][r] = sum_j S(i, j, r) * sum_ks y[ks][j][m][r] for RCH values of r, every i ------------------
     // Thread (g, rr): first g is the input block j whose y it fetches, then the output block i it emits.
@@ -395,6 +402,7 @@ __global__ __launch_bounds__(D3_NT) void decode3_kernel(Decode3Params p) {
       }
     }
     TR3(9);
+    if (closer) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, p.spin_limit);
     return;
   }
 
@@ -562,7 +570,6 @@ __global__ __launch_bounds__(D3_NT) void decode3_kernel(Decode3Params p) {
     }
   }
   TR3(7);
-  if (w == 0) finish_epoch(p.arrive_word, p.epoch_word, p.err_word, epoch, G, p.spin_limit);
 }
 
 // ---- host side --------------------------------------------------------------------------------------------------
