@@ -79,27 +79,33 @@ struct Decode3Params {
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Totals over the row groups of a workgroup.  Every thread holds EPL columns of one row group; red is laid out
-// [m][row group][column].  Thread (column = tid >> sub, lane of SUB = 512 / columns) adds EPL row groups, then the SUB
-// lanes of a column add up: every lane of a column ends up with its total.
+// [m][row group][column], a row of nc columns padded to nc + nc / 8 floats so that the lanes of a column, which read
+// different row groups, meet different banks.  Thread (column = tid >> sub, lane of SUB = 512 / columns) adds EPL row
+// groups, then the SUB lanes of a column - neighbours inside a row of 16 lanes - add up by DPP: every lane of a column
+// ends up with its total.  red holds MT * 512 * EPL * 9 / 8 floats.
 template <int MT, int EPL>
 __device__ __forceinline__ void wg_reduce_lds(float (&acc)[MT][EPL], int lpr_log2, float* red, float (&tot)[MT]) {
   const int tid = threadIdx.x;
   const int cv = tid & ((1 << lpr_log2) - 1), rs = tid >> lpr_log2;
   const int nc_log2 = lpr_log2 + ilog2c(EPL), nrs_log2 = 9 - lpr_log2, sub_log2 = 9 - nc_log2;
+  const int ld = (1 << nc_log2) + (1 << (nc_log2 - 3));
   lds_barrier();                                   // earlier readers of red are done
 #pragma unroll
   for (int m = 0; m < MT; ++m)
 #pragma unroll
     for (int e = 0; e < EPL; e += 4)
-      *reinterpret_cast<f32x4*>(&red[((((m << nrs_log2) + rs) << nc_log2)) + cv * EPL + e]) = f32x4{acc[m][e], acc[m][e + 1], acc[m][e + 2], acc[m][e + 3]};
+      *reinterpret_cast<f32x4*>(&red[((m << nrs_log2) + rs) * ld + cv * EPL + e]) = f32x4{acc[m][e], acc[m][e + 1], acc[m][e + 2], acc[m][e + 3]};
   lds_barrier();
   const int col = tid >> sub_log2, sub = tid & ((1 << sub_log2) - 1);
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
     float v = 0.0f;
 #pragma unroll
-    for (int t = 0; t < EPL; ++t) v += red[((((m << nrs_log2) + sub + (t << sub_log2)) << nc_log2)) + col];
-    for (int o = 1; o < (1 << sub_log2); o <<= 1) v += __shfl_xor(v, o, 64);
+    for (int t = 0; t < EPL; ++t) v += red[((m << nrs_log2) + sub + (t << sub_log2)) * ld + col];
+    if (sub_log2 >= 1) v = dpp_add<0xB1>(v);         // lanes 1 0 3 2
+    if (sub_log2 >= 2) v = dpp_add<0x4E>(v);         // lanes 2 3 0 1
+    if (sub_log2 >= 3) v = dpp_add<0x141>(v);        // the other quad of eight lanes (row_half_mirror)
+    if (sub_log2 >= 4) v = dpp_add<0x140>(v);        // the other half of sixteen lanes (row_mirror)
     tot[m] = v;
   }
 }
@@ -126,7 +132,7 @@ __global__ __launch_bounds__(D3_NT) void decode3_kernel(Decode3Params p) {
   constexpr int ZR = MT <= 2 ? 2 : 1;                // 16-byte fetches of tagged z per lane and token row (two ranks each)
   constexpr int D3_PF = d3_pf(WB), D3_PFA = D3_PF - D3_PFB;
   __shared__ __attribute__((aligned(16))) float a_s[D3_AS];
-  __shared__ __attribute__((aligned(16))) float red[MT * D3_NT * EPL];
+  __shared__ __attribute__((aligned(16))) float red[MT * D3_NT * EPL * 9 / 8];
   __shared__ __attribute__((aligned(16))) T s_s[16 * D3_NT];   // a mix item's block of S as (i, j, r)
   const int tid = threadIdx.x;
   const int w = blockIdx.x, G = gridDim.x;

@@ -73,6 +73,12 @@ __device__ __forceinline__ void finish_epoch(unsigned* arrive_word, unsigned* ep
   }
 }
 
+// v + the value of v in another lane of the same row of 16 lanes (DPP control word CTRL)
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
 // Workgroup w of a launch runs on XCD w % 8, and each XCD has its own L2.  Item order that gives every XCD a contiguous
 // run of the G items: neighbouring items (column chunks of one factor block, whose row pieces share cache lines when they
 // are not whole lines) then meet in one L2 instead of fetching the shared lines twice.

@@ -71,33 +71,33 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t rbuf2(const void* p, uint32_t 
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
-// v + the value of v in another lane of the same row of 16 lanes (DPP control word CTRL)
-template <int CTRL>
-__device__ __forceinline__ float dpp_add(float v) {
-  return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
-}
-
-// Totals over the row groups of a workgroup (see decode3_kernel): red is [m][row group][column]; every lane of a column
-// ends up with its total.
+// Totals over the row groups of a workgroup (see decode3_kernel): red is [m][row group][column], a row of nc columns padded
+// to nc + nc / 8 floats so that the lanes of a column, which read different row groups, meet different banks; every lane of
+// a column ends up with its total (the lanes of a column are neighbours inside a row of 16 lanes: DPP adds, no LDS trips).
+// red holds MT * 512 * EPL * 9 / 8 floats.
 template <int MT, int EPL>
 __device__ __forceinline__ void pair_reduce(float (&acc)[MT][EPL], int lpr_log2, float* red, float (&tot)[MT]) {
   const int tid = threadIdx.x;
   const int cv = tid & ((1 << lpr_log2) - 1), rs = tid >> lpr_log2;
   const int nc_log2 = lpr_log2 + ilog2k(EPL), nrs_log2 = 9 - lpr_log2, sub_log2 = 9 - nc_log2;
+  const int ld = (1 << nc_log2) + (1 << (nc_log2 - 3));
   lds_barrier2();                                    // earlier readers of red are done
 #pragma unroll
   for (int m = 0; m < MT; ++m)
 #pragma unroll
     for (int e = 0; e < EPL; e += 4)
-      *reinterpret_cast<f32x4*>(&red[((((m << nrs_log2) + rs) << nc_log2)) + cv * EPL + e]) = f32x4{acc[m][e], acc[m][e + 1], acc[m][e + 2], acc[m][e + 3]};
+      *reinterpret_cast<f32x4*>(&red[((m << nrs_log2) + rs) * ld + cv * EPL + e]) = f32x4{acc[m][e], acc[m][e + 1], acc[m][e + 2], acc[m][e + 3]};
   lds_barrier2();
   const int col = tid >> sub_log2, sub = tid & ((1 << sub_log2) - 1);
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
     float v = 0.0f;
 #pragma unroll
-    for (int t = 0; t < EPL; ++t) v += red[((((m << nrs_log2) + sub + (t << sub_log2)) << nc_log2)) + col];
-    for (int o = 1; o < (1 << sub_log2); o <<= 1) v += __shfl_xor(v, o, 64);
+    for (int t = 0; t < EPL; ++t) v += red[((m << nrs_log2) + sub + (t << sub_log2)) * ld + col];
+    if (sub_log2 >= 1) v = dpp_add<0xB1>(v);           // lanes 1 0 3 2
+    if (sub_log2 >= 2) v = dpp_add<0x4E>(v);           // lanes 2 3 0 1
+    if (sub_log2 >= 3) v = dpp_add<0x141>(v);          // the other quad of eight lanes (row_half_mirror)
+    if (sub_log2 >= 4) v = dpp_add<0x140>(v);          // the other half of sixteen lanes (row_mirror)
     tot[m] = v;
   }
 }
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(DP_NT) void pair_stage1_kernel(PairParams p) {
   constexpr int TR4_BASE = 0; (void)TR4_BASE;
   constexpr int EPL = 128 / WB;
   __shared__ __attribute__((aligned(16))) float a_s[4096];
-  __shared__ __attribute__((aligned(16))) float red[MT * DP_NT * EPL];
+  __shared__ __attribute__((aligned(16))) float red[MT * DP_NT * EPL * 9 / 8];
   const int tid = threadIdx.x;
   TR4(0);
   if (blockIdx.x >= (uint32_t)p.items1) {
@@ -297,7 +297,7 @@ __global__ __launch_bounds__(DP_NT) void pair_slab_kernel(PairParams p) {
   constexpr int KSM = dp_ks_max(MT);                 // k-slices of stage 1 this instantiation can add up
   using V8 = typename TypeTraits<T>::vec8;
   __shared__ __attribute__((aligned(16))) float a_s[DP_AS];
-  __shared__ __attribute__((aligned(16))) float red[MT * DP_NT * EPL];
+  __shared__ __attribute__((aligned(16))) float red[MT * DP_NT * EPL * 9 / 8];
   const int tid = threadIdx.x;
   TR4(0);
   const int M = p.M, R = p.R;
