@@ -833,10 +833,10 @@ __global__ __launch_bounds__(NWV * 64, (NWV / 4) * PER_CU) void gemm_ring64_kern
     tail_kn[i] = B_KN ? (uint32_t)((krow - min(krow, rmax)) * g.ldb * 2) : tail_kc;
   }
   const uint32_t lds0 = ring_lds_addr(smem + wave * 1024);
-  // HALF (eight waves, two stages, every tile inside the matrices, no partial stage: the launcher checks): a stage's loads cannot
+  // HALF (eight waves, two stages, no clamped row of either K-contiguous operand, no partial stage: the launcher checks): a stage's loads cannot
   // be spread over the step here, and every wave that issues one waits in the compute unit's address path while its SIMD's other
   // wave may be waiting there too.  Waves 0..3 - one per SIMD - therefore issue the loads of waves 4..7 as well: those rows lie
-  // NWV / 2 load instructions further down, a wave-uniform offset, so the same per-lane offsets serve (nothing is clamped).
+  // NWV / 2 load instructions further down, a wave-uniform offset, so the same per-lane offsets serve (no row is clamped; the column clamp of a (k, n) operand belongs to the lane and is the same for both).
   static_assert(!HALF || (NWV == 8 && NST == 2), "the one configuration this is for");
   constexpr int ISS = HALF ? 2 : 1;
   const bool issuer = !HALF || wave < NWV / 2;
@@ -1237,8 +1237,9 @@ static int launch_ring64(const GemmArgs& g, hipStream_t st) {
   void* fn = ep ? (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, true, NWV, NST, PER_CU> : (void*)gemm_ring64_kernel<T, false, BM, BN, true, NWV, NST, PER_CU>)
                 : (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, false, NWV, NST, PER_CU> : (void*)gemm_ring64_kernel<T, false, BM, BN, false, NWV, NST, PER_CU>);
   if constexpr (NWV == 8 && NST == 2) {
-    // no tile with a clamped row or column and no partial stage: four of the eight waves issue all loads (see the kernel)
-    if (g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0)
+    // no tile with a clamped row and no partial stage: four of the eight waves issue all loads (see the kernel).  A ragged last
+    // column tile is fine with a (k, n) operand: its clamp is on the lane's column, the same in both halves of a stage's rows
+    if (g.M % BM == 0 && (g.N % BN == 0 || (g.b_kn && g.N % 8 == 0)) && g.K % 64 == 0)
       fn = ep ? (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, true, NWV, NST, PER_CU, true> : (void*)gemm_ring64_kernel<T, false, BM, BN, true, NWV, NST, PER_CU, true>)
               : (g.b_kn ? (void*)gemm_ring64_kernel<T, true, BM, BN, false, NWV, NST, PER_CU, true> : (void*)gemm_ring64_kernel<T, false, BM, BN, false, NWV, NST, PER_CU, true>);
   }
