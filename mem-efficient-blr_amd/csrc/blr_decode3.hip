@@ -12,9 +12,9 @@
 //     500 instructions are a microsecond;
 //   * a workgroup of 512 threads is a whole compute unit: placement is not left to the dispatcher, a slab of U
 //     spans the full rank (8 waves x 32 loads x 16 bytes = 256 KiB of registers), and stage 2 needs no k split.
-// So every workgroup first asks for its stage-1 items (pieces of V: what heads the chain is requested first,
-// everywhere), "slab" workgroups ask for their whole slab of U right behind, without pacing, and "chain"
-// workgroups (no slab, so nothing queued in front of their polls) run the mix.  A slab workgroup places a
+// So a workgroup has one role.  "Chain" workgroups ask for their stage-1 items (pieces of V: what heads the chain is
+// requested first) and, with no slab queued in front of their polls, the first of them run the mix; "slab" workgroups
+// ask for their whole slab of U at once, without pacing.  A slab workgroup places a
 // speculative fetch of its slice of z in front of its last eight loads: if the chain has delivered by the time
 // three quarters of the slab have landed, the products run under the rest of the stream.  Index arithmetic uses
 // shifts and multiply-high by launch constants, reductions go through LDS once.
@@ -58,7 +58,7 @@ struct Decode3Params {
   int zrep;                                      // bo == 1: z is published in zrep copies so that the slabs do not all poll one address range
   int M, b, bo, P, R, Q;                         // b blocks of the input (stage 1), bo blocks of the output (stage 2)
   int64_t s_si, s_sj, s_sr;
-  int lpr1_log2, ks1, kc1, nb1, kpad1_log2, items1, n1s, nchain;
+  int lpr1_log2, ks1, kc1, nb1, kpad1_log2, items1, nchain;
   FastDiv nch1, bdiv;
   int lpr2_log2, ks2, kc2, items2, pfn, kpad2, kld2_log2, zspec;
   FastDiv nch2, bodiv;
@@ -654,8 +654,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   if (min_chain >= resident) return d2_bail(__LINE__);
 
   // ---- stage 1 for a given number of slab and chain workgroups; false when it does not fit ----------------------
-  struct S1 { int lpr, nch, ks, kc, nb, kpad, items, n1s, nchain; double t_chain, extra_slab; };
-  const double vbytes = (double)b * P * R * WBITS / 8.0;
+  struct S1 { int lpr, nch, ks, kc, nb, kpad, items, nchain; double t_chain; };
   auto plan1 = [&](int nslab, double slab_bytes, S1& s) -> bool {
     const int navail = resident - nslab;
     int lpr = 16;
@@ -689,7 +688,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
         const double est = t_chain + 2.2 > t_slab ? t_chain + 2.2 : t_slab;     // chain: + two hand-overs and the mix
         if (est < best) {
           best = est; have = true;
-          s = {lpr, nch, ks, kc, nb, kpad, items, 0, nchain, t_chain, 0.0};
+          s = {lpr, nch, ks, kc, nb, kpad, items, nchain, t_chain};
         }
       }
     }
@@ -715,7 +714,6 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
         if (ks != ks0) continue;
         const int pfn = kc / rpp;
         if (pfn > d3_pf(WBITS)) continue;                // the whole slab stays in registers
-        const int left = 0;
         const int kpad2 = pfn * rpp;
         if (MT * kpad2 > D3_AS || (kc >> 1) > (MT <= 2 ? 2 : 1) * D3_NT) continue;
         const int nslab = bo * nch * ks;
@@ -723,7 +721,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
         const double slab_bytes = (double)kc * lpr * 16.0;
         S1 t = {};
         if (!plan1(nslab, slab_bytes, t)) continue;
-        const double t_slab = d3_stream_us(slab_bytes + t.extra_slab) + (left > 0 ? 1.0 : 0.0);
+        const double t_slab = d3_stream_us(slab_bytes);
         const double t_z = t.t_chain + 2.2;
         const double est = (t_slab > t_z ? t_slab : t_z) + 0.8 + (ks > 1 ? 0.8 : 0.0) + (lpr < 16 ? (lpr < 8 ? 0.4 : 0.15) : 0.0);
         if (est < best) {
@@ -736,7 +734,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   }
   p.bodiv = fd_make((uint32_t)bo);
   p.lpr1_log2 = ilog2(s1.lpr); p.nch1 = fd_make((uint32_t)s1.nch); p.bdiv = fd_make((uint32_t)b);
-  p.ks1 = s1.ks; p.kc1 = s1.kc; p.nb1 = s1.nb; p.kpad1_log2 = ilog2(s1.kpad); p.items1 = s1.items; p.n1s = s1.n1s; p.nchain = s1.nchain;
+  p.ks1 = s1.ks; p.kc1 = s1.kc; p.nb1 = s1.nb; p.kpad1_log2 = ilog2(s1.kpad); p.items1 = s1.items; p.nchain = s1.nchain;
   if ((1 << p.kpad1_log2) != s1.kpad) return d2_bail(__LINE__);
   {
     int kld = 1;
@@ -748,7 +746,7 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
     // the speculative fetch of z pays when the chain is expected to deliver before the last eight loads of a slab land
     const double t_z = s1.t_chain + 2.2;
     const double slab_bytes = (double)p.kc2 * (1 << p.lpr2_log2) * 16.0;
-    const double t_a = d3_stream_us((slab_bytes + s1.extra_slab) * (p.pfn > D3_PFB ? (double)(p.pfn - D3_PFB) / p.pfn : 0.0));
+    const double t_a = d3_stream_us(slab_bytes * (p.pfn > D3_PFB ? (double)(p.pfn - D3_PFB) / p.pfn : 0.0));
     p.zspec = (p.pfn > D3_PFB && t_z + 0.5 < t_a) ? 1 : 0;
   }
 
@@ -762,8 +760,8 @@ int decode3_blast_launch(const StreamBlastArgs& a, void* region, unsigned* epoch
   const int grid = p.items2 + p.nchain;
   if (grid > resident) return d2_bail(__LINE__);
   static const int dbg = env_i("BLR_D2_DEBUG", 0);
-  if (dbg) fprintf(stderr, "decode3: M=%d b=%d bo=%d P=%d R=%d Q=%d wb=%d | slabs %d (lpr %d, nch %u, ks %d, kc %d, pfn %d, zspec %d) chain %d (items %d: %d on slabs, ks %d, kc %d, nb %d) mix %d\n",
-                   M, b, bo, P, R, Q, WBITS, p.items2, 1 << p.lpr2_log2, p.nch2.d, p.ks2, p.kc2, p.pfn, p.zspec, p.nchain, p.items1, p.n1s, p.ks1, p.kc1, p.nb1, p.itemsM);
+  if (dbg) fprintf(stderr, "decode3: M=%d b=%d bo=%d P=%d R=%d Q=%d wb=%d | slabs %d (lpr %d, nch %u, ks %d, kc %d, pfn %d, zspec %d) chain %d (items %d, ks %d, kc %d, nb %d) mix %d\n",
+                   M, b, bo, P, R, Q, WBITS, p.items2, 1 << p.lpr2_log2, p.nch2.d, p.ks2, p.kc2, p.pfn, p.zspec, p.nchain, p.items1, p.ks1, p.kc1, p.nb1, p.itemsM);
   void* args[] = {&p};
   hipError_t e = hipLaunchKernel(fn, dim3(grid), dim3(D3_NT), args, 0, st);
   if (e != hipSuccess) { set_error("decode3: launch failed: %s", hipGetErrorString(e)); return BLR_ERR_LAUNCH; }
