@@ -19,6 +19,7 @@
 // the mix is too much work to be redone by every slab of an output block (as the two-launch path for up to four rows
 // does).  The number of column pieces per chunk is planned so that the chunks spread evenly over the compute units
 // (a compute unit draws about 35 GB/s, so the bytes of the busiest one bound the launch).
+#include <type_traits>
 #include "blr_common.h"
 #include "blr_decode.h"
 #include "blr_decode_dev.h"
@@ -377,22 +378,26 @@ __device__ __forceinline__ void rows_prefetch(const RowsPrefetch& f, uint32_t fi
 }
 
 // ---- the mix between the two products: z[i][m][r] = sum_j S(i, j, r) y[j][m][r], rank contiguous in S ------------------------
-// One thread per four ranks of one (i, m): 2 b eight-byte loads, all in flight at once, neighbouring threads on neighbouring
-// ranks.  Y is re-read b times and S M times - from L2, both are a few hundred KiB.  fp32 sums in input-block order.
-template <typename T, int B>
+// One thread per VW (four or eight) ranks of one (i, m): 2 b loads of 2 VW bytes, all in flight at once, neighbouring threads on
+// neighbouring ranks.  Y is re-read b times and S M times - from L2, both are a few hundred KiB.  fp32 sums in input-block order.
+// (A load instruction costs a compute unit's address path the same whether a lane takes 8 or 16 bytes: eight ranks per thread in
+// workgroups of 128 threads halve the instructions of every compute unit - the launcher takes them when there is enough work.)
+template <typename T, int B, int VW>
 __global__ __launch_bounds__(256) void rows_mix_kernel(const T* __restrict__ Y, const T* __restrict__ S, T* __restrict__ Z,
                                                         int M, int b, int R, int64_t s_si, int64_t s_sj, FastDiv r4div, FastDiv bdiv, uint32_t total,
                                                         RowsPrefetch pf, uint32_t nmix) {
   if (blockIdx.x >= nmix) { rows_prefetch(pf, nmix); return; }
-  const uint32_t item = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t item = blockIdx.x * blockDim.x + threadIdx.x;
   if (item >= total) return;
-  const uint32_t t = fd_div(item, r4div), r4 = item - t * r4div.d;
+  const uint32_t t = fd_div(item, r4div), r4 = item - t * r4div.d;         // (r4: the thread's piece of VW ranks)
   const uint32_t m = fd_div(t, bdiv), i = t - m * bdiv.d;
-  const T* sp = S + (int64_t)i * s_si + r4 * 4;
-  const T* yp = Y + (int64_t)m * R + r4 * 4;
+  const T* sp = S + (int64_t)i * s_si + r4 * VW;
+  const T* yp = Y + (int64_t)m * R + r4 * VW;
   const int64_t y_sj = (int64_t)M * R;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  using V4 = typename TypeTraits<T>::vec4;
+  float acc[VW];
+#pragma unroll
+  for (int e = 0; e < VW; ++e) acc[e] = 0.f;
+  using V4 = typename std::conditional<VW == 8, typename TypeTraits<T>::vec8, typename TypeTraits<T>::vec4>::type;
   if constexpr (B > 0) {
     V4 sv[B], yv[B];
 #pragma unroll
@@ -400,18 +405,18 @@ __global__ __launch_bounds__(256) void rows_mix_kernel(const T* __restrict__ Y, 
 #pragma unroll
     for (int j = 0; j < B; ++j)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] += TypeTraits<T>::to_f32(sv[j][e]) * TypeTraits<T>::to_f32(yv[j][e]);
+      for (int e = 0; e < VW; ++e) acc[e] += TypeTraits<T>::to_f32(sv[j][e]) * TypeTraits<T>::to_f32(yv[j][e]);
   } else {
     for (int j = 0; j < b; ++j) {
       const V4 sv = *reinterpret_cast<const V4*>(sp + j * s_sj), yv = *reinterpret_cast<const V4*>(yp + j * y_sj);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] += TypeTraits<T>::to_f32(sv[e]) * TypeTraits<T>::to_f32(yv[e]);
+      for (int e = 0; e < VW; ++e) acc[e] += TypeTraits<T>::to_f32(sv[e]) * TypeTraits<T>::to_f32(yv[e]);
     }
   }
   V4 o;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) o[e] = TypeTraits<T>::from_f32(acc[e]);
-  *reinterpret_cast<V4*>(Z + ((int64_t)i * M + m) * R + r4 * 4) = o;
+  for (int e = 0; e < VW; ++e) o[e] = TypeTraits<T>::from_f32(acc[e]);
+  *reinterpret_cast<V4*>(Z + ((int64_t)i * M + m) * R + r4 * VW) = o;
 }
 
 // Low rank seen as BLAST with one output block and S = 1: z[m][r] = sum_j y[j][m][r] (the k-slices of x A).  The slices are
@@ -518,12 +523,19 @@ int rows_mix_rij_t(const void* Y, const void* S, void* Z, int M, int R, const Ro
 
 template <typename T>
 int rows_mix_t(const void* Y, const void* S, void* Z, int M, int b, int R, int64_t s_si, int64_t s_sj, const RowsPrefetch& pf, hipStream_t st) {
-  const uint32_t total = (uint32_t)((int64_t)M * b * (R / 4));
-  const uint32_t nmix = (uint32_t)cdiv(total, 256);
-  const dim3 grid(nmix + prefetch_blocks(pf)), block(256);
-  const FastDiv r4div = fd_make((uint32_t)(R / 4)), bdiv = fd_make((uint32_t)b);
-  if (b == 16) hipLaunchKernelGGL((rows_mix_kernel<T, 16>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total, pf, nmix);
-  else hipLaunchKernelGGL((rows_mix_kernel<T, 0>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total, pf, nmix);
+  // eight ranks per thread once four would make more than two workgroups of 256 threads per compute unit (side by side at 64 rows:
+  // 4096 -> 4096 20.4 -> 19.95 us, 4096 -> 22016 31.7 -> 30.5, 11008 -> 4096 30.1 -> 28.9; at 4 and 16 rows, where four ranks per
+  // thread just fill the chip, the wider threads are 0.1 - 0.3 us slower)
+  const bool wide = b == 16 && R % 8 == 0 && s_si % 8 == 0 && s_sj % 8 == 0 && aligned(Y, 16) && aligned(S, 16) && aligned(Z, 16) &&
+                    (int64_t)M * b * (R / 4) >= 131072;
+  const int vw = wide ? 8 : 4, nt = wide ? 128 : 256;
+  const uint32_t total = (uint32_t)((int64_t)M * b * (R / vw));
+  const uint32_t nmix = (uint32_t)cdiv(total, nt);
+  const dim3 grid(nmix + prefetch_blocks(pf)), block(nt);
+  const FastDiv r4div = fd_make((uint32_t)(R / vw)), bdiv = fd_make((uint32_t)b);
+  if (wide) hipLaunchKernelGGL((rows_mix_kernel<T, 16, 8>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total, pf, nmix);
+  else if (b == 16) hipLaunchKernelGGL((rows_mix_kernel<T, 16, 4>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total, pf, nmix);
+  else hipLaunchKernelGGL((rows_mix_kernel<T, 0, 4>), grid, block, 0, st, (const T*)Y, (const T*)S, (T*)Z, M, b, R, s_si, s_sj, r4div, bdiv, total, pf, nmix);
   BLR_CHECK_LAUNCH("rows_mix");
   return BLR_OK;
 }
