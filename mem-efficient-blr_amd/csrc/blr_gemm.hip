@@ -1311,7 +1311,7 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
     const int64_t fill = ((int64_t)cus * 9 + 9) / 10;
     const int64_t r128 = cdiv(g.M, 128) * cdiv(g.N, 128) * g.batch;
     int per_cu = option_value(OPT_GEMM_RING_PER_CU, 0);
-    bool wide64 = false;                       // a 256 x 256 tile chosen together with stages of 64 k
+    bool wide64 = false;                       // a tile chosen together with stages of 64 k
     // interleaved columns are bound by their two-byte stores: only worth it with several tiles per compute unit
     if (rt == 0 && g.cn != 1 && ring < 2 && t128 < 2 * (int64_t)cus) rt = -1;
     if (rt == 0) {
@@ -1328,6 +1328,10 @@ static int pick_mfma(const GemmArgs& g, hipStream_t st) {
       // 1024 columns, K = 688 (x V of 11008 -> 4096) 75.1 -> 66.8 us
       else if (g.cn == 1 && g.K >= 512 && g.K <= 2048 && g.N >= 1024 && cdiv(g.N, 256) * 256 * 8 <= (int64_t)g.N * 9 && t256 >= 2 * (int64_t)cus) { rt = 256256; wide64 = true; }
       else if (g.K <= 2048 && t128 >= 2 * (int64_t)cus) { rt = 256128; if (!per_cu) per_cu = 2; }
+      // batched products from eight stages of 64 k that are exactly one round of 256 x 128 tiles: one such tile per compute unit on
+      // 64-k stages rather than two workgroups of 128 x 128 (Z U of BLAST 4096 -> 4096 at 2048 rows, 16 x 2048 x 256 x 512: the call
+      // 55.1 -> 52.8 us; 54.2 with 64-k stages on the 128 x 128 tiles)
+      else if (g.batch > 1 && g.cn == 1 && g.K >= 512 && g.K < 1024 && t128 >= fill && t128 <= (int64_t)cus) { rt = 256128; wide64 = true; }
       else if (g.K <= 512 && r128 >= fill) rt = 128128;
       // a narrow output (one 128-column tile, mostly empty at 256): more, smaller tiles (4096 x 72 x 576 in 16 batches:
       // 26.8 us with 256 x 256 tiles, 20.7 with 256 x 128, 19.7 with 128 x 128)
