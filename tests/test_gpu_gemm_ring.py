@@ -106,13 +106,14 @@ def test_seeded_random_shapes_through_every_variant(ring_forced):
 def test_whole_tiles_of_the_eight_wave_kernels(dtype, tile):
     """Problems made of whole 256 x 256 tiles and whole 64-k stages take a variant of the eight-wave, two-stage kernel in which
     four waves issue every load (the others' rows at a wave-uniform offset): plain, with bias + SiLU-gated pairs of tiles, and
-    with a K-contiguous second operand (U of the bmm layout), each against the oracle; one more k stage, one more row and one
-    more column group leave that variant again and must give the same kind of answer.  The 256 x 128 kernel (three stages, every
-    wave issuing its own loads) runs the same problems."""
+    with a K-contiguous second operand (U of the bmm layout), each against the oracle; one more k stage and one more row leave
+    that variant again and must give the same kind of answer, while a ragged last column tile of a (k, n) operand (eight or 96
+    columns of its 256 inside the matrix) stays in it - its column clamp belongs to the lane and is the same for both halves of a
+    stage's rows.  The 256 x 128 kernel (three stages, every wave issuing its own loads) runs the same problems."""
     from triton_funcs import _lib as L, blast_kernels as KB, dense_kernels as KD
     rng = np.random.default_rng(11)
     with L.options(BLR_GEMM_RING=2, BLR_GEMM_RING_TILE=tile, BLR_GEMM_RING_PER_CU="1", BLR_GEMM_RING_WAVES="8", BLR_GEMM_RING_BK="64"):
-        for M, in_f, out_f in [(512, 1088, 768), (256, 64, 256), (512, 1096, 768), (513, 1088, 768), (512, 1088, 776)]:
+        for M, in_f, out_f in [(512, 1088, 768), (256, 64, 256), (512, 1096, 768), (513, 1088, 768), (512, 1088, 776), (512, 1088, 608)]:
             x = rng.standard_normal((M, in_f)); w = rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)
             say(f"[case] whole tiles {tile} dense M={M} in={in_f} out={out_f} {dtype}")
             out = KD.triton_dense_fp16(dev(x, dtype), dev(w, dtype), TILED)
