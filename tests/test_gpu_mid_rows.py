@@ -152,3 +152,28 @@ def test_slices_whose_partial_sums_leave_the_fp16_range():
         z = rounded(rounded(x[:rows], dtype) @ rounded(a, dtype), dtype)
         ref = z @ rounded(bm, dtype)
         assert np.isfinite(got).all() and np.abs(got - ref).max() <= ulp(ref, dtype).max()
+
+
+def test_blast_seeded_random_shapes_from_one_to_300_rows():
+    """Sixty seeded random BLAST problems (2 to 16 blocks, block widths and ranks from 8 to 1488 - multiples of 8 and not powers
+    of two among them -, 1 to 300 rows, both layouts, both 16-bit types) through whatever kernels the default choice gives them:
+    the single-row kernels and their padded LDS reductions, the three launches with narrow and wide mix threads, the GEMM path
+    above 128 rows.  Each against the oracle on the same rounded inputs, to the bound of the other parity tests."""
+    from test_gpu_blast import _ref, _run_blast
+    rng = np.random.default_rng(77)
+    done = 0
+    while done < 60:
+        b = int(rng.choice([2, 4, 8, 16, 16, 16]))
+        p = int(rng.choice([8, 16, 40, 64, 72, 128, 256, 344, 688]))
+        q = int(rng.choice([8, 24, 64, 72, 128, 256, 288, 1376]))
+        r = int(rng.choice([8, 16, 64, 128, 136, 256, 512, 1024, 1488]))
+        M = int(rng.choice([1, 1, 1, 2, 3, 4, 7, 16, 17, 33, 64, 100, 128, 129, 300]))
+        if b * p * r > 8e6 or b * q * r > 12e6:
+            continue
+        dtype = [torch.float16, torch.bfloat16][done % 2]
+        name = ["triton_blast_full_fp16", "triton_blast_bmm_fp16"][(done // 2) % 2]
+        x, U, Vt, S = blast_inputs(b, p, q, r, (M,), seed=500 + done)
+        say(f"[case {done}] {name} b={b} p={p} q={q} r={r} M={M} {dtype}")
+        out = _run_blast(name, x, U, Vt, S, dtype, "auto")
+        assert_close(out, _ref(x, U, Vt, S, dtype)[0], dtype, f"{name} b={b} p={p} q={q} r={r} M={M}")
+        done += 1
