@@ -570,7 +570,10 @@ int blast_ymixw_launch(const void* x, int64_t ldx, const void* V, const void* S,
   if (((int64_t)(M - 1) * ldx + in_f) * 2 >= ((int64_t)1 << 31) || (int64_t)64 * R * 2 >= ((int64_t)1 << 31) || (int64_t)256 * R * 2 >= ((int64_t)1 << 31)) return 1;
   // (A variant with 64 rows x 128 ranks on eight waves - two per SIMD, three quarters of the operand bytes per product, the tile's
   // two halves of 64 ranks mixed one after the other - passed the same tests and measured slower: a stage of its loop took 575 ns
-  // against 270 ns, 4096 -> 22016 at 2048 rows 177 against 173 us for the call.)
+  // against 270 ns, 4096 -> 22016 at 2048 rows 177 against 173 us for the call.  The same tile on four waves - a wave holding 32 rows
+  // x 64 ranks, its 256 dwords of Y spilling over into the accumulation registers, a ring of four stages of 24 KiB, the mix a quarter
+  // of the tile at a time - was no better: 39.2 us in the loop for twice the products of the 17.3 us here, 30 us in the mix against
+  // 2 x 6.8, the call 177.5 against 171.7 us.  Fewer load instructions per product do not speed this loop up.)
   const int nmt = (int)cdiv(M, 64), nrt = R / 64;
   if ((int64_t)nmt * nrt >= 65536) return 1;
   YmixwParams p = {};
